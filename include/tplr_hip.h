@@ -1,0 +1,154 @@
+/*
+ * tplr_hip.h - C ABI of libtplr_hip.so, the gfx950 implementation of templar's
+ * gradient codec (reference: src/tplr/compress.py, tplr 2.1.28).
+ *
+ * Conventions
+ *   - every pointer named d_* is DEVICE memory owned by the caller; the library
+ *     allocates nothing and keeps no state between calls;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); all
+ *     work is enqueued on it and the call returns without synchronising;
+ *   - return value: 0 = ok, negative = TPLR_E_* (bad argument, nothing launched),
+ *     positive = a hipError_t from the launch;
+ *   - "chunk" = one 64x64 fp32 tile of a 2-D tensor, stored row-major inside the
+ *     chunked layout (Y, X, 64, 64); flat index inside a chunk = row*64 + col
+ *     (reference: rearrange "y x h w -> y x (h w)", src/tplr/compress.py:402-403);
+ *   - top-k output order is canonical: descending |value|, lowest flat index first
+ *     on exact ties, every NaN ranking above +inf.  This is the order
+ *     torch.topk(sorted=False) produces on the CPU for k*64 <= n when magnitudes
+ *     are distinct (reference call: src/tplr/compress.py:409-411).
+ */
+#ifndef TPLR_HIP_H
+#define TPLR_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TPLR_E_BADARG   (-1) /* null pointer, negative size, unsupported k            */
+#define TPLR_E_ODD      (-2) /* number of 12-bit indices is odd                        */
+#define TPLR_E_SHAPE    (-3) /* dimension not a multiple of the chunk size             */
+#define TPLR_E_TOOMANY  (-4) /* more peers / larger row than the kernel supports       */
+
+#define TPLR_CHUNK        64   /* chunk edge handled by the factorised transform       */
+#define TPLR_MAX_PEERS    128  /* peers per tplr_decode_aggregate call                 */
+#define TPLR_MAX_ROW      4096 /* longest row the select / scatter kernels accept      */
+
+/* reduce_mode of tplr_decode_aggregate / tplr_scatter_rows */
+#define TPLR_REDUCE_MEAN  0    /* mean over the peers that sent the coefficient (reference) */
+#define TPLR_REDUCE_SUM   1    /* plain sum                                             */
+
+/* Library / ABI version (major*10000 + minor*100 + patch). */
+int tplr_version(void);
+
+/* Text for a status code returned by any function below (static storage). */
+const char* tplr_status_string(int status);
+
+/* ---- 12-bit index packing ------------------------------------------------------
+ * Replaces pack_12bit_indices (src/tplr/compress.py:51-99): pairs (i0,i1) become
+ * b0 = i0 & 0xFF, b1 = (i0>>8 & 0xF) | (i1 & 0xF)<<4, b2 = i1>>4 & 0xFF.
+ * n must be even (TPLR_E_ODD).  d_err (int32, caller-zeroed) receives, by atomic
+ * max, the largest index value > 4095 seen (clamped to INT32_MAX), so the caller can
+ * raise the reference's "exceeds 12-bit limit" error at its next synchronisation;
+ * negative indices are packed by their low bits exactly as the reference does. */
+int tplr_pack12(const int64_t* d_idx, int64_t n, uint8_t* d_packed, int32_t* d_err, void* stream);
+
+/* Replaces unpack_12bit_indices (src/tplr/compress.py:102-142): n int64 indices
+ * from 3n/2 bytes.  n must be even. */
+int tplr_unpack12(const uint8_t* d_packed, int64_t n, int64_t* d_idx, void* stream);
+
+/* The same two routines on HOST memory, for payloads that are validated before they are
+ * moved to the device (unpack_12bit_indices is called on downloaded tensors by
+ * src/tplr/comms.py:2599 and src/tplr/neurons.py:1361).  *bad (nullable) receives the
+ * largest index > 4095, or 0. */
+int tplr_pack12_host(const int64_t* idx, int64_t n, uint8_t* packed, int64_t* bad);
+int tplr_unpack12_host(const uint8_t* packed, int64_t n, int64_t* idx);
+
+/* ---- chunked 2-D DCT ------------------------------------------------------------
+ * Replaces ChunkingTransformer.encode(use_dct=True) for 2-D tensors whose chunk is
+ * 64x64 (src/tplr/compress.py:236-246, einsum :203): d_x is (R, C) row-major with
+ * row stride ld_x elements, d_coef is (R/64, C/64, 64, 64) contiguous,
+ * coef[y,x] = F^T X[y,x] F with the orthonormal DCT-II basis. */
+int tplr_dct2d_fwd(const float* d_x, int64_t R, int64_t C, int64_t ld_x, float* d_coef, void* stream);
+
+/* Replaces ChunkingTransformer.decode(use_dct=True) (src/tplr/compress.py:271-281,
+ * einsum :222): d_coef (R/64, C/64, 64, 64) -> d_x (R, C), x[y,x] = F coef[y,x] F^T. */
+int tplr_dct2d_inv(const float* d_coef, int64_t R, int64_t C, float* d_x, int64_t ld_x, void* stream);
+
+/* 1-D tensors (src/tplr/compress.py:248-255, :283-290): n_vec rows of 64 floats,
+ * each row r <- r @ F (inverse = 0) or r @ F^T (inverse = 1). */
+int tplr_dct1d(const float* d_in, int64_t n_vec, int inverse, float* d_out, void* stream);
+
+/* Any chunk size h, w <= 64 (non-64 divisors chosen by _get_smaller_split,
+ * src/tplr/compress.py:853-872; also einsum_2d / einsum_2d_t, :186-222, with arbitrary
+ * bases): dense contraction out = Bh^T X Bw per (h, w) chunk with caller-supplied
+ * d_bh (h, h) and d_bw (w, w), row-major.  Pass f_dict[h], f_dict[w] to encode and
+ * b_dict[h], b_dict[w] to decode.  in_chunked / out_chunked select the layout of each
+ * side: 0 = (R, C) row-major, 1 = (R/h, C/w, h, w) contiguous.  h = 1 gives the 1-D
+ * form row @ Bw. */
+int tplr_dct2d_dense(const float* d_in, int64_t R, int64_t C, int h, int w,
+                     const float* d_bh, const float* d_bw, int in_chunked, int out_chunked,
+                     float* d_out, void* stream);
+
+/* ---- top-k select + value gather + 12-bit pack -----------------------------------
+ * Replaces TopKCompressor.compress without quantisation (src/tplr/compress.py:402-416)
+ * on n_rows rows of row_len fp32 coefficients (row_len = 4096 for 2-D chunks, 64 for
+ * 1-D tensors, anything <= TPLR_MAX_ROW otherwise).  k even, 2 <= k <= min(row_len, 128).
+ * Outputs: d_idx12 = n_rows * k * 3/2 bytes, d_val = (n_rows, k) signed values.
+ * This is the coefficient-input entry used for the bit-exact parity stage. */
+int tplr_topk_pack(const float* d_coef, int64_t n_rows, int64_t row_len, int k,
+                   uint8_t* d_idx12, float* d_val, void* stream);
+
+/* Fused encode: tplr_dct2d_fwd (use_dct != 0) or plain chunking (use_dct == 0)
+ * followed by tplr_topk_pack with row_len 4096, without writing the coefficients
+ * to memory (src/tplr/neurons.py:155-159 calls encode then compress back to back).
+ * k in {2,...,128}, even. */
+int tplr_encode_topk_pack(const float* d_x, int64_t R, int64_t C, int64_t ld_x, int k, int use_dct,
+                          uint8_t* d_idx12, float* d_val, void* stream);
+
+/* ---- decode side -----------------------------------------------------------------
+ * Fused TopKCompressor.batch_decompress + ChunkingTransformer.decode
+ * (src/tplr/compress.py:483-580 then :259-292; caller: src/tplr/neurons.py:355-367).
+ * For every chunk: unpack the 12-bit indices of n_peers payloads, multiply peer p's
+ * values by d_peer_scale[p] (NULL = 1; the median-norm clip factors of
+ * src/tplr/compress.py:553-556), or, when normalise != 0, divide them by their
+ * per-chunk L2 norm + 1e-8 (:541-545); accumulate in peer order; divide every touched
+ * coefficient by its number of contributions (scatter_reduce "mean",
+ * include_self=False, :472-474) unless reduce_mode = TPLR_REDUCE_SUM; then apply the
+ * inverse DCT (use_dct != 0, output (R, C) row stride ld_out) or write the dense
+ * coefficients as (R/64, C/64, 64, 64) (use_dct == 0, ld_out ignored).
+ * h_idx12 / h_val are HOST arrays of n_peers DEVICE pointers: payload p holds
+ * n_chunks*k*3/2 index bytes and (n_chunks, k) values.  d_sumsq (nullable) receives
+ * n_chunks partial sums of squares of the output, one per chunk. */
+int tplr_decode_aggregate(const uint8_t* const* h_idx12, const float* const* h_val,
+                          const float* d_peer_scale, int n_peers, int k,
+                          int64_t R, int64_t C, int reduce_mode, int normalise, int use_dct,
+                          float* d_out, int64_t ld_out, float* d_sumsq, void* stream);
+
+/* Row-wise scatter for layouts that are not 64x64 chunks (1-D tensors, un-chunked
+ * 2-D rows; TopKCompressor.decompress, src/tplr/compress.py:452-474): d_out is
+ * (n_rows, row_len) zero-filled then d_val[r, j] * scale accumulated at d_idx[r, j]
+ * in j order and averaged per destination.  Exactly one of d_idx12 (packed) and
+ * d_idx64 (int64, as produced by unpack / batch concatenation) is non-NULL.
+ * row_len <= TPLR_MAX_ROW.  d_err as in tplr_pack12: receives the largest
+ * out-of-range index (>= row_len) seen; such entries are skipped. */
+int tplr_scatter_rows(const uint8_t* d_idx12, const int64_t* d_idx64, const float* d_val,
+                      int64_t n_rows, int64_t k_per_row, int64_t row_len, int reduce_mode,
+                      float* d_out, int32_t* d_err, void* stream);
+
+/* ---- peer statistics (src/tplr/compress.py:526-535, :553-556) ---------------------
+ * d_sumsq[p] = sum of squares of payload p's n values (h_val: HOST array of n_peers
+ * DEVICE pointers). */
+int tplr_peer_sumsq(const float* const* h_val, int n_peers, int64_t n, float* d_sumsq, void* stream);
+
+/* d_scale[p] = min(1, med / (norm_p + 1e-8)), med = lower median of the norms
+ * (torch.median), norm_p = d_norm[p] (is_sumsq == 0) or sqrt(d_norm[p]) (is_sumsq != 0).
+ * d_median (nullable) receives med. */
+int tplr_clip_scales(const float* d_norm, int n_peers, int is_sumsq, float* d_scale, float* d_median,
+                     void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPLR_HIP_H */

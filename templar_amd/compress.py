@@ -1,0 +1,751 @@
+"""Host-side mirror of templar's gradient codec API (reference: src/tplr/compress.py,
+tplr 2.1.28) on top of libtplr_hip.so.
+
+Same names, arguments, return tuples and error messages as the reference, so that
+`neurons/miner.py`, `neurons/validator.py` and `src/tplr/neurons.py` can use this module in
+place of `tplr.compress`:
+
+    pack_12bit_indices / unpack_12bit_indices          (reference :51-142)
+    ChunkingTransformer.encode / decode / einsum_2d(_t) (reference :145-292)
+    TopKCompressor.compress / decompress / batch_decompress / quantiser (reference :295-696)
+    _dct, _idct, _get_smaller_split, _get_divisors, _get_prime_divisors (reference :700-872)
+    TransformDCT = ChunkingTransformer, CompressDCT = TopKCompressor     (DeMo-era names)
+
+All tensor arithmetic of the codec runs in the HIP library on the tensor's device and on
+torch's current stream; nothing here synchronises except where the reference does
+(`pack_12bit_indices` reads back the range-check flag, as the reference's `.item()` does).
+Only the basis construction at start-up and the small statistical quantiser use torch ops.
+The two fused entry points `encode_compress` and `batch_decompress_decode` do what the
+callers' back-to-back `encode`+`compress` and `batch_decompress`+`decode` do, in one kernel
+each and without materialising the dense coefficient tensor.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Sequence, TypeAlias
+
+import torch
+
+from . import _lib
+
+try:  # DTensor inputs are unwrapped exactly where the reference does (:398-399)
+    from torch.distributed.tensor import DTensor as _DT
+except Exception:  # pragma: no cover - torch without distributed
+    _DT = ()
+
+ShapeT: TypeAlias = tuple[int, ...]
+Shape4D = tuple[int, int, int, int]
+TotK: TypeAlias = int
+IdxT: TypeAlias = torch.Tensor
+ValT: TypeAlias = torch.Tensor
+QuantParamsT: TypeAlias = tuple[torch.Tensor, float, int, torch.Tensor, torch.dtype]
+
+_CH = 64  # chunk edge served by the factorised transform kernels
+
+
+# ----------------------------------------------------------------------------------------
+# plumbing
+# ----------------------------------------------------------------------------------------
+def _ptr(t: torch.Tensor | None):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream(dev: torch.device):
+    return C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _need_device(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"templar_amd.{what}: tensor is on '{t.device}'; the codec kernels run on a HIP device only "
+            "(there is no CPU code path)"
+        )
+
+
+def _f32c(t: torch.Tensor) -> torch.Tensor:
+    """fp32, contiguous (the kernels' only element type)."""
+    if t.dtype != torch.float32:
+        t = t.float()
+    return t.contiguous()
+
+
+# ----------------------------------------------------------------------------------------
+# 12-bit index packing (reference :51-142)
+# ----------------------------------------------------------------------------------------
+def pack_12bit_indices(indices: torch.Tensor) -> torch.Tensor:
+    """Pack an even number of indices < 4096 into 3 bytes per pair (reference :51-99)."""
+    lib = _lib.load()
+    n = indices.numel()
+    flat = indices.reshape(-1)
+    if flat.dtype != torch.int64:
+        flat = flat.to(torch.int64)
+    flat = flat.contiguous()
+    if flat.is_cuda:
+        with torch.cuda.device(flat.device):
+            # the reference finds the maximum first (and raises on it) before the parity check
+            err = torch.zeros(1, dtype=torch.int32, device=flat.device)
+            out = torch.empty((n // 2) * 3, dtype=torch.uint8, device=flat.device)
+            if n >= 2:
+                st = lib.tplr_pack12(_ptr(flat), n - (n % 2), _ptr(out), _ptr(err), _stream(flat.device))
+                _lib.check(st, "tplr_pack12")
+            worst = int(err.item())  # the reference synchronises here as well (.item(), :64)
+            if n % 2:
+                worst = max(worst, int(flat[-1].item()))
+    else:
+        out = torch.empty((n // 2) * 3, dtype=torch.uint8)
+        bad = C.c_int64(0)
+        if n >= 2:
+            st = lib.tplr_pack12_host(_ptr(flat), n - (n % 2), _ptr(out), C.byref(bad))
+            _lib.check(st, "tplr_pack12_host")
+        worst = int(bad.value)
+        if n % 2:
+            worst = max(worst, int(flat[-1]))
+    if worst >= 4096:
+        raise ValueError(f"Index {worst} exceeds 12-bit limit (4095)")
+    if n % 2 != 0:
+        raise ValueError(f"Number of indices must be even, got {n}")
+    return out
+
+
+def unpack_12bit_indices(packed: torch.Tensor, values_shape: ShapeT) -> torch.Tensor:
+    """Inverse of pack_12bit_indices; int64 tensor of `values_shape` (reference :102-142)."""
+    n = int(math.prod(tuple(values_shape)))
+    if n == 0:
+        return torch.zeros(tuple(values_shape), dtype=torch.int64, device=packed.device)
+    if n % 2 != 0:
+        raise ValueError(f"Number of indices must be even, got {n}")
+    if packed.dtype != torch.uint8:
+        packed = packed.to(torch.uint8)
+    packed = packed.reshape(-1).contiguous()
+    if packed.numel() * 2 != n * 3:
+        # the reference fails here with torch's shape-mismatch RuntimeError
+        raise RuntimeError(
+            f"shape mismatch: {packed.numel()} packed bytes cannot hold {n} 12-bit indices (need {n // 2 * 3})"
+        )
+    lib = _lib.load()
+    out = torch.empty(n, dtype=torch.int64, device=packed.device)
+    if packed.is_cuda:
+        with torch.cuda.device(packed.device):
+            _lib.check(lib.tplr_unpack12(_ptr(packed), n, _ptr(out), _stream(packed.device)), "tplr_unpack12")
+    else:
+        _lib.check(lib.tplr_unpack12_host(_ptr(packed), n, _ptr(out)), "tplr_unpack12_host")
+    return out.reshape(tuple(values_shape))
+
+
+# ----------------------------------------------------------------------------------------
+# divisor rule and basis (reference :700-872)
+# ----------------------------------------------------------------------------------------
+def _get_prime_divisors(n: int) -> list[int]:
+    """Prime factors of n with multiplicity, ascending (reference :791-817)."""
+    out: list[int] = []
+    p = 2
+    while p * p <= n:
+        while n % p == 0:
+            out.append(p)
+            n //= p
+        p += 1 if p == 2 else 2
+    if n > 1:
+        out.append(n)
+    return out
+
+
+def _get_divisors(n: int) -> list[int]:
+    """All divisors of n, ascending; [] for n < 1 (reference :820-850)."""
+    if n < 1:
+        return []
+    small = [d for d in range(1, math.isqrt(n) + 1) if n % d == 0]
+    large = [n // d for d in reversed(small) if d * d != n]
+    return small + large
+
+
+def _get_smaller_split(n: int, close_to: int) -> int:
+    """Largest divisor of n that is <= close_to; the smallest divisor if none is; n itself
+    when every divisor is below close_to (reference :853-872)."""
+    divs = _get_divisors(n)
+    for pos, d in enumerate(divs):
+        if d == close_to:
+            return d
+        if d > close_to:
+            return d if pos == 0 else divs[pos - 1]
+    return n
+
+
+def _cos_table(n: int, dtype, device) -> torch.Tensor:
+    i = torch.arange(n, dtype=torch.float64, device=device)
+    return torch.cos(math.pi * (2.0 * i[:, None] + 1.0) * i[None, :] / (2.0 * n))  # [sample, freq]
+
+
+def _dct(x: torch.Tensor, norm: str | None = None) -> torch.Tensor:
+    """DCT-II over the last dimension with torch-dct scaling (reference :710-741):
+    norm=None gives 2*sum_n x[n] cos(pi(2n+1)k/2N); norm="ortho" the orthonormal transform."""
+    n = x.shape[-1]
+    m = 2.0 * _cos_table(n, x.dtype, x.device)
+    if norm == "ortho":
+        m[:, 0] *= 1.0 / (2.0 * math.sqrt(n))
+        m[:, 1:] *= 1.0 / (2.0 * math.sqrt(n / 2.0))
+    return (x.to(torch.float64) @ m).to(x.dtype)
+
+
+def _idct(X: torch.Tensor, norm: str | None = None) -> torch.Tensor:
+    """Inverse of _dct (a scaled DCT-III), reference :744-788."""
+    n = X.shape[-1]
+    c = _cos_table(n, X.dtype, X.device)  # [sample, freq]
+    if norm == "ortho":
+        w = torch.full((n,), math.sqrt(2.0 / n), dtype=torch.float64, device=X.device)
+        w[0] = math.sqrt(1.0 / n)
+    else:
+        w = torch.full((n,), 1.0 / n, dtype=torch.float64, device=X.device)
+        w[0] = 1.0 / (2.0 * n)
+    return ((X.to(torch.float64) * w) @ c.T).to(X.dtype)
+
+
+# ----------------------------------------------------------------------------------------
+# ChunkingTransformer (reference :145-292)
+# ----------------------------------------------------------------------------------------
+class ChunkingTransformer:
+    """Chunks tensors into (y, x, h, w) blocks and applies the per-chunk 2-D DCT."""
+
+    @torch.no_grad()
+    def __init__(self, model, target_chunk, norm="ortho"):
+        self.target_chunk = target_chunk
+        self.shape_dict: dict[int, int] = {}
+        self.f_dict: dict[int, torch.Tensor] = {}
+        self.b_dict: dict[int, torch.Tensor] = {}
+        for _, p in model.named_parameters():
+            if not p.requires_grad:
+                continue
+            for s in p.shape:
+                sc = _get_smaller_split(s, self.target_chunk)
+                self.shape_dict[s] = sc
+                if sc not in self.f_dict:
+                    eye = torch.eye(sc)
+                    self.f_dict[sc] = _dct(eye, norm=norm).to(p.dtype).to(p.device)
+                    self.b_dict[sc] = _idct(eye, norm=norm).to(p.dtype).to(p.device)
+
+    # -- dense contraction through the library (any basis, chunk edge <= 64) --------------
+    @staticmethod
+    def _basis32(table: dict, n: int, dev: torch.device) -> torch.Tensor:
+        return table[n].to(device=dev, dtype=torch.float32).contiguous()
+
+    @staticmethod
+    def _dense(x: torch.Tensor, R: int, Cc: int, h: int, w: int, bh: torch.Tensor, bw: torch.Tensor,
+               in_chunked: bool, out_chunked: bool) -> torch.Tensor:
+        _need_device(x, "ChunkingTransformer (DCT)")
+        if h > 64 or w > 64:
+            raise NotImplementedError(f"chunk {h}x{w}: the HIP transform kernels handle chunk edges up to 64")
+        lib = _lib.load()
+        xin = _f32c(x)
+        out = torch.empty((R // h, Cc // w, h, w) if out_chunked else (R, Cc), dtype=torch.float32, device=x.device)
+        if out.numel():
+            with torch.cuda.device(x.device):
+                st = lib.tplr_dct2d_dense(_ptr(xin), R, Cc, h, w, _ptr(_f32c(bh)), _ptr(_f32c(bw)), int(in_chunked),
+                                          int(out_chunked), _ptr(out), _stream(x.device))
+            _lib.check(st, "tplr_dct2d_dense")
+        return out
+
+    @torch.no_grad()
+    def einsum_2d(self, x, b, d=None) -> torch.Tensor:
+        """"...ij, jb -> ...ib" (d is None) or "...ijkl, kb, ld -> ...ijbd" (reference :186-203)."""
+        if d is None:
+            rows = x.reshape(-1, x.shape[-1])
+            one = torch.ones(1, 1, dtype=torch.float32, device=x.device)
+            out = self._dense(rows, rows.shape[0], rows.shape[1], 1, rows.shape[1], one, b, False, True)
+            return out.reshape(x.shape[:-1] + (b.shape[1],)).to(x.dtype)
+        lead = x.shape[:-4]
+        y4 = x.reshape((-1,) + tuple(x.shape[-3:]))  # fold leading dims and y together
+        Y, X, h, w = y4.shape
+        out = self._dense(y4, Y * h, X * w, h, w, b, d, True, True)
+        return out.reshape(lead + tuple(x.shape[-4:])).to(x.dtype)
+
+    @torch.no_grad()
+    def einsum_2d_t(self, x, b, d=None) -> torch.Tensor:
+        """"...ij, jb -> ...ib" (d is None) or "...ijbd, bk, dl -> ...ijkl" (reference :205-222)."""
+        return self.einsum_2d(x, b, d)
+
+    # -- encode / decode ------------------------------------------------------------------
+    @torch.no_grad()
+    def encode(self, x: torch.Tensor, *, use_dct: bool = False) -> torch.Tensor:
+        """(R, C) -> (R/h, C/w, h, w), or (N,) -> (N/w, w); DCT-II per chunk when use_dct
+        (reference :224-257).  Without use_dct the result is a view, as in the reference."""
+        if x.dim() > 1:
+            n1 = self.shape_dict[x.shape[0]]
+            n2 = self.shape_dict[x.shape[1]]
+            R, Cc = x.shape
+            if not use_dct:
+                return x.reshape(R // n1, n1, Cc // n2, n2).permute(0, 2, 1, 3)
+            _need_device(x, "ChunkingTransformer.encode(use_dct=True)")
+            if n1 == _CH and n2 == _CH:
+                lib = _lib.load()
+                xin = x if (x.dtype == torch.float32 and x.stride(1) == 1 and x.stride(0) >= Cc) else _f32c(x)
+                out = torch.empty((R // _CH, Cc // _CH, _CH, _CH), dtype=torch.float32, device=x.device)
+                with torch.cuda.device(x.device):
+                    st = lib.tplr_dct2d_fwd(_ptr(xin), R, Cc, xin.stride(0), _ptr(out), _stream(x.device))
+                _lib.check(st, "tplr_dct2d_fwd")
+                return out if x.dtype == torch.float32 else out.to(x.dtype)
+            out = self._dense(x, R, Cc, n1, n2, self._basis32(self.f_dict, n1, x.device),
+                              self._basis32(self.f_dict, n2, x.device), False, True)
+            return out if x.dtype == torch.float32 else out.to(x.dtype)
+        n1 = self.shape_dict[x.shape[0]]
+        rows = x.reshape(-1, n1)
+        if not use_dct:
+            return rows
+        _need_device(x, "ChunkingTransformer.encode(use_dct=True)")
+        if n1 == _CH:
+            lib = _lib.load()
+            xin = _f32c(rows)
+            out = torch.empty_like(xin)
+            with torch.cuda.device(x.device):
+                st = lib.tplr_dct1d(_ptr(xin), xin.shape[0], 0, _ptr(out), _stream(x.device))
+            _lib.check(st, "tplr_dct1d")
+            return out if x.dtype == torch.float32 else out.to(x.dtype)
+        return self.einsum_2d(rows, self._basis32(self.f_dict, n1, x.device))
+
+    @torch.no_grad()
+    def decode(self, x: torch.Tensor, *, use_dct: bool = False) -> torch.Tensor:
+        """(y, x, h, w) -> (y*h, x*w), or (x, w) -> (x*w,); inverse DCT per chunk when use_dct
+        (reference :259-292)."""
+        if isinstance(x, LazyAggregate):
+            return x.decode(use_dct=use_dct)
+        if x.dim() > 2:
+            Y, X, h, w = x.shape
+            if not use_dct:
+                return x.permute(0, 2, 1, 3).reshape(Y * h, X * w)
+            _need_device(x, "ChunkingTransformer.decode(use_dct=True)")
+            if h == _CH and w == _CH:
+                lib = _lib.load()
+                xin = _f32c(x)
+                out = torch.empty((Y * h, X * w), dtype=torch.float32, device=x.device)
+                with torch.cuda.device(x.device):
+                    st = lib.tplr_dct2d_inv(_ptr(xin), Y * h, X * w, _ptr(out), X * w, _stream(x.device))
+                _lib.check(st, "tplr_dct2d_inv")
+                return out if x.dtype == torch.float32 else out.to(x.dtype)
+            out = self._dense(x, Y * h, X * w, h, w, self._basis32(self.b_dict, h, x.device),
+                              self._basis32(self.b_dict, w, x.device), True, False)
+            return out if x.dtype == torch.float32 else out.to(x.dtype)
+        if not use_dct:
+            return x.reshape(-1)
+        _need_device(x, "ChunkingTransformer.decode(use_dct=True)")
+        n1 = x.shape[1]
+        if n1 == _CH:
+            lib = _lib.load()
+            xin = _f32c(x)
+            out = torch.empty_like(xin)
+            with torch.cuda.device(x.device):
+                st = lib.tplr_dct1d(_ptr(xin), xin.shape[0], 1, _ptr(out), _stream(x.device))
+            _lib.check(st, "tplr_dct1d")
+            out = out.reshape(-1)
+            return out if x.dtype == torch.float32 else out.to(x.dtype)
+        return self.einsum_2d_t(x, self._basis32(self.b_dict, n1, x.device)).reshape(-1)
+
+
+# ----------------------------------------------------------------------------------------
+# kernels behind TopKCompressor
+# ----------------------------------------------------------------------------------------
+def _as_chunk_view(x: torch.Tensor):
+    """If x is the zero-copy (Y, X, 64, 64) view of a row-major (R, C) fp32 tensor that
+    encode(use_dct=False) returns, give (R, C, ld); else None."""
+    if x.dim() != 4 or x.dtype != torch.float32 or x.shape[2] != _CH or x.shape[3] != _CH:
+        return None
+    Y, X = x.shape[0], x.shape[1]
+    s = x.stride()
+    ld = s[2]
+    if s[3] == 1 and s[1] == _CH and ld >= X * _CH and (s[0] == _CH * ld or Y == 1):
+        return Y * _CH, X * _CH, ld
+    return None
+
+
+def _clamp_k(last_dim: int, topk: int) -> int:
+    k = max(min(int(topk), int(last_dim)), 2)
+    return k - (k % 2)
+
+
+def _row_layout(xshape: tuple) -> tuple[int, int]:
+    """(number of rows, row length) of the flattened-last-dims view compress/decompress use."""
+    if len(xshape) > 2:
+        return xshape[0] * xshape[1], xshape[2] * xshape[3]
+    return (math.prod(xshape[:-1]) if len(xshape) > 1 else 1), xshape[-1]
+
+
+def _topk_rows(rows: torch.Tensor, k: int):
+    """rows (n_rows, n) fp32 contiguous on device -> (packed idx uint8, val (n_rows, k))."""
+    n_rows, n = rows.shape
+    if n > _lib.TPLR_MAX_ROW or k > _lib.TPLR_MAX_K:
+        raise NotImplementedError(
+            f"top-{k} of rows of {n}: the HIP select kernel handles rows up to {_lib.TPLR_MAX_ROW} and "
+            f"k up to {_lib.TPLR_MAX_K}"
+        )
+    lib = _lib.load()
+    idx = torch.empty(n_rows * (k // 2) * 3, dtype=torch.uint8, device=rows.device)
+    val = torch.empty((n_rows, k), dtype=torch.float32, device=rows.device)
+    if n_rows:
+        with torch.cuda.device(rows.device):
+            st = lib.tplr_topk_pack(_ptr(rows), n_rows, n, k, _ptr(idx), _ptr(val), _stream(rows.device))
+        _lib.check(st, "tplr_topk_pack")
+    return idx, val
+
+
+def _encode_topk(x2d: torch.Tensor, R: int, Cc: int, ld: int, k: int, use_dct: bool):
+    if k > _lib.TPLR_MAX_K:
+        raise NotImplementedError(f"top-{k}: the HIP select kernel handles k up to {_lib.TPLR_MAX_K}")
+    lib = _lib.load()
+    n_chunks = (R // _CH) * (Cc // _CH)
+    idx = torch.empty(n_chunks * (k // 2) * 3, dtype=torch.uint8, device=x2d.device)
+    val = torch.empty((R // _CH, Cc // _CH, k), dtype=torch.float32, device=x2d.device)
+    if n_chunks:
+        with torch.cuda.device(x2d.device):
+            st = lib.tplr_encode_topk_pack(_ptr(x2d), R, Cc, ld, k, int(use_dct), _ptr(idx), _ptr(val),
+                                           _stream(x2d.device))
+        _lib.check(st, "tplr_encode_topk_pack")
+    return idx, val
+
+
+def _peer_scales(vals: Sequence[torch.Tensor], block_norms: torch.Tensor | None, dev: torch.device) -> torch.Tensor:
+    """Clip factors min(1, median / (norm_p + 1e-8)) on the device (reference :526-535, :553-556)."""
+    lib = _lib.load()
+    P = len(vals)
+    if P > _lib.TPLR_MAX_PEERS:
+        raise NotImplementedError(f"{P} peers: the HIP aggregate kernel takes up to {_lib.TPLR_MAX_PEERS}")
+    scale = torch.empty(P, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        if block_norms is not None:
+            norms = block_norms.to(device=dev, dtype=torch.float32).contiguous()
+            st = lib.tplr_clip_scales(_ptr(norms), P, 0, _ptr(scale), None, _stream(dev))
+        else:
+            ptrs = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
+            ss = torch.empty(P, dtype=torch.float32, device=dev)
+            n = vals[0].numel()
+            if any(v.numel() != n for v in vals):
+                raise ValueError("batch_decompress: all peers must send the same number of values")
+            _lib.check(lib.tplr_peer_sumsq(ptrs, P, n, _ptr(ss), _stream(dev)), "tplr_peer_sumsq")
+            st = lib.tplr_clip_scales(_ptr(ss), P, 1, _ptr(scale), None, _stream(dev))
+    _lib.check(st, "tplr_clip_scales")
+    return scale
+
+
+def _aggregate_chunks(idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], scale: torch.Tensor | None,
+                      Y: int, X: int, k: int, *, normalise: bool, use_dct: bool, mean: bool = True,
+                      out: torch.Tensor | None = None, sumsq: torch.Tensor | None = None) -> torch.Tensor:
+    """Fused unpack + scatter over peers (+ inverse DCT) on 64x64 chunks."""
+    lib = _lib.load()
+    P = len(vals)
+    dev = vals[0].device
+    if P > _lib.TPLR_MAX_PEERS:
+        raise NotImplementedError(f"{P} peers: the HIP aggregate kernel takes up to {_lib.TPLR_MAX_PEERS}")
+    n_chunks = Y * X
+    for i, v in zip(idxs, vals):
+        if v.numel() != n_chunks * k or i.numel() * 2 != n_chunks * k * 3:
+            raise RuntimeError(
+                f"payload size mismatch: {i.numel()} index bytes / {v.numel()} values for {n_chunks} chunks, k={k}"
+            )
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+    vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
+    R, Cc = Y * _CH, X * _CH
+    if out is None:
+        out = torch.empty((R, Cc) if use_dct else (Y, X, _CH, _CH), dtype=torch.float32, device=dev)
+    if n_chunks:
+        with torch.cuda.device(dev):
+            st = lib.tplr_decode_aggregate(ip, vp, _ptr(scale), P, k, R, Cc,
+                                           _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM, int(normalise), int(use_dct),
+                                           _ptr(out), out.stride(0) if use_dct else 0, _ptr(sumsq), _stream(dev))
+        _lib.check(st, "tplr_decode_aggregate")
+    return out
+
+
+def _scatter_rows(idx: torch.Tensor, val: torch.Tensor, n_rows: int, kk: int, row_len: int) -> torch.Tensor:
+    """Generic rows: idx is packed uint8 or int64, val is (rows_sent, kk) with rows_sent <= n_rows
+    (torch's scatter lets the index cover fewer rows than the target; the rest stay zero)."""
+    if row_len > _lib.TPLR_MAX_ROW:
+        raise NotImplementedError(f"rows of {row_len}: the HIP scatter kernel handles rows up to {_lib.TPLR_MAX_ROW}")
+    lib = _lib.load()
+    dev = val.device
+    rows_sent = val.numel() // kk if kk else 0
+    if rows_sent > n_rows:
+        raise RuntimeError(f"{rows_sent} rows of values for a target of {n_rows} rows")
+    out = torch.empty((n_rows, row_len), dtype=torch.float32, device=dev)
+    if rows_sent < n_rows:
+        out[rows_sent:].zero_()
+    n_rows = rows_sent
+    if n_rows == 0:
+        return out
+    err = torch.zeros(1, dtype=torch.int32, device=dev)
+    packed = idx.dtype == torch.uint8
+    with torch.cuda.device(dev):
+        st = lib.tplr_scatter_rows(_ptr(idx) if packed else None, None if packed else _ptr(idx), _ptr(val), n_rows, kk,
+                                   row_len, _lib.REDUCE_MEAN, _ptr(out), _ptr(err), _stream(dev))
+    _lib.check(st, "tplr_scatter_rows")
+    bad = int(err.item())  # the reference's scatter raises on an out-of-range index as well
+    if bad:
+        raise RuntimeError(f"index {bad} is out of bounds for dimension -1 with size {row_len}")
+    return out
+
+
+class LazyAggregate:
+    """What batch_decompress returns when `defer=True`: the peers' payloads plus clip factors,
+    not yet scattered.  ChunkingTransformer.decode() turns it into the dense gradient with the
+    fused kernel; `.dense()` gives the coefficient tensor the reference would have returned."""
+
+    def __init__(self, idxs, vals, scale, xshape, k, normalise, dtype):
+        self.idxs, self.vals, self.scale = idxs, vals, scale
+        self.shape = tuple(xshape)
+        self.k, self.normalise, self.dtype = k, normalise, dtype
+        self.device = vals[0].device
+
+    def dense(self) -> torch.Tensor:
+        Y, X = self.shape[0], self.shape[1]
+        out = _aggregate_chunks(self.idxs, self.vals, self.scale, Y, X, self.k, normalise=self.normalise, use_dct=False)
+        return out if self.dtype == torch.float32 else out.to(self.dtype)
+
+    def decode(self, *, use_dct: bool) -> torch.Tensor:
+        Y, X = self.shape[0], self.shape[1]
+        if not use_dct:
+            return self.dense().permute(0, 2, 1, 3).reshape(Y * _CH, X * _CH)
+        out = _aggregate_chunks(self.idxs, self.vals, self.scale, Y, X, self.k, normalise=self.normalise, use_dct=True)
+        return out if self.dtype == torch.float32 else out.to(self.dtype)
+
+
+# ----------------------------------------------------------------------------------------
+# TopKCompressor (reference :295-696)
+# ----------------------------------------------------------------------------------------
+class TopKCompressor:
+    """Top-k sparsifier with 12-bit index packing and the optional 8-bit value quantiser."""
+
+    use_quantization: bool
+    n_bins: int
+    range_in_sigmas: int
+
+    def __class_getitem__(cls, item):  # TopKCompressor[Literal[True]] in annotations
+        return cls
+
+    @torch.no_grad()
+    def __init__(self, *, use_quantization: bool = False, quantization_bins: int = 256,
+                 quantization_range: int = 6) -> None:
+        self.use_quantization = use_quantization
+        if self.use_quantization:
+            self.n_bins = quantization_bins
+            self.range_in_sigmas = quantization_range
+
+    def _clamp_topk(self, x, topk) -> int:
+        """min(topk, last dim), at least 2, rounded down to even (reference :352-367)."""
+        return _clamp_k(x.shape[-1], topk)
+
+    @torch.no_grad()
+    def compress(self, x: torch.Tensor, topk: int):
+        """Top-k by magnitude per chunk / row -> (packed idx, values, xshape, totalk[, qparams])
+        (reference :385-423).  Values come out in descending-magnitude order."""
+        if _DT and isinstance(x, _DT):
+            x = x.to_local()
+        xshape = x.shape
+        _need_device(x, "TopKCompressor.compress")
+        totalk = (x.shape[2] * x.shape[3]) if x.dim() > 2 else x.shape[-1]
+        topk = _clamp_k(totalk, topk)
+
+        view = _as_chunk_view(x)
+        if view is not None and topk <= _lib.TPLR_MAX_K:
+            R, Cc, ld = view  # the un-transformed chunk view of a dense tensor: select straight from it
+            idx, val = _encode_topk(x, R, Cc, ld, topk, use_dct=False)
+        else:
+            rows = _f32c(x).reshape(-1, totalk)
+            idx, val = _topk_rows(rows, topk)
+            val = val.reshape(tuple(x.shape[:2]) + (topk,)) if x.dim() > 2 else val.reshape(tuple(x.shape[:-1]) + (topk,))
+        if val.dtype != x.dtype:
+            val = val.to(x.dtype)
+        if self.use_quantization:
+            val, qparams = self._quantize_values(val)
+            return idx, val, xshape, totalk, qparams
+        return idx, val, xshape, totalk
+
+    @torch.no_grad()
+    def decompress(self, p: torch.Tensor, idx: torch.Tensor, val: torch.Tensor, xshape: ShapeT, totalk: int,
+                   quantize_params: QuantParamsT | None = None) -> torch.Tensor:
+        """Scatter values back into a zero tensor of `xshape`, averaging duplicates
+        (reference :425-481).  `p` only supplies device and dtype."""
+        if self.use_quantization and quantize_params is not None:
+            val = self._dequantize_values(val, quantize_params)
+        if idx.dtype not in (torch.uint8, torch.int64):
+            raise ValueError(f"Expected uint8 (packed) or int64 (unpacked) indices, got {idx.dtype}")
+        _need_device(p, "TopKCompressor.decompress")
+        dev = p.device
+        val = _f32c(val.to(dev))
+        idx = idx.to(dev).contiguous()
+        xshape = tuple(xshape)
+        kk = val.shape[-1]
+        n_rows, row_len = _row_layout(xshape)
+        if (len(xshape) > 2 and xshape[2] == _CH and xshape[3] == _CH and idx.dtype == torch.uint8 and kk % 2 == 0
+                and kk >= 2 and val.numel() == n_rows * kk):
+            out = _aggregate_chunks([idx.reshape(-1)], [val], None, xshape[0], xshape[1], kk, normalise=False,
+                                    use_dct=False)
+        else:
+            if idx.dtype == torch.uint8:
+                if kk % 2:
+                    # the reference's unpack rejects an odd count
+                    raise ValueError(f"Number of indices must be even, got {val.numel()}")
+                if idx.numel() * 2 != val.numel() * 3:
+                    raise RuntimeError(f"{idx.numel()} packed bytes cannot hold {val.numel()} 12-bit indices")
+            elif idx.numel() != val.numel():
+                raise RuntimeError(f"index shape {tuple(idx.shape)} does not match values {tuple(val.shape)}")
+            out = _scatter_rows(idx.reshape(-1), val, n_rows, kk, row_len).reshape(xshape)
+        return out if p.dtype == torch.float32 else out.to(p.dtype)
+
+    @torch.no_grad()
+    def batch_decompress(self, p: torch.Tensor, idx: torch.Tensor | Sequence[torch.Tensor],
+                         val: torch.Tensor | Sequence[torch.Tensor], xshape: ShapeT, totalk: int,
+                         quantize_params: Sequence[QuantParamsT] | None = None, *,
+                         block_norms: torch.Tensor | None = None, normalise: bool = False, clip_norm: bool = True,
+                         defer: bool = False):
+        """Combine several peers' payloads: per-peer median-norm clip (or per-chunk
+        normalisation), then the coefficient-wise mean over the peers that sent each
+        coefficient (reference :483-580).  With `defer=True` (an extension) the scatter is
+        postponed so that ChunkingTransformer.decode() can run it fused with the inverse DCT."""
+        if quantize_params is not None and not isinstance(quantize_params, list):
+            quantize_params = [quantize_params] * len(val)
+        val_list = list(val) if isinstance(val, (list, tuple)) else [val]
+        idx_list = list(idx) if isinstance(idx, (list, tuple)) else [idx]
+        if self.use_quantization and quantize_params:
+            val_list = [self._dequantize_values(v, quantize_params[i]) for i, v in enumerate(val_list)]
+        for i_data in idx_list:
+            if i_data.dtype != torch.uint8:
+                raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i_data.dtype}")
+        _need_device(p, "TopKCompressor.batch_decompress")
+        dev = p.device
+        vals = [_f32c(v.to(dev)) for v in val_list]
+        idxs = [i.to(dev).reshape(-1).contiguous() for i in idx_list]
+        xshape = tuple(xshape)
+        k = vals[0].shape[-1]
+        scale = None
+        if clip_norm and not normalise:
+            scale = _peer_scales(vals, block_norms, dev)
+        chunked = len(xshape) > 2 and xshape[2] == _CH and xshape[3] == _CH and k % 2 == 0 and \
+            all(v.shape[-1] == k and v.numel() == xshape[0] * xshape[1] * k for v in vals)
+        if chunked:
+            if defer:
+                return LazyAggregate(idxs, vals, scale, xshape, k, normalise, p.dtype)
+            out = _aggregate_chunks(idxs, vals, scale, xshape[0], xshape[1], k, normalise=normalise, use_dct=False)
+            return out if p.dtype == torch.float32 else out.to(p.dtype)
+        # generic layout (1-D tensors, un-chunked rows): unpack, scale, concatenate in peer order
+        # (reference :559-575), then one row scatter
+        n_rows, row_len = _row_layout(xshape)
+        parts_i, parts_v = [], []
+        for pi, (i_data, v) in enumerate(zip(idxs, vals)):
+            v2 = v.reshape(-1, v.shape[-1])
+            if normalise:
+                v2 = v2 / (torch.linalg.vector_norm(v2, dim=1, keepdim=True) + 1e-8)
+            elif scale is not None:
+                v2 = v2 * scale[pi]
+            parts_i.append(unpack_12bit_indices(i_data, v2.shape))
+            parts_v.append(v2)
+        cat_i = torch.cat(parts_i, dim=1).contiguous()
+        cat_v = torch.cat(parts_v, dim=1).contiguous()
+        out = _scatter_rows(cat_i, cat_v, n_rows, cat_v.shape[1], row_len).reshape(xshape)
+        return out if p.dtype == torch.float32 else out.to(p.dtype)
+
+    # -- statistical 8-bit quantiser (reference :582-696); payload-sized torch ops ----------
+    @torch.no_grad()
+    def _quantize_values(self, val: torch.Tensor) -> tuple[torch.Tensor, QuantParamsT]:
+        half = self.n_bins // 2
+        shift = val.mean()
+        centred = val - shift
+        scale = self.range_in_sigmas * (centred.norm() / math.sqrt(centred.numel() - 1)) / self.n_bins
+        if scale == 0 or torch.isnan(scale) or torch.isinf(scale):
+            scale = torch.tensor(1.0, dtype=centred.dtype, device=val.device)
+        c32 = centred.to(torch.float32)
+        q = (c32 / scale + half).round().clamp(0, self.n_bins - 1).to(torch.uint8)
+        bins = q.flatten().long()
+        sums = torch.zeros(self.n_bins, dtype=torch.float32, device=q.device).scatter_add_(0, bins, c32.flatten())
+        counts = torch.zeros(self.n_bins, dtype=torch.float32, device=q.device).scatter_add_(
+            0, bins, torch.ones_like(c32.flatten()))
+        lookup = torch.where(counts > 0, sums / counts, torch.zeros_like(sums))
+        return q, (shift, float(scale), half, lookup, val.dtype)
+
+    @torch.no_grad()
+    def _dequantize_values(self, val: torch.Tensor, qparams: QuantParamsT) -> torch.Tensor:
+        if val.dtype != torch.uint8:
+            return val
+        shift, _, _, lookup, orig_dtype = qparams
+        if isinstance(lookup, torch.Tensor):
+            lookup = lookup.to(val.device)
+        return (lookup[val.long()] + shift).to(orig_dtype)
+
+    def maybe_dequantize_values(self, vals: list[torch.Tensor], qparams: list[QuantParamsT],
+                                device: torch.device) -> list[torch.Tensor]:
+        """Dequantise a list of per-peer values when all of them are uint8 (reference :646-696)."""
+        if not isinstance(vals, (list, tuple)):
+            vals = [vals]
+        if qparams is None or not all(v.dtype == torch.uint8 for v in vals):
+            return vals
+        if isinstance(qparams, tuple) and len(qparams) == 5 and not all(
+                isinstance(q, (tuple, list)) and len(q) == 5 for q in qparams):
+            qparams = [qparams]  # a single 5-tuple
+        if not isinstance(qparams, list):
+            qparams = [qparams]
+        out: list[torch.Tensor] = []
+        for i, v in enumerate(vals):
+            v = v.to(device)
+            if v.dtype == torch.uint8:
+                if qparams[i] is None:
+                    import logging
+                    logging.getLogger("templar").warning(f"Missing quant_params for vals[{i}]]; skip.")
+                    break
+                v = self._dequantize_values(v, qparams[i]).to(device)
+            out.append(v)
+        if len(out) != len(vals):
+            raise IndexError(f"Mismatch in val lengths: dequant({len(out)}) vs original({len(vals)})")
+        return out
+
+
+# ----------------------------------------------------------------------------------------
+# fused entry points (what the callers' back-to-back calls amount to)
+# ----------------------------------------------------------------------------------------
+@torch.no_grad()
+def encode_compress(x: torch.Tensor, topk: int, *, use_dct: bool = True):
+    """encode(x, use_dct) followed by compress(., topk) for a 2-D fp32 tensor whose dimensions
+    are multiples of 64 (src/tplr/neurons.py:155-159), in one kernel: the 2-D DCT of every
+    64x64 chunk stays in registers and only indices and values are written.
+    Returns (packed idx, values (Y, X, k), xshape (Y, X, 64, 64), totalk 4096)."""
+    _need_device(x, "encode_compress")
+    if x.dim() != 2 or x.shape[0] % _CH or x.shape[1] % _CH:
+        raise ValueError(f"encode_compress needs a 2-D tensor with dimensions divisible by {_CH}, got {tuple(x.shape)}")
+    R, Cc = x.shape
+    k = max(min(topk, _CH * _CH), 2)
+    k -= k % 2
+    xin = x if (x.dtype == torch.float32 and x.stride(1) == 1 and x.stride(0) >= Cc) else _f32c(x)
+    idx, val = _encode_topk(xin, R, Cc, xin.stride(0), k, use_dct)
+    return idx, val, (R // _CH, Cc // _CH, _CH, _CH), _CH * _CH
+
+
+@torch.no_grad()
+def batch_decompress_decode(idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], xshape: ShapeT, *,
+                            block_norms: torch.Tensor | None = None, normalise: bool = False,
+                            clip_norm: bool = True, use_dct: bool = True, mean: bool = True,
+                            out: torch.Tensor | None = None, sumsq: torch.Tensor | None = None) -> torch.Tensor:
+    """batch_decompress(...) followed by decode(., use_dct) (src/tplr/neurons.py:355-367) in one
+    kernel per tensor: unpack, clip, scatter-mean over the peers and inverse DCT per chunk in
+    LDS; the per-peer dense tensors and the dense coefficient tensor never exist in memory.
+    `mean=False` gives the plain sum; `sumsq` (n_chunks floats) receives per-chunk sums of
+    squares of the result for callers that normalise it."""
+    xshape = tuple(xshape)
+    if len(xshape) != 4 or xshape[2] != _CH or xshape[3] != _CH:
+        raise ValueError(f"batch_decompress_decode needs xshape (Y, X, {_CH}, {_CH}), got {xshape}")
+    for i in idxs:
+        if i.dtype != torch.uint8:
+            raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
+    dev = vals[0].device
+    _need_device(vals[0], "batch_decompress_decode")
+    vals = [_f32c(v.to(dev)) for v in vals]
+    idxs = [i.to(dev).reshape(-1).contiguous() for i in idxs]
+    scale = None
+    if clip_norm and not normalise:
+        scale = _peer_scales(vals, block_norms, dev)
+    return _aggregate_chunks(idxs, vals, scale, xshape[0], xshape[1], vals[0].shape[-1], normalise=normalise,
+                             use_dct=use_dct, mean=mean, out=out, sumsq=sumsq)
+
+
+# the names BASELINE.json's north star uses (DeMo-era)
+TransformDCT = ChunkingTransformer
+CompressDCT = TopKCompressor
+
+__all__ = [
+    "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
+    "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "ShapeT", "Shape4D", "TotK",
+    "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
+]

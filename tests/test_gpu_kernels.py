@@ -1,0 +1,415 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU oracle.  Needs an MI355X.
+
+Bars: bit-exact for packed bytes, index sets/order and gathered values on identical
+coefficient inputs, and for scattered sums/means given identical clip factors; transforms
+and reconstructions within 1e-5 of the tensor's largest magnitude (fp32 tolerance).
+"""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import codec as orc  # noqa: E402  (the checker)
+import templar_amd.compress as tc  # noqa: E402
+from templar_amd import _lib  # noqa: E402
+import workloads  # noqa: E402
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+TOL = 1e-5
+
+
+def t3(shape, seed, row_scale=False):
+    return workloads.student_t3(shape, seed, row_scale=row_scale)
+
+
+def relerr(a, b):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+# ---------------------------------------------------------------- pack / unpack
+def test_pack_unpack_reference_vectors(dev):
+    kats = json.load(open(os.path.join(GOLD, "reference_kats.json")))
+    for case in kats["pack_roundtrip"]:
+        idx = torch.tensor(case["indices"], dtype=torch.int64, device=dev)
+        packed = tc.pack_12bit_indices(idx)
+        assert packed.dtype == torch.uint8 and packed.device == idx.device
+        assert packed.numel() == case["packed_len"]
+        assert np.array_equal(packed.cpu().numpy(), orc.pack12(case["indices"]))
+        back = tc.unpack_12bit_indices(packed, idx.shape)
+        assert back.dtype == torch.int64 and torch.equal(back, idx)
+
+
+@pytest.mark.parametrize("n", [2, 6, 8, 10, 100, 4098, 1 << 20])
+def test_pack_unpack_random(dev, n):
+    g = torch.Generator().manual_seed(n)
+    idx = torch.randint(0, 4096, (n,), generator=g, dtype=torch.int64)
+    packed = tc.pack_12bit_indices(idx.to(dev))
+    assert np.array_equal(packed.cpu().numpy(), orc.pack12(idx.numpy()))
+    assert torch.equal(tc.unpack_12bit_indices(packed, (n,)).cpu(), idx)
+    # a view that starts at an odd byte offset
+    buf = torch.zeros(packed.numel() + 1, dtype=torch.uint8, device=dev)
+    buf[1:] = packed
+    assert torch.equal(tc.unpack_12bit_indices(buf[1:], (n // 2, 2)).cpu().reshape(-1), idx)
+
+
+def test_pack_errors(dev):
+    with pytest.raises(ValueError, match="Number of indices must be even"):
+        tc.pack_12bit_indices(torch.tensor([1, 2, 3], device=dev))
+    with pytest.raises(ValueError, match="exceeds 12-bit limit"):
+        tc.pack_12bit_indices(torch.tensor([0, 4096], device=dev))
+    with pytest.raises(ValueError, match="Index 70000 exceeds"):
+        tc.pack_12bit_indices(torch.tensor([5, 1, 70000, 3], device=dev))
+    with pytest.raises(ValueError, match="Number of indices must be even"):
+        tc.unpack_12bit_indices(torch.zeros(6, dtype=torch.uint8, device=dev), (3,))
+    e = tc.pack_12bit_indices(torch.tensor([], dtype=torch.int64, device=dev))
+    assert e.numel() == 0 and tc.unpack_12bit_indices(e, (0,)).numel() == 0
+
+
+# ---------------------------------------------------------------- transforms
+def test_dct2d_fixture(dev):
+    z = np.load(os.path.join(GOLD, "codec_small.npz"))
+    x = torch.from_numpy(z["x"]).to(dev)
+    tr = tc.ChunkingTransformer(_Stub([x]), 64)
+    coef = tr.encode(x, use_dct=True)
+    assert coef.shape == (2, 3, 64, 64)
+    assert relerr(coef.cpu().numpy(), z["coef"]) <= TOL
+    back = tr.decode(coef, use_dct=True)
+    assert back.shape == x.shape and relerr(back.cpu().numpy(), z["x"]) <= TOL
+    dec = tr.decode(torch.from_numpy(z["coef"]).to(dev), use_dct=True)
+    assert relerr(dec.cpu().numpy(), orc.decode2d(z["coef"])) <= TOL
+
+
+class _Stub:
+    """Anything with named_parameters() works as the `model` argument."""
+
+    def __init__(self, tensors):
+        self.t = tensors
+
+    def named_parameters(self):
+        from types import SimpleNamespace
+
+        for i, t in enumerate(self.t):
+            yield f"p{i}", SimpleNamespace(requires_grad=True, shape=t.shape, dtype=t.dtype, device=t.device)
+
+
+@pytest.mark.parametrize("shape", [(64, 64), (192, 64), (64, 448), (512, 1024)])
+def test_dct2d_random_and_strided(dev, shape):
+    x = t3(shape, 11 + shape[0], row_scale=True)
+    want = orc.encode2d(x.numpy())
+    lib = _lib.load()
+    xd = x.to(dev)
+    R, Cc = shape
+    out = torch.empty(want.shape, dtype=torch.float32, device=dev)
+    st = lib.tplr_dct2d_fwd(tc._ptr(xd), R, Cc, Cc, tc._ptr(out), None)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert relerr(out.cpu().numpy(), want) <= TOL
+    # input living inside a wider buffer (row stride > C)
+    wide = torch.zeros(R, Cc + 64, device=dev)
+    wide[:, 32:32 + Cc] = xd
+    sub = wide[:, 32:32 + Cc]
+    out2 = torch.empty_like(out)
+    assert lib.tplr_dct2d_fwd(tc._ptr(sub), R, Cc, sub.stride(0), tc._ptr(out2), None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    # inverse of the oracle's coefficients
+    back = torch.empty(R, Cc, device=dev)
+    assert lib.tplr_dct2d_inv(tc._ptr(torch.from_numpy(want).to(dev)), R, Cc, tc._ptr(back), Cc, None) == 0
+    torch.cuda.synchronize()
+    assert relerr(back.cpu().numpy(), x.numpy()) <= TOL
+
+
+def test_dct1d_and_dense_chunks(dev):
+    v = t3((2048,), 5)
+    p2 = torch.randn(20, 30)
+    tr = tc.ChunkingTransformer(_Stub([v.clone(), p2.clone(), torch.randn(100)]), 64)
+    assert tr.shape_dict[2048] == 64 and tr.shape_dict[20] == 20 and tr.shape_dict[30] == 30 and tr.shape_dict[100] == 50
+    e = tr.encode(v.to(dev), use_dct=True)
+    assert e.shape == (32, 64)
+    assert relerr(e.cpu().numpy(), orc.dct1d(v.numpy().reshape(32, 64))) <= TOL
+    d = tr.decode(e, use_dct=True)
+    assert d.shape == (2048,) and relerr(d.cpu().numpy(), v.numpy()) <= TOL
+    # odd row count through the 1-D kernel (tail of a 64-vector group)
+    lib = _lib.load()
+    rows = torch.randn(70, 64)
+    out = torch.empty(70, 64, device=dev)
+    assert lib.tplr_dct1d(tc._ptr(rows.to(dev)), 70, 0, tc._ptr(out), None) == 0
+    torch.cuda.synchronize()
+    assert relerr(out.cpu().numpy(), orc.dct1d(rows.numpy())) <= TOL
+    # chunk sizes other than 64 take the dense kernel
+    e2 = tr.encode(p2.to(dev), use_dct=True)
+    assert e2.shape == (1, 1, 20, 30)
+    assert relerr(e2.cpu().numpy(), orc.encode2d(p2.numpy(), 20, 30)) <= TOL
+    assert relerr(tr.decode(e2, use_dct=True).cpu().numpy(), p2.numpy()) <= TOL
+    w = torch.randn(100)
+    e3 = tr.encode(w.to(dev), use_dct=True)
+    assert e3.shape == (2, 50) and relerr(e3.cpu().numpy(), orc.dct1d(w.numpy().reshape(2, 50))) <= TOL
+    assert relerr(tr.decode(e3, use_dct=True).cpu().numpy(), w.numpy()) <= TOL
+
+
+# ---------------------------------------------------------------- top-k on identical coefficients
+def check_topk(rows_np, k, dev):
+    rows = torch.from_numpy(rows_np).to(dev)
+    idx12, val = tc._topk_rows(rows, k)
+    torch.cuda.synchronize()
+    want_i, want_v = orc.topk_rows(rows_np, k)
+    got_i = orc.unpack12(idx12.cpu().numpy(), want_i.shape)
+    assert np.array_equal(got_i, want_i)
+    assert np.array_equal(idx12.cpu().numpy(), orc.pack12(want_i))
+    assert np.array_equal(val.cpu().numpy().view(np.uint32), want_v.view(np.uint32))
+
+
+def test_topk_fixture_bit_exact(dev):
+    z = np.load(os.path.join(GOLD, "codec_small.npz"))
+    idx12, val = tc._topk_rows(torch.from_numpy(z["coef"]).to(dev).reshape(-1, 4096), 32)
+    assert np.array_equal(idx12.cpu().numpy(), z["idx12"])
+    assert np.array_equal(val.cpu().numpy().reshape(z["val"].shape), z["val"])
+
+
+@pytest.mark.parametrize("k", [2, 16, 32, 34, 64, 100, 128])
+def test_topk_chunks_bit_exact(dev, k):
+    rows = t3((48, 4096), 1000 + k).numpy()
+    check_topk(rows, k, dev)
+
+
+def test_topk_skewed_chunks(dev):
+    # energy concentrated in a few tile rows: the per-lane bound is loose, the exact search runs
+    rows = t3((16, 4096), 77).numpy().reshape(16, 64, 64)
+    rows[:, :3, :] *= 1e4
+    rows[5] = 0.0
+    rows[6] = 1.5  # one value everywhere: all ties
+    rows[7, 10:, :] = 0.0
+    check_topk(rows.reshape(16, 4096), 32, dev)
+    check_topk(rows.reshape(16, 4096), 64, dev)
+
+
+def test_topk_special_values(dev):
+    rows = np.zeros((6, 4096), np.float32)
+    rows[1, [5, 900, 17]] = [2.0, -2.0, 2.0]
+    rows[1, 100] = np.nan
+    rows[1, 4000] = -np.inf
+    rows[1, 7] = -0.0
+    rows[2] = np.float32(1e-42)  # denormals everywhere
+    rows[2, 4095] = np.float32(3e-42)
+    rows[3, :] = np.nan
+    rows[4, ::2] = 1.0
+    rows[4, 1::2] = -1.0
+    rows[5] = np.linspace(-1, 1, 4096, dtype=np.float32)
+    for k in (2, 32, 64):
+        rows_d = torch.from_numpy(rows).to(dev)
+        idx12, val = tc._topk_rows(rows_d, k)
+        want_i, want_v = orc.topk_rows(rows, k)
+        got_i = orc.unpack12(idx12.cpu().numpy(), want_i.shape)
+        assert np.array_equal(got_i, want_i)
+        assert np.array_equal(val.cpu().numpy().view(np.uint32), want_v.view(np.uint32))
+
+
+@pytest.mark.parametrize("n,k", [(64, 32), (64, 64), (100, 10), (37, 6), (4095, 32), (2048, 128), (2, 2)])
+def test_topk_generic_rows(dev, n, k):
+    rows = t3((9, n), n * 7 + k).numpy()
+    rows[3] = 0.0
+    check_topk(rows, k, dev)
+
+
+# ---------------------------------------------------------------- fused encode
+@pytest.mark.parametrize("shape,k", [((128, 192), 32), ((64, 64), 64), ((256, 128), 2), ((192, 320), 128)])
+def test_fused_encode_equals_unfused(dev, shape, k):
+    x = t3(shape, 31 + k, row_scale=True).to(dev)
+    idx_f, val_f, xshape, totalk = tc.encode_compress(x, k, use_dct=True)
+    tr = tc.ChunkingTransformer(_Stub([x]), 64)
+    coef = tr.encode(x, use_dct=True)
+    idx_u, val_u, xshape_u, totalk_u = tc.TopKCompressor().compress(coef, k)
+    assert tuple(xshape) == tuple(xshape_u) and totalk == totalk_u == 4096
+    assert torch.equal(idx_f, idx_u) and torch.equal(val_f, val_u)
+    # selection on the device's own coefficients is exactly the oracle's selection
+    want_i, want_v = orc.topk_rows(coef.cpu().numpy().reshape(-1, 4096), k)
+    assert np.array_equal(idx_f.cpu().numpy(), orc.pack12(want_i))
+    assert np.array_equal(val_f.cpu().numpy().reshape(-1, k), want_v)
+
+
+def near_tie_audit(x_np, idx12, val, k, tol=TOL):
+    """End-to-end check against the oracle's own transform: every selected value within
+    tolerance, and any chunk whose index set differs differs only in entries whose
+    magnitudes are within tolerance of the k-th largest."""
+    coef = orc.encode2d(x_np).reshape(-1, 4096)
+    want_i, want_v = orc.topk_rows(coef, k)
+    got_i = orc.unpack12(idx12, want_i.shape)
+    scale = np.abs(coef).max()
+    differing = 0
+    for r in range(coef.shape[0]):
+        a, b = set(got_i[r].tolist()), set(want_i[r].tolist())
+        assert len(a) == k
+        if a != b:
+            differing += 1
+            kth = np.abs(want_v[r]).min()
+            for i in a ^ b:
+                assert abs(abs(coef[r, i]) - kth) <= 4 * tol * scale, (r, i)
+        got = val.reshape(-1, k)[r]
+        assert np.abs(got - coef[r, got_i[r]]).max() <= tol * scale
+    return differing, coef.shape[0]
+
+
+def test_fused_encode_end_to_end_tolerance(dev):
+    x = t3((512, 768), 4242, row_scale=True)
+    idx12, val, _, _ = tc.encode_compress(x.to(dev), 32)
+    diff, n = near_tie_audit(x.numpy(), idx12.cpu().numpy(), val.cpu().numpy(), 32)
+    assert diff <= max(1, n // 20)
+
+
+def test_no_dct_view_path(dev):
+    # encode(use_dct=False) is a view; compress() then selects straight from the dense tensor
+    x = t3((128, 256), 9).to(dev)
+    tr = tc.ChunkingTransformer(_Stub([x]), 64)
+    enc = tr.encode(x, use_dct=False)
+    assert enc.data_ptr() == x.data_ptr() and enc.shape == (2, 4, 64, 64)
+    idx12, val, xshape, totalk = tc.TopKCompressor().compress(enc, 32)
+    want_i, want_v = orc.topk_rows(orc.encode2d(x.cpu().numpy(), use_dct=False).reshape(-1, 4096), 32)
+    assert np.array_equal(idx12.cpu().numpy(), orc.pack12(want_i))
+    assert np.array_equal(val.cpu().numpy().reshape(-1, 32), want_v)
+    assert tuple(xshape) == (2, 4, 64, 64) and totalk == 4096
+    dec = tr.decode(tc.TopKCompressor().decompress(x, idx12, val, xshape, totalk), use_dct=False)
+    assert dec.shape == x.shape
+    assert np.array_equal(dec.cpu().numpy(), orc.decode2d(orc.decompress(idx12.cpu().numpy(), val.cpu().numpy(),
+                                                                         xshape, totalk), use_dct=False))
+
+
+# ---------------------------------------------------------------- decode-aggregate
+def make_peers(P, Y, X, k, seed):
+    rng = np.random.default_rng(seed)
+    shared = rng.standard_normal((Y, X, 4096)).astype(np.float32)
+    idxs, vals = [], []
+    for p in range(P):
+        g = (0.5 * shared + rng.standard_normal((Y, X, 4096)) * (1 + 0.3 * p)).astype(np.float32) * 1e-3
+        i, v = orc.topk_rows(g, k)
+        idxs.append(orc.pack12(i))
+        vals.append(v)
+    return idxs, vals
+
+
+@pytest.mark.parametrize("P,k", [(1, 32), (2, 32), (15, 32), (15, 64), (3, 2), (5, 128), (7, 20), (128, 4)])
+def test_aggregate_dense_bit_exact(dev, P, k):
+    Y, X = 2, 3
+    idxs, vals = make_peers(P, Y, X, k, 100 * P + k)
+    norms = np.array([orc.norm2(v) for v in vals], np.float32)
+    want = orc.batch_decompress(idxs, vals, (Y, X, 64, 64), 4096, block_norms=norms)
+    comp = tc.TopKCompressor()
+    p = torch.empty(Y * 64, X * 64, device=dev)
+    got = comp.batch_decompress(p, [torch.from_numpy(i).to(dev) for i in idxs], [torch.from_numpy(v).to(dev) for v in vals],
+                                (Y, X, 64, 64), 4096, block_norms=torch.from_numpy(norms).to(dev))
+    assert got.shape == (Y, X, 64, 64)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    # norms computed on the device: same result to rounding of the clip factors
+    got2 = comp.batch_decompress(p, [torch.from_numpy(i).to(dev) for i in idxs],
+                                 [torch.from_numpy(v).to(dev) for v in vals], (Y, X, 64, 64), 4096)
+    assert relerr(got2.cpu().numpy(), want) <= 1e-6
+    # no clipping, plain sum
+    want_sum = orc.batch_decompress(idxs, vals, (Y, X, 64, 64), 4096, clip_norm=False, mean=False)
+    got_sum = tc._aggregate_chunks([torch.from_numpy(i).to(dev) for i in idxs], [torch.from_numpy(v).to(dev) for v in vals],
+                                   None, Y, X, k, normalise=False, use_dct=False, mean=False)
+    assert np.array_equal(got_sum.cpu().numpy(), want_sum)
+
+
+def test_aggregate_normalise(dev):
+    P, k, Y, X = 4, 32, 2, 2
+    idxs, vals = make_peers(P, Y, X, k, 5)
+    want = orc.batch_decompress(idxs, vals, (Y, X, 64, 64), 4096, normalise=True)
+    got = tc.TopKCompressor().batch_decompress(torch.empty(1, device=dev), [torch.from_numpy(i).to(dev) for i in idxs],
+                                               [torch.from_numpy(v).to(dev) for v in vals], (Y, X, 64, 64), 4096,
+                                               normalise=True)
+    assert relerr(got.cpu().numpy(), want) <= 1e-6
+    assert np.array_equal(got.cpu().numpy() != 0, want != 0)
+
+
+@pytest.mark.parametrize("P,k", [(1, 32), (15, 32), (15, 64)])
+def test_aggregate_fused_with_inverse_dct(dev, P, k):
+    Y, X = 3, 2
+    idxs, vals = make_peers(P, Y, X, k, 9 * P + k)
+    norms = np.array([orc.norm2(v) for v in vals], np.float32)
+    want = orc.decode2d(orc.batch_decompress(idxs, vals, (Y, X, 64, 64), 4096, block_norms=norms))
+    di = [torch.from_numpy(i).to(dev) for i in idxs]
+    dv = [torch.from_numpy(v).to(dev) for v in vals]
+    ss = torch.zeros(Y * X, device=dev)
+    got = tc.batch_decompress_decode(di, dv, (Y, X, 64, 64), block_norms=torch.from_numpy(norms).to(dev), sumsq=ss)
+    assert got.shape == (Y * 64, X * 64)
+    assert relerr(got.cpu().numpy(), want) <= TOL
+    per_chunk = (want.reshape(Y, 64, X, 64).astype(np.float64) ** 2).sum((1, 3)).reshape(-1)
+    assert np.allclose(ss.cpu().numpy(), per_chunk, rtol=1e-4)
+    # the two-call form through the reference API gives the same tensor
+    comp, tr = tc.TopKCompressor(), tc.ChunkingTransformer(_Stub([torch.empty(Y * 64, X * 64)]), 64)
+    lazy = comp.batch_decompress(torch.empty(1, device=dev), di, dv, (Y, X, 64, 64), 4096,
+                                 block_norms=torch.from_numpy(norms).to(dev), defer=True)
+    assert torch.equal(tr.decode(lazy, use_dct=True), got)
+    dense = comp.batch_decompress(torch.empty(1, device=dev), di, dv, (Y, X, 64, 64), 4096,
+                                  block_norms=torch.from_numpy(norms).to(dev))
+    assert relerr(tr.decode(dense, use_dct=True).cpu().numpy(), want) <= TOL
+
+
+def test_scatter_rows_generic(dev):
+    rng = np.random.default_rng(8)
+    comp = tc.TopKCompressor()
+    # 1-D tensor layout (x, w) = (32, 64), packed
+    v = rng.standard_normal((32, 64)).astype(np.float32)
+    i, vv = orc.topk_rows(v, 32)
+    got = comp.decompress(torch.empty(1, device=dev), torch.from_numpy(orc.pack12(i)).to(dev), torch.from_numpy(vv).to(dev),
+                          (32, 64), 64)
+    assert np.array_equal(got.cpu().numpy(), orc.scatter_rows(i, vv, 64))
+    # unpacked int64 indices with many duplicates: exact source-order sums
+    idx = rng.integers(0, 50, size=(7, 300))
+    val = (rng.standard_normal((7, 300)) * 10.0 ** rng.integers(-3, 4, size=(7, 300))).astype(np.float32)
+    got = comp.decompress(torch.empty(1, device=dev), torch.from_numpy(idx).to(dev), torch.from_numpy(val).to(dev),
+                          (7, 100), 100)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), orc.scatter_rows(idx, val, 100).view(np.uint32))
+    with pytest.raises(RuntimeError, match="out of bounds"):
+        comp.decompress(torch.empty(1, device=dev), torch.tensor([[3, 100]], device=dev), torch.ones(1, 2, device=dev),
+                        (1, 100), 100)
+    # batch form on a non-chunk layout
+    P = 3
+    payload = []
+    for p in range(P):
+        g = rng.standard_normal((32, 64)).astype(np.float32)
+        ii, gv = orc.topk_rows(g, 32)
+        payload.append((orc.pack12(ii), gv))
+    norms = np.array([orc.norm2(v_) for _, v_ in payload], np.float32)
+    want = orc.batch_decompress([a for a, _ in payload], [b for _, b in payload], (32, 64), 64, block_norms=norms)
+    got = comp.batch_decompress(torch.empty(1, device=dev), [torch.from_numpy(a).to(dev) for a, _ in payload],
+                                [torch.from_numpy(b).to(dev) for _, b in payload], (32, 64), 64,
+                                block_norms=torch.from_numpy(norms).to(dev))
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+def test_clip_scales_and_norms(dev):
+    lib = _lib.load()
+    for norms in ([3.0, 1.0, 2.0, 10.0], [5.0], [2.0, 8.0], [1.0, 1.0, 4.0, 0.0, 9.0], list(np.linspace(0.1, 7, 128))):
+        n = torch.tensor(norms, dtype=torch.float32, device=dev)
+        s = torch.empty_like(n)
+        m = torch.empty(1, device=dev)
+        assert lib.tplr_clip_scales(tc._ptr(n), len(norms), 0, tc._ptr(s), tc._ptr(m), None) == 0
+        med, want = orc.clip_scales(np.array(norms, np.float32))
+        assert m.item() == np.float32(med) and np.array_equal(s.cpu().numpy(), want)
+    vals = [torch.randn(1000 + 0 * p, device=dev) * (p + 1) for p in range(5)]
+    ss = torch.empty(5, device=dev)
+    ptrs = (C.c_void_p * 5)(*[v.data_ptr() for v in vals])
+    assert lib.tplr_peer_sumsq(ptrs, 5, 1000, tc._ptr(ss), None) == 0
+    want = np.array([float((v.double() ** 2).sum()) for v in vals])
+    assert np.allclose(ss.cpu().numpy(), want, rtol=1e-5)
+
+
+def test_bad_arguments_are_rejected(dev):
+    lib = _lib.load()
+    x = torch.zeros(64, 64, device=dev)
+    o = torch.zeros(4096, device=dev)
+    b = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    assert lib.tplr_dct2d_fwd(tc._ptr(x), 64, 65, 65, tc._ptr(o), None) == _lib.TPLR_E_SHAPE
+    assert lib.tplr_dct2d_fwd(None, 64, 64, 64, tc._ptr(o), None) == _lib.TPLR_E_BADARG
+    assert lib.tplr_topk_pack(tc._ptr(o), 1, 4096, 33, tc._ptr(b), tc._ptr(o), None) == _lib.TPLR_E_BADARG
+    assert lib.tplr_topk_pack(tc._ptr(o), 1, 5000, 32, tc._ptr(b), tc._ptr(o), None) == _lib.TPLR_E_TOOMANY
+    assert lib.tplr_pack12(tc._ptr(o), 3, tc._ptr(b), None, None) == _lib.TPLR_E_ODD
+    assert lib.tplr_encode_topk_pack(tc._ptr(x), 64, 64, 32, 32, 1, tc._ptr(b), tc._ptr(o), None) == _lib.TPLR_E_BADARG
+    assert b"even" in lib.tplr_status_string(_lib.TPLR_E_ODD)

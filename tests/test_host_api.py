@@ -1,0 +1,197 @@
+"""Host-side logic of templar_amd that needs no GPU: the C ABI's symbol table, the helper
+functions the reference's tests import, argument validation and error text, the host-memory
+pack/unpack entry points, and the zero-copy chunk view."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import templar_amd
+import templar_amd.compress as tc
+from templar_amd import _lib
+from oracle import codec as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+KATS = json.load(open(os.path.join(ROOT, "tests", "golden", "reference_kats.json")))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "tplr_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b(tplr_[a-z0-9_]+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    names = header_functions()
+    assert len(names) >= 15 and len(set(names)) == len(names)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert set(names) == set(_lib.SIGNATURES), "ctypes table and header disagree"
+    assert _lib.load().tplr_version() >= 100
+    assert _lib.load().tplr_status_string(0) == b"ok"
+
+
+def test_api_surface_matches_reference_module():
+    for name in ["pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "_dct", "_idct",
+                 "_get_smaller_split", "_get_divisors", "_get_prime_divisors", "TransformDCT", "CompressDCT",
+                 "ShapeT", "Shape4D", "TotK", "IdxT", "ValT", "QuantParamsT"]:
+        assert hasattr(tc, name), name
+    assert tc.TransformDCT is tc.ChunkingTransformer and tc.CompressDCT is tc.TopKCompressor
+    c = tc.TopKCompressor(use_quantization=True, quantization_bins=4, quantization_range=6)
+    assert c.use_quantization and c.n_bins == 4 and c.range_in_sigmas == 6
+    for m in ["compress", "decompress", "batch_decompress", "_quantize_values", "_dequantize_values",
+              "maybe_dequantize_values", "_clamp_topk"]:
+        assert callable(getattr(c, m))
+    assert templar_amd.compress is tc
+
+
+@pytest.mark.parametrize("n,c,want", [tuple(x) for x in KATS["smaller_split"]])
+def test_smaller_split_reference_vectors(n, c, want):
+    assert tc._get_smaller_split(n, c) == want
+
+
+def test_divisor_helpers_against_oracle():
+    for n in list(range(1, 300)) + [768, 2048, 3072, 8192, 29568, 32000]:
+        assert tc._get_divisors(n) == orc.divisors(n)
+        prod = 1
+        for p in tc._get_prime_divisors(n):
+            prod *= p
+            assert all(p % q for q in range(2, int(p ** 0.5) + 1))
+        assert prod == n
+        for c in (1, 7, 16, 64, 100):
+            assert tc._get_smaller_split(n, c) == orc.smaller_split(n, c)
+    assert tc._get_divisors(0) == []
+
+
+def test_dct_helpers():
+    x = torch.randn(4, 8)
+    X = tc._dct(x, norm="ortho")
+    assert torch.allclose(tc._idct(X, norm="ortho"), x, atol=1e-6)  # tests/unit/test_compress.py:281-290
+    assert np.allclose(tc._dct(torch.eye(64), norm="ortho").numpy(), orc.dct_basis(64), atol=1e-7)
+    assert np.allclose(tc._idct(torch.eye(64), norm="ortho").numpy(), orc.dct_basis(64).T, atol=1e-7)
+    # un-normalised convention of torch-dct: X_k = 2 sum x_n cos(pi (2n+1) k / 2N)
+    e = torch.zeros(1, 8)
+    e[0, 0] = 1.0
+    assert torch.allclose(tc._dct(e)[0], 2 * torch.cos(torch.arange(8) * torch.pi / 16), atol=1e-6)
+    assert torch.allclose(tc._idct(tc._dct(x)), x, atol=1e-5)
+
+
+class _Model:
+    def __init__(self, shapes, dtype=torch.float32):
+        self.params = [torch.nn.Parameter(torch.zeros(s, dtype=dtype)) for s in shapes]
+        self.params.append(torch.nn.Parameter(torch.zeros(7, 7), requires_grad=False))
+
+    def named_parameters(self):
+        return [(f"w{i}", p) for i, p in enumerate(self.params)]
+
+
+def test_chunking_transformer_tables():
+    tr = tc.ChunkingTransformer(_Model([(64, 32), (128, 64), (128,), (100, 30)]), 16)
+    assert tr.target_chunk == 16
+    assert tr.shape_dict == {64: 16, 32: 16, 128: 16, 100: 10, 30: 15}
+    assert 7 not in tr.shape_dict  # frozen parameters are skipped
+    assert set(tr.f_dict) == {16, 10, 15} == set(tr.b_dict)
+    for n in tr.f_dict:
+        assert np.allclose(tr.f_dict[n].numpy(), orc.dct_basis(n), atol=1e-6)
+        assert np.allclose(tr.b_dict[n].numpy(), orc.dct_basis(n).T, atol=1e-6)
+    tr16 = tc.ChunkingTransformer(_Model([(64, 64)], dtype=torch.bfloat16), 64)
+    assert tr16.f_dict[64].dtype == torch.bfloat16
+
+
+def test_encode_decode_without_dct_is_a_view():
+    tr = tc.ChunkingTransformer(_Model([(32, 64), (64,)]), 8)
+    x = torch.arange(32 * 64, dtype=torch.float32).reshape(32, 64)
+    e = tr.encode(x, use_dct=False)
+    assert e.shape == (4, 8, 8, 8) and e.data_ptr() == x.data_ptr()
+    assert np.array_equal(e.numpy(), orc.encode2d(x.numpy(), 8, 8, use_dct=False))
+    assert torch.equal(tr.decode(e, use_dct=False), x)
+    v = torch.arange(64, dtype=torch.float32)
+    ev = tr.encode(v, use_dct=False)
+    assert ev.shape == (8, 8) and torch.equal(tr.decode(ev, use_dct=False), v)
+    with pytest.raises(KeyError):
+        tr.encode(torch.zeros(48, 64), use_dct=False)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        tr.encode(x, use_dct=True)
+
+
+def test_clamp_topk():
+    c = tc.TopKCompressor()
+    for last in (1, 2, 3, 10, 64, 100, 4096):
+        for k in (0, 1, 2, 3, 31, 32, 33, 64, 5000):
+            assert c._clamp_topk(torch.empty(3, last), k) == orc.clamp_topk(last, k)
+
+
+def test_host_pack_unpack_vectors():
+    for case in KATS["pack_roundtrip"]:
+        idx = torch.tensor(case["indices"], dtype=torch.int64)
+        packed = tc.pack_12bit_indices(idx)
+        assert packed.dtype == torch.uint8 and packed.numel() == case["packed_len"]
+        assert np.array_equal(packed.numpy(), orc.pack12(case["indices"]))
+        back = tc.unpack_12bit_indices(packed, idx.shape)
+        assert back.dtype == torch.int64 and torch.equal(back, idx)
+    torch.manual_seed(42)
+    idx = torch.randint(0, 4096, (100,), dtype=torch.int64)
+    packed = tc.pack_12bit_indices(idx)
+    assert packed.numel() == 150 and torch.equal(tc.unpack_12bit_indices(packed, idx.shape), idx)
+    two_d = torch.tensor([[10, 20, 30, 40], [50, 60, 70, 80]])
+    assert torch.equal(tc.unpack_12bit_indices(tc.pack_12bit_indices(two_d), two_d.shape), two_d)
+    assert tc.pack_12bit_indices(torch.arange(1000)).numel() == 1500  # 75 % of int16
+
+
+def test_pack_unpack_errors():
+    with pytest.raises(ValueError, match="Number of indices must be even, got 3"):
+        tc.pack_12bit_indices(torch.tensor([1, 2, 3]))
+    with pytest.raises(ValueError, match=r"Index 4096 exceeds 12-bit limit \(4095\)"):
+        tc.pack_12bit_indices(torch.tensor([0, 4096]))
+    with pytest.raises(ValueError, match="exceeds 12-bit limit"):
+        tc.pack_12bit_indices(torch.tensor([1, 2, 5000]))  # the range check comes first
+    with pytest.raises(ValueError, match="Number of indices must be even, got 3"):
+        tc.unpack_12bit_indices(torch.zeros(6, dtype=torch.uint8), (3,))
+    with pytest.raises(RuntimeError, match="shape mismatch"):
+        tc.unpack_12bit_indices(torch.zeros(5, dtype=torch.uint8), (4,))
+    empty = tc.pack_12bit_indices(torch.tensor([], dtype=torch.int64))
+    assert empty.numel() == 0
+    assert tc.unpack_12bit_indices(empty, (0,)).shape == (0,)
+
+
+def test_decompress_validation_happens_before_any_kernel():
+    c = tc.TopKCompressor()
+    p = torch.zeros(10, 10)
+    with pytest.raises(ValueError, match=r"Expected uint8 \(packed\) or int64 \(unpacked\) indices, got torch.int32"):
+        c.decompress(p, torch.zeros(4, dtype=torch.int32), torch.zeros(2, 2), (10, 10), 10)
+    with pytest.raises(ValueError, match="Expected uint8 for 12-bit packed indices, got torch.int64"):
+        c.batch_decompress(p, [torch.zeros(4, dtype=torch.int64)], [torch.zeros(2, 2)], (10, 10), 10)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        c.compress(torch.randn(10, 10), 4)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        c.decompress(p, torch.zeros(6, dtype=torch.uint8), torch.zeros(2, 2), (10, 10), 10)
+
+
+def test_quantiser_matches_oracle_and_reference_contract():
+    c = tc.TopKCompressor(use_quantization=True, quantization_bins=256, quantization_range=6)
+    g = torch.Generator().manual_seed(3)
+    v = torch.randn(4, 3, 32, generator=g)
+    q, qp = c._quantize_values(v)
+    assert q.dtype == torch.uint8 and len(qp) == 5 and qp[2] == 128 and qp[4] == torch.float32
+    oq, (oshift, oscale, ooff, olook) = orc.quantize(v.numpy(), 256, 6)
+    assert abs(qp[1] - oscale) <= 1e-6 * oscale and abs(float(qp[0]) - oshift) < 1e-7
+    assert (q.numpy() != oq).mean() < 0.01  # rounding of the scale may move a value on a bin edge
+    assert np.allclose(qp[3].numpy(), olook, atol=1e-5)
+    deq = c._dequantize_values(q, qp)
+    assert deq.dtype == torch.float32 and (deq - v).abs().max() <= qp[1]
+    assert c._dequantize_values(v, qp) is v  # not uint8: returned untouched
+    # constant tensor -> scale 1.0
+    _, qp2 = tc.TopKCompressor(use_quantization=True, quantization_bins=4)._quantize_values(torch.full((8,), 0.25))
+    assert qp2[1] == 1.0
+    # list handling of maybe_dequantize_values (reference :646-696)
+    out = c.maybe_dequantize_values([q, q], [qp, qp], torch.device("cpu"))
+    assert len(out) == 2 and torch.equal(out[0], deq)
+    assert c.maybe_dequantize_values([v], [qp], torch.device("cpu"))[0] is v
+    assert torch.equal(c.maybe_dequantize_values([q], qp, torch.device("cpu"))[0], deq)  # a bare 5-tuple
+    with pytest.raises(IndexError, match="Mismatch in val lengths"):
+        c.maybe_dequantize_values([q, q], [qp, None], torch.device("cpu"))
