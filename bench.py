@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""Benchmark of the gradient-codec hot path on one MI355X.
+
+Workload (BASELINE.json configs[2] and configs[3]): the LLaMA-style 1B gradient set
+(16 layers, hidden 2048, intermediate 8192, vocab 32000; 115 two-dimensional tensors =
+294 144 chunks of 64x64, plus 33 norm vectors), synthetic Student-t(df=3) x 1e-3 gradients
+with log-normal row scales, chunk 64, top-k 32.
+
+  step       = one encode + top-k + pack pass over the whole set (fused kernel per tensor)
+  value      = algorithmic bytes of that pass / time, in GB/s (inputs resident in HBM)
+  aggregate  = one 15-peer decode-aggregate pass over the same shapes (clip factors, fused
+               unpack + scatter-mean + inverse DCT per tensor), reported as ms and GB/s
+  roofline   = the same figures against the 8 TB/s HBM peak, per kernel, from HIP events on
+               the launch stream
+  cpu_baseline = the reference's op sequence in torch on the host cores (oracle port), timed
+               on a bounded sample of the same workload
+
+Prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg3_llama1b", help="cfg1_2048x2048 | cfg2_llama150m | cfg3_llama1b | cfg5_72b_block")
+    ap.add_argument("--peers", type=int, default=15)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline sample")
+    return ap.parse_args()
+
+
+def event_ms(fn, steps, warmup):
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_time(stop) / steps, wall
+
+
+def cpu_baseline(workload_name, k, peers, budget_s):
+    """Reference op sequence on torch CPU (oracle/torch_cpu_path.py) on a bounded sample."""
+    import torch
+
+    import workloads
+    from oracle import torch_cpu_path as tcp
+
+    f, b = tcp.basis(64)
+    sample_shapes = [(2048, 2048)] * 2 + [(8192, 2048)] if "cfg1" not in workload_name else [(2048, 2048)]
+    xs = [workloads.student_t3(s, 900 + i, row_scale=True) for i, s in enumerate(sample_shapes)]
+    nbytes = workloads.encode_bytes(sample_shapes, k)
+
+    def enc_pass():
+        return [tcp.compress(tcp.encode(x, 64, 64, f, f), k) for x in xs]
+
+    enc_pass()
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_begin < budget_s / 2 and len(times) < 10):
+        t0 = time.perf_counter()
+        pay = enc_pass()
+        times.append(time.perf_counter() - t0)
+    enc_s = sorted(times)[len(times) // 2]
+
+    # aggregate: `peers` payloads of the first sample tensor
+    x0 = xs[0]
+    ppay = []
+    for p in range(peers):
+        g = 0.5 * x0 + workloads.student_t3(x0.shape, 1000 * (p + 1), row_scale=True)
+        ppay.append(tcp.compress(tcp.encode(g, 64, 64, f, f), k))
+    idxs, vals = [a[0] for a in ppay], [a[1] for a in ppay]
+    xshape, totalk = ppay[0][2], ppay[0][3]
+
+    def agg_pass():
+        norms = torch.stack([torch.norm(v, p=2) for v in vals])
+        return tcp.decode(tcp.batch_decompress(idxs, vals, xshape, totalk, block_norms=norms), b, b)
+
+    agg_pass()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        agg_pass()
+        times.append(time.perf_counter() - t0)
+    agg_s = sorted(times)[1]
+    agg_bytes = workloads.aggregate_bytes([tuple(x0.shape)], k, peers)
+    return {
+        "value": round(nbytes / enc_s / 1e9, 3),
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "host_cpus": os.cpu_count(),
+        "kind": "port",
+        "sample": f"encode+top-k+pack of {[list(s) for s in sample_shapes]} fp32 (k={k}), median of {len(times)}+ runs; "
+                  f"aggregate of {peers} peers on {list(x0.shape)}",
+        "aggregate_GBps": round(agg_bytes / agg_s / 1e9, 3),
+        "encode_sample_s": round(enc_s, 4),
+        "aggregate_sample_s": round(agg_s, 4),
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {args.gpus}); every box in this build has one GPU and the "
+              "path has no collective.  Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import templar_amd.compress as tc
+    import workloads
+
+    dev = torch.device("cuda:0")
+    cfg = workloads.CONFIGS[args.workload]
+    k, shapes = cfg["k"], cfg["shapes"]
+    P = args.peers
+
+    class Shapes:
+        def named_parameters(self):
+            from types import SimpleNamespace
+            for i, s in enumerate(shapes):
+                yield f"p{i}", SimpleNamespace(requires_grad=True, shape=tuple(s), dtype=torch.float32, device=dev)
+
+    tr = tc.ChunkingTransformer(Shapes(), 64)
+    comp = tc.TopKCompressor()
+
+    # ---- inputs resident in HBM
+    grads = workloads.gradient_set(args.workload, device=dev)
+    two_d = [g for g in grads if g.dim() == 2]
+    one_d = [g for g in grads if g.dim() == 1]
+
+    def encode_pass():
+        out = [tc.encode_compress(g, k, use_dct=True) for g in two_d]
+        for g in one_d:
+            out.append(comp.compress(tr.encode(g, use_dct=True), k))
+        return out
+
+    enc_ms, enc_wall = event_ms(encode_pass, args.steps, args.warmup)
+    enc_bytes = workloads.encode_bytes(shapes, k)
+    # kernel-only figure for the fused 2-D kernel (the dominant one)
+    def encode2d_only():
+        for g in two_d:
+            tc.encode_compress(g, k, use_dct=True)
+    enc2d_ms, _ = event_ms(encode2d_only, args.steps, 1)
+    enc2d_bytes = workloads.chunks_2d(shapes) * (16384 + 11 * k // 2)
+
+    # ---- P peers' payloads for the aggregation side (peer p = 0.5 shared + own)
+    payloads = []  # per tensor: (idxs[P], vals[P], xshape)
+    for j, g in enumerate(two_d):
+        idxs, vals = [], []
+        for p in range(P):
+            own = workloads.student_t3(tuple(g.shape), 1000 * (p + 1) + j, row_scale=True, device=dev)
+            own.add_(g, alpha=0.5)
+            i12, v, xshape, _ = tc.encode_compress(own, k, use_dct=True)
+            idxs.append(i12)
+            vals.append(v)
+            del own
+        payloads.append((idxs, vals, xshape))
+    del grads, two_d
+    torch.cuda.empty_cache()
+    outs = [torch.empty(xs[0] * 64, xs[1] * 64, device=dev) for _, _, xs in payloads]
+
+    def aggregate_pass():
+        for (idxs, vals, xshape), out in zip(payloads, outs):
+            tc.batch_decompress_decode(idxs, vals, xshape, clip_norm=True, use_dct=True, out=out)
+
+    agg_ms, agg_wall = event_ms(aggregate_pass, max(3, args.steps // 2), 2)
+    agg_bytes = workloads.chunks_2d(shapes) * (P * 11 * k // 2 + 16384)
+
+    result = {
+        "metric": "encode+topk+pack GB/s and 15-peer decode-aggregate ms, 1B grads, 1 GPU",
+        "value": round(enc_bytes / (enc_ms * 1e-3) / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(enc_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: encode+top-k+pack of {len(shapes)} tensors "
+                               f"({workloads.chunks_2d(shapes)} chunks 64x64, k={k}) and {P}-peer decode-aggregate",
+                   "chunk": 64, "topk": k, "peers": P, "use_dct": True},
+        "encode_wall_ms": round(enc_wall, 4),
+        "aggregate_ms": round(agg_ms, 4),
+        "aggregate_GBps": round(agg_bytes / (agg_ms * 1e-3) / 1e9, 2),
+        "aggregate_wall_ms": round(agg_wall, 4),
+        "roofline": {
+            "bound": "hbm", "kernel": "k_encode_topk_pack",
+            "achieved": round(enc2d_bytes / (enc2d_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(enc2d_bytes / (enc2d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+            "launches_per_step": len(payloads), "bytes_per_step": enc2d_bytes, "ms_per_step": round(enc2d_ms, 4),
+        },
+        "roofline_aggregate": {
+            "bound": "hbm", "kernel": "k_decode_aggregate",
+            "achieved": round(agg_bytes / (agg_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(agg_bytes / (agg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+            "launches_per_step": len(payloads), "bytes_per_step": agg_bytes,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.workload, k, P, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
