@@ -39,6 +39,18 @@ extern "C" {
 #define TPLR_REDUCE_MEAN  0    /* mean over the peers that sent the coefficient (reference) */
 #define TPLR_REDUCE_SUM   1    /* plain sum                                             */
 
+/* One 2-D fp32 tensor of a batch whose dimensions are multiples of 64.  A batch is the
+ * concatenation of its tensors' chunk lists (tensor by tensor, chunks row-major); the
+ * packed payload of a batch is indexed by that global chunk id: chunk g's indices are the
+ * 3k/2 bytes at g*3k/2, its values the k floats at g*k. */
+typedef struct tplr_tensor_desc {
+    void*   dense;        /* the (R, C) tensor: input of encode, output of decode-aggregate */
+    int64_t ld;           /* its row stride in elements                                     */
+    int64_t chunk_begin;  /* id of its first chunk in the batch (running sum of x*y chunks) */
+    int32_t x_chunks;     /* C / 64                                                         */
+    int32_t y_chunks;     /* R / 64                                                         */
+} tplr_tensor_desc;
+
 /* Library / ABI version (major*10000 + minor*100 + patch). */
 int tplr_version(void);
 
@@ -107,6 +119,13 @@ int tplr_topk_pack(const float* d_coef, int64_t n_rows, int64_t row_len, int k,
 int tplr_encode_topk_pack(const float* d_x, int64_t R, int64_t C, int64_t ld_x, int k, int use_dct,
                           uint8_t* d_idx12, float* d_val, void* stream);
 
+/* The same over a whole gradient set in ONE launch (the per-parameter loop of
+ * src/tplr/neurons.py:114-159 without its per-tensor kernel tails): d_desc is a DEVICE
+ * array of n_tensors descriptors sorted by chunk_begin, total_chunks their chunk count;
+ * outputs are the flat payload described at tplr_tensor_desc. */
+int tplr_encode_topk_pack_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, int k,
+                                int use_dct, uint8_t* d_idx12, float* d_val, void* stream);
+
 /* ---- decode side -----------------------------------------------------------------
  * Fused TopKCompressor.batch_decompress + ChunkingTransformer.decode
  * (src/tplr/compress.py:483-580 then :259-292; caller: src/tplr/neurons.py:355-367).
@@ -125,6 +144,16 @@ int tplr_decode_aggregate(const uint8_t* const* h_idx12, const float* const* h_v
                           const float* d_peer_scale, int n_peers, int k,
                           int64_t R, int64_t C, int reduce_mode, int normalise, int use_dct,
                           float* d_out, int64_t ld_out, float* d_sumsq, void* stream);
+
+/* The same over a whole gradient set in ONE launch (the per-parameter loop of
+ * src/tplr/neurons.py:309-367): every peer's payload is flat over the batch
+ * (tplr_tensor_desc), results go to each descriptor's `dense` tensor ((R, C) with stride ld
+ * when use_dct != 0, contiguous (R/64, C/64, 64, 64) otherwise); d_scale (nullable) holds
+ * n_tensors x n_peers clip factors, d_sumsq (nullable) total_chunks partial sums. */
+int tplr_decode_aggregate_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale,
+                                int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
+                                int64_t total_chunks, int reduce_mode, int normalise, int use_dct, float* d_sumsq,
+                                void* stream);
 
 /* Row-wise scatter for layouts that are not 64x64 chunks (1-D tensors, un-chunked
  * 2-D rows; TopKCompressor.decompress, src/tplr/compress.py:452-474): d_out is
@@ -147,6 +176,14 @@ int tplr_peer_sumsq(const float* const* h_val, int n_peers, int64_t n, float* d_
  * d_median (nullable) receives med. */
 int tplr_clip_scales(const float* d_norm, int n_peers, int is_sumsq, float* d_scale, float* d_median,
                      void* stream);
+
+/* Batch forms for flat payloads: d_sumsq[t * n_peers + p] = sum of squares of peer p's values
+ * that belong to tensor t (the per-peer, per-parameter norms of src/tplr/neurons.py:346);
+ * d_scale[t * n_peers + p] from the lower median over the peers of tensor t. */
+int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr_tensor_desc* d_desc,
+                       int n_tensors, float* d_sumsq, void* stream);
+int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int is_sumsq, float* d_scale,
+                           float* d_median, void* stream);
 
 #ifdef __cplusplus
 }

@@ -740,12 +740,130 @@ def batch_decompress_decode(idxs: Sequence[torch.Tensor], vals: Sequence[torch.T
                              use_dct=use_dct, mean=mean, out=out, sumsq=sumsq)
 
 
+# ----------------------------------------------------------------------------------------
+# whole-gradient-set entry points: one launch for all tensors, flat payloads
+# ----------------------------------------------------------------------------------------
+class TensorBatch:
+    """A set of 2-D fp32 device tensors (dimensions multiples of 64) addressed as one list of
+    64x64 chunks: tensor by tensor, chunks row-major.  Holds the device-side descriptor table
+    the batch kernels walk.  The flat payload of a batch is indexed by the global chunk id:
+    indices of chunk g at byte g*3k/2, values at float g*k.  Build it once per model; the
+    tensors' storage must stay where it is (error-feedback buffers, gradients)."""
+
+    def __init__(self, tensors: Sequence[torch.Tensor]):
+        import numpy as np
+
+        if not tensors:
+            raise ValueError("TensorBatch needs at least one tensor")
+        dev = tensors[0].device
+        desc = np.zeros(len(tensors), dtype=np.dtype([("dense", "<u8"), ("ld", "<i8"), ("chunk_begin", "<i8"),
+                                                      ("x_chunks", "<i4"), ("y_chunks", "<i4")]))
+        begin = 0
+        self.offsets: list[int] = []
+        for i, t in enumerate(tensors):
+            _need_device(t, "TensorBatch")
+            if t.device != dev or t.dtype != torch.float32 or t.dim() != 2 or t.shape[0] % _CH or t.shape[1] % _CH \
+                    or t.stride(1) != 1 or t.stride(0) < t.shape[1]:
+                raise ValueError(f"tensor {i}: need fp32, 2-D, row-major, dimensions divisible by {_CH}, one device")
+            y, x = t.shape[0] // _CH, t.shape[1] // _CH
+            desc[i] = (t.data_ptr(), t.stride(0), begin, x, y)
+            self.offsets.append(begin)
+            begin += x * y
+        self.tensors = list(tensors)  # keeps the storage alive
+        self.total_chunks = begin
+        self.device = dev
+        self.table = torch.from_numpy(desc.view(np.uint8).copy()).to(dev)
+
+    def __len__(self) -> int:
+        return len(self.tensors)
+
+    def xshape(self, i: int) -> Shape4D:
+        t = self.tensors[i]
+        return (t.shape[0] // _CH, t.shape[1] // _CH, _CH, _CH)
+
+    def payload_slice(self, i: int, idx12: torch.Tensor, val: torch.Tensor, k: int):
+        """Tensor i's part of a flat payload, in the reference's per-parameter form."""
+        y, x, _, _ = self.xshape(i)
+        b, n = self.offsets[i], y * x
+        return idx12[b * (k // 2) * 3:(b + n) * (k // 2) * 3], val[b:b + n].reshape(y, x, k)
+
+
+@torch.no_grad()
+def encode_compress_batch(batch: TensorBatch, topk: int, *, use_dct: bool = True, idx12: torch.Tensor | None = None,
+                          val: torch.Tensor | None = None):
+    """encode + compress of every tensor of the batch in one launch (the per-parameter loop of
+    src/tplr/neurons.py:114-159).  Returns the flat payload (idx12 uint8, val (total_chunks, k))."""
+    lib = _lib.load()
+    k = _clamp_k(_CH * _CH, topk)
+    if k > _lib.TPLR_MAX_K:
+        raise NotImplementedError(f"top-{k}: the HIP select kernel handles k up to {_lib.TPLR_MAX_K}")
+    n = batch.total_chunks
+    if idx12 is None:
+        idx12 = torch.empty(n * (k // 2) * 3, dtype=torch.uint8, device=batch.device)
+    if val is None:
+        val = torch.empty((n, k), dtype=torch.float32, device=batch.device)
+    with torch.cuda.device(batch.device):
+        st = lib.tplr_encode_topk_pack_batch(_ptr(batch.table), len(batch), n, k, int(use_dct), _ptr(idx12), _ptr(val),
+                                             _stream(batch.device))
+    _lib.check(st, "tplr_encode_topk_pack_batch")
+    return idx12, val
+
+
+@torch.no_grad()
+def peer_clip_scales_batch(batch: TensorBatch, vals: Sequence[torch.Tensor], k: int) -> torch.Tensor:
+    """(n_tensors, n_peers) clip factors min(1, median_t / (norm_tp + 1e-8)) from flat payloads:
+    what outer_step's block_norms and batch_decompress's clip compute per parameter
+    (src/tplr/neurons.py:346, src/tplr/compress.py:526-556), for all parameters in two launches."""
+    lib = _lib.load()
+    P = len(vals)
+    if P > _lib.TPLR_MAX_PEERS:
+        raise NotImplementedError(f"{P} peers: the HIP aggregate kernel takes up to {_lib.TPLR_MAX_PEERS}")
+    dev = batch.device
+    ss = torch.empty((len(batch), P), dtype=torch.float32, device=dev)
+    scale = torch.empty_like(ss)
+    vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
+    with torch.cuda.device(dev):
+        _lib.check(lib.tplr_segment_sumsq(vp, P, k, _ptr(batch.table), len(batch), _ptr(ss), _stream(dev)),
+                   "tplr_segment_sumsq")
+        _lib.check(lib.tplr_clip_scales_batch(_ptr(ss), len(batch), P, 1, _ptr(scale), None, _stream(dev)),
+                   "tplr_clip_scales_batch")
+    return scale
+
+
+@torch.no_grad()
+def batch_decompress_decode_batch(out: TensorBatch, idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], k: int,
+                                  *, clip_norm: bool = True, scale: torch.Tensor | None = None, normalise: bool = False,
+                                  use_dct: bool = True, mean: bool = True, sumsq: torch.Tensor | None = None) -> None:
+    """batch_decompress + decode of every parameter in one launch (src/tplr/neurons.py:309-367):
+    peer p's flat payload is (idxs[p], vals[p]); results are written into the tensors of `out`."""
+    lib = _lib.load()
+    P = len(vals)
+    if P > _lib.TPLR_MAX_PEERS:
+        raise NotImplementedError(f"{P} peers: the HIP aggregate kernel takes up to {_lib.TPLR_MAX_PEERS}")
+    n = out.total_chunks
+    for i, v in zip(idxs, vals):
+        if i.dtype != torch.uint8:
+            raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
+        if v.dtype != torch.float32 or v.numel() != n * k or i.numel() * 2 != n * k * 3 or not v.is_contiguous():
+            raise RuntimeError(f"flat payload mismatch: {i.numel()} index bytes / {v.numel()} values for {n} chunks, k={k}")
+    if scale is None and clip_norm and not normalise:
+        scale = peer_clip_scales_batch(out, vals, k)
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+    vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
+    with torch.cuda.device(out.device):
+        st = lib.tplr_decode_aggregate_batch(ip, vp, _ptr(scale), P, k, _ptr(out.table), len(out), n,
+                                             _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM, int(normalise), int(use_dct),
+                                             _ptr(sumsq), _stream(out.device))
+    _lib.check(st, "tplr_decode_aggregate_batch")
+
+
 # the names BASELINE.json's north star uses (DeMo-era)
 TransformDCT = ChunkingTransformer
 CompressDCT = TopKCompressor
 
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
-    "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "ShapeT", "Shape4D", "TotK",
+    "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
+    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

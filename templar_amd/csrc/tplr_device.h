@@ -28,6 +28,14 @@ __device__ __forceinline__ int64_t xcd_contiguous(int64_t bid, int64_t grid) {
     return (bid & 7) * per + (bid >> 3);
 }
 
+// One wavefront per workgroup: LDS instructions of a wave execute in order, so lanes only need
+// the compiler to keep program order.  (A workgroup barrier would also drain the vector-memory
+// counter and stall the prefetch of the next chunk.)
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 __device__ __forceinline__ uint64_t* cand_slot(float* tile, int s) {
     return reinterpret_cast<uint64_t*>(tile + (s >> 1) * kLd + kChunk + ((s & 1) << 1));
 }
@@ -158,20 +166,46 @@ __device__ __forceinline__ uint32_t stat_threshold(uint32_t b1, uint32_t b2, int
 // 64-bit per-lane mask (hi: d = 0..31 at bits 31..0, lo: d = 32..63) of the values that are
 // not below the float threshold.  A superset is fine here, so NaN and any denormal-flush
 // behaviour of the compare only add candidates.
+__device__ __forceinline__ void filter16(uint32_t& m, float thr, float x0, float x1, float x2, float x3, float x4,
+                                         float x5, float x6, float x7, float x8, float x9, float x10, float x11,
+                                         float x12, float x13, float x14, float x15) {
+    // m = (m << 16) | predicate bits, first value in the highest bit: compare writes the carry,
+    // add-with-carry of m to itself shifts it in.
+    asm("v_cmp_nlt_f32_e64 vcc, |%[a0]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a1]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a2]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a3]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a4]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a5]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a6]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a7]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a8]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a9]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a10]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a11]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a12]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a13]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a14]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
+        "v_cmp_nlt_f32_e64 vcc, |%[a15]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc"
+        : [m] "+v"(m)
+        : [t] "s"(thr), [a0] "v"(x0), [a1] "v"(x1), [a2] "v"(x2), [a3] "v"(x3), [a4] "v"(x4), [a5] "v"(x5),
+          [a6] "v"(x6), [a7] "v"(x7), [a8] "v"(x8), [a9] "v"(x9), [a10] "v"(x10), [a11] "v"(x11), [a12] "v"(x12),
+          [a13] "v"(x13), [a14] "v"(x14), [a15] "v"(x15)
+        : "vcc");
+}
+
+// 64-bit per-lane mask (hi: d = 0..31 at bits 31..0, lo: d = 32..63) of the values that are
+// not below the float threshold.  A superset is fine here, so NaN and any denormal-flush
+// behaviour of the compare only add candidates.
 __device__ __forceinline__ void filter_masks(const float (&v)[64], float thr, uint32_t& mhi, uint32_t& mlo) {
     uint32_t hi = 0, lo = 0;
-#pragma unroll
-    for (int d = 0; d < 32; ++d)
-        asm volatile("v_cmp_nlt_f32_e64 vcc, |%1|, %2\n\tv_addc_co_u32_e32 %0, vcc, %0, %0, vcc"
-                     : "+v"(hi)
-                     : "v"(v[d]), "s"(thr)
-                     : "vcc");
-#pragma unroll
-    for (int d = 32; d < 64; ++d)
-        asm volatile("v_cmp_nlt_f32_e64 vcc, |%1|, %2\n\tv_addc_co_u32_e32 %0, vcc, %0, %0, vcc"
-                     : "+v"(lo)
-                     : "v"(v[d]), "s"(thr)
-                     : "vcc");
+    filter16(hi, thr, v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9], v[10], v[11], v[12], v[13], v[14], v[15]);
+    filter16(hi, thr, v[16], v[17], v[18], v[19], v[20], v[21], v[22], v[23], v[24], v[25], v[26], v[27], v[28], v[29],
+             v[30], v[31]);
+    filter16(lo, thr, v[32], v[33], v[34], v[35], v[36], v[37], v[38], v[39], v[40], v[41], v[42], v[43], v[44], v[45],
+             v[46], v[47]);
+    filter16(lo, thr, v[48], v[49], v[50], v[51], v[52], v[53], v[54], v[55], v[56], v[57], v[58], v[59], v[60], v[61],
+             v[62], v[63]);
     mhi = hi;
     mlo = lo;
 }
@@ -226,50 +260,66 @@ __device__ __forceinline__ void keep_first(uint32_t& hi, uint32_t& lo, int keep)
     lo = l;
 }
 
-__device__ __forceinline__ uint64_t u64_max(uint64_t a, uint64_t b) { return a > b ? a : b; }
-__device__ __forceinline__ uint64_t u64_min(uint64_t a, uint64_t b) { return a > b ? b : a; }
-
 __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t x, int j) {
     const uint32_t lo = __shfl_xor(static_cast<uint32_t>(x), j);
     const uint32_t hi = __shfl_xor(static_cast<uint32_t>(x >> 32), j);
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
-// bitonic sort, descending, of 64 (one per lane) or 128 (two per lane) keys
-__device__ __forceinline__ void sort64_desc(uint64_t& e, int lane) {
-#pragma unroll
-    for (int k2 = 2; k2 <= 64; k2 <<= 1) {
-#pragma unroll
-        for (int j = k2 >> 1; j > 0; j >>= 1) {
-            const uint64_t o = shfl_xor_u64(e, j);
-            const bool keepmax = ((lane & k2) == 0) == ((lane & j) == 0);
-            e = keepmax ? u64_max(e, o) : u64_min(e, o);
-        }
+// lanes (bit i = lane i) that keep the larger key in the compare-exchange with partner lane ^ j
+// of a bitonic stage of block size k2 (descending result); `base` is the element index of lane 0
+constexpr uint64_t keepmax_mask(int k2, int j, int base) {
+    uint64_t m = 0;
+    for (int lane = 0; lane < 64; ++lane) {
+        const int i = base + lane;
+        if (((i & k2) == 0) == ((i & j) == 0)) m |= 1ull << lane;
     }
+    return m;
 }
 
-__device__ __forceinline__ void sort128_desc(uint64_t& e0, uint64_t& e1, int lane) {
-#pragma unroll
-    for (int k2 = 2; k2 <= 128; k2 <<= 1) {
-#pragma unroll
-        for (int j = k2 >> 1; j > 0; j >>= 1) {
-            if (j == 64) {
-                // only reached with k2 = 128: one descending block, lower half keeps the max
-                const uint64_t a = u64_max(e0, e1), b = u64_min(e0, e1);
-                e0 = a;
-                e1 = b;
-            } else {
-                const uint64_t o0 = shfl_xor_u64(e0, j);
-                const uint64_t o1 = shfl_xor_u64(e1, j);
-                const bool low = (lane & j) == 0;
-                const bool up0 = (lane & k2) == 0;         // element index = lane
-                const bool up1 = ((lane + 64) & k2) == 0;  // element index = lane + 64
-                e0 = (up0 == low) ? u64_max(e0, o0) : u64_min(e0, o0);
-                e1 = (up1 == low) ? u64_max(e1, o1) : u64_min(e1, o1);
-            }
-        }
-    }
+// e <- max(e, o) on the lanes of `keepmax`, min(e, o) elsewhere: one 64-bit compare, one scalar
+// xnor with the lane mask, two selects.
+__device__ __forceinline__ uint64_t cmp_exchange(uint64_t e, uint64_t o, uint64_t keepmax) {
+    uint64_t take;
+    asm("v_cmp_gt_u64_e64 %0, %1, %2\n\ts_xnor_b64 %0, %0, %3" : "=&s"(take) : "v"(o), "v"(e), "s"(keepmax) : "scc");
+    uint32_t lo, hi;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(lo) : "v"(static_cast<uint32_t>(e)), "v"(static_cast<uint32_t>(o)), "s"(take));
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3"
+        : "=v"(hi)
+        : "v"(static_cast<uint32_t>(e >> 32)), "v"(static_cast<uint32_t>(o >> 32)), "s"(take));
+    return (static_cast<uint64_t>(hi) << 32) | lo;
 }
+
+// bitonic sort, descending, of 64 (one per lane) or 128 (two per lane) keys
+template <int K2, int J>
+__device__ __forceinline__ void sort64_step(uint64_t& e) {
+    e = cmp_exchange(e, shfl_xor_u64(e, J), keepmax_mask(K2, J, 0));
+    if constexpr (J > 1)
+        sort64_step<K2, J / 2>(e);
+    else if constexpr (K2 < 64)
+        sort64_step<K2 * 2, K2>(e);
+}
+
+__device__ __forceinline__ void sort64_desc(uint64_t& e, int) { sort64_step<2, 1>(e); }
+
+template <int K2, int J>
+__device__ __forceinline__ void sort128_step(uint64_t& e0, uint64_t& e1) {
+    if constexpr (J == 64) {
+        // only reached with K2 = 128: one descending block, the lower half keeps the max
+        const uint64_t a = e0 > e1 ? e0 : e1, b = e0 > e1 ? e1 : e0;
+        e0 = a;
+        e1 = b;
+    } else {
+        e0 = cmp_exchange(e0, shfl_xor_u64(e0, J), keepmax_mask(K2, J, 0));
+        e1 = cmp_exchange(e1, shfl_xor_u64(e1, J), keepmax_mask(K2, J, 64));
+    }
+    if constexpr (J > 1)
+        sort128_step<K2, J / 2>(e0, e1);
+    else if constexpr (K2 < 128)
+        sort128_step<K2 * 2, K2>(e0, e1);
+}
+
+__device__ __forceinline__ void sort128_desc(uint64_t& e0, uint64_t& e1, int) { sort128_step<2, 1>(e0, e1); }
 
 template <bool kTwo>
 __device__ __forceinline__ Selected select_topk(const float (&v)[64], float* tile, int lane, int k) {
@@ -348,7 +398,7 @@ __device__ __forceinline__ Selected select_topk(const float (&v)[64], float* til
         const uint32_t key = mag_key(__float_as_uint(row[d]));
         *cand_slot(tile, slot++) = (static_cast<uint64_t>(key) << 32) | (0xffffffffu - (lane * 64 + d));
     }
-    __syncthreads();
+    wave_lds_fence();
 
     Selected out;
     out.idx1 = 0;

@@ -77,30 +77,59 @@ __global__ __launch_bounds__(256) void k_unpack12(const uint8_t* __restrict__ in
 // =========================================================================================
 // chunk loaders / storers for the (R, C) row-major side: lane = column
 // =========================================================================================
+// Chunk rows through buffer instructions: one resource descriptor per chunk (scalar base,
+// byte range for bounds checking), the row offset r*ld in a scalar register and lane*4 as the
+// only vector operand, so addressing costs no vector ALU work.  ld*4*63 must fit in 31 bits.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t chunk_rsrc(const void* chunk0, int64_t ld) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(chunk0), 0, static_cast<int>((63 * ld + 64) * 4),
+                                             0x00020000);
+}
+
+template <int kRow0 = 0, int kRow1 = 64>
+__device__ __forceinline__ void load_chunk_rows(float (&v)[64], const void* chunk0, int64_t ld, int lane) {
+    const __amdgpu_buffer_rsrc_t rs = chunk_rsrc(chunk0, ld);
+    const int ld4 = static_cast<int>(ld) * 4;
+#pragma unroll
+    for (int r = kRow0; r < kRow1; ++r)
+        v[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4, r * ld4, 2));
+}
+
+__device__ __forceinline__ void store_chunk_rows(const float (&v)[64], void* chunk0, int64_t ld, int lane) {
+    const __amdgpu_buffer_rsrc_t rs = chunk_rsrc(chunk0, ld);
+    const int ld4 = static_cast<int>(ld) * 4;
+#pragma unroll
+    for (int r = 0; r < 64; ++r)
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v[r]), rs, lane * 4, r * ld4, 2);
+}
+
 __device__ __forceinline__ void load_chunk_cols(float (&v)[64], const float* __restrict__ x, int64_t ld,
                                                 int64_t y, int64_t xc, int lane) {
-    const float* p = x + (y * 64) * ld + xc * 64 + lane;
-#pragma unroll
-    for (int r = 0; r < 64; ++r) v[r] = __builtin_nontemporal_load(p + r * ld);
+    load_chunk_rows(v, x + (y * 64) * ld + xc * 64, ld, lane);
 }
 
 __device__ __forceinline__ void store_chunk_cols(const float (&v)[64], float* __restrict__ x, int64_t ld,
                                                  int64_t y, int64_t xc, int lane) {
-    float* p = x + (y * 64) * ld + xc * 64 + lane;
-#pragma unroll
-    for (int r = 0; r < 64; ++r) __builtin_nontemporal_store(v[r], p + r * ld);
+    store_chunk_rows(v, x + (y * 64) * ld + xc * 64, ld, lane);
 }
 
 // forward 2-D transform of the chunk held column-per-lane; result row-per-lane:
 // v[d] = coef[lane][d], and the tile is left free
-template <bool kUseDct>
-__device__ __forceinline__ void chunk_forward(float (&v)[64], float* tile, int lane) {
+struct NoHook {
+    __device__ __forceinline__ void operator()() const {}
+};
+
+template <bool kUseDct, typename Hook = NoHook>
+__device__ __forceinline__ void chunk_forward(float (&v)[64], float* tile, int lane, Hook between_passes = Hook()) {
     if (kUseDct) dct64_fwd(v);  // along rows k: v[b] = sum_k X[k][lane] F[k][b]
+    // keep the hook's memory requests behind the first pass: tie them to its last results
+    asm volatile("" : "+v"(v[1]), "+v"(v[31]), "+v"(v[63])::"memory");
+    between_passes();
+    asm volatile("" ::: "memory");
     regs_to_tile_cols(v, tile, lane);
-    __syncthreads();
+    wave_lds_fence();
     tile_rows_to_regs(v, tile, lane);
     if (kUseDct) dct64_fwd(v);  // along columns l: v[d] = sum_l T[lane][l] F[l][d]
-    __syncthreads();
+    wave_lds_fence();
 }
 
 // inverse: tile holds coef rows; result column-per-lane v[k] = x[k][lane]
@@ -109,12 +138,108 @@ __device__ __forceinline__ void chunk_inverse(float (&v)[64], float* tile, int l
     if (kUseDct) {
         tile_rows_to_regs(v, tile, lane);
         dct64_inv(v);  // along d: v[l] = sum_d Y[lane][d] F[l][d]
-        __syncthreads();
+        wave_lds_fence();
         regs_to_tile_rows(v, tile, lane);
-        __syncthreads();
+        wave_lds_fence();
     }
     tile_cols_to_regs(v, tile, lane);
     if (kUseDct) dct64_inv(v);  // along b: v[k] = sum_b Z[b][lane] F[k][b]
+}
+
+// -----------------------------------------------------------------------------------------
+// Persistent kernels walk a contiguous range of the batch's chunk list.  A cursor keeps the
+// current tensor's descriptor and the chunk's (y, x) position in wave-uniform registers.
+// -----------------------------------------------------------------------------------------
+// Pointers that come out of descriptor tables are not kernel arguments, so the compiler
+// cannot tell that they are global memory; say so, or it emits FLAT accesses (which also
+// count as LDS traffic and serialise against the tile).
+using gfloat = __attribute__((address_space(1))) float;
+using gbyte = __attribute__((address_space(1))) uint8_t;
+
+struct Cursor {
+    const tplr_tensor_desc* table;
+    int n_tensors;
+    int t;
+    gfloat* base;
+    int64_t ld;
+    int64_t begin, end;  // chunk ids covered by tensor t
+    int X;
+    int64_t y;
+    int xc;
+};
+
+// descriptor fields are the same for every lane: move them to scalar registers so that chunk
+// rows are addressed as scalar base + 32-bit lane offset
+__device__ __forceinline__ int64_t uniform64(int64_t x) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(x));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(static_cast<uint64_t>(x) >> 32));
+    return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+__device__ __forceinline__ void cursor_take(Cursor& c, const tplr_tensor_desc& d) {
+    c.base = (gfloat*)uniform64(reinterpret_cast<int64_t>(d.dense));
+    c.ld = uniform64(d.ld);
+    c.begin = uniform64(d.chunk_begin);
+    c.X = __builtin_amdgcn_readfirstlane(d.x_chunks);
+    c.end = c.begin + static_cast<int64_t>(c.X) * __builtin_amdgcn_readfirstlane(d.y_chunks);
+}
+
+__device__ __forceinline__ void cursor_seek(Cursor& c, const tplr_tensor_desc* table, const tplr_tensor_desc& single,
+                                            int n_tensors, int64_t g) {
+    c.table = table;
+    c.n_tensors = n_tensors;
+    c.t = 0;
+    if (table) {
+        int lo = 0, hi = n_tensors;  // last tensor whose chunk_begin <= g and that is not empty
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (table[mid].chunk_begin <= g)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        c.t = lo;
+        cursor_take(c, table[lo]);
+    } else {
+        cursor_take(c, single);
+    }
+    const int64_t local = g - c.begin;
+    c.y = local / c.X;
+    c.xc = static_cast<int>(local - c.y * c.X);
+}
+
+// advance to chunk g (= previous chunk + 1)
+__device__ __forceinline__ void cursor_next(Cursor& c, int64_t g) {
+    if (++c.xc == c.X) {
+        c.xc = 0;
+        ++c.y;
+    }
+    while (g >= c.end && c.t + 1 < c.n_tensors) {  // batch mode only: single tensors never get here
+        ++c.t;
+        cursor_take(c, c.table[c.t]);
+        c.y = 0;
+        c.xc = 0;
+    }
+}
+
+// the contiguous slice of [0, total) that workgroup `bid` of a grid of G (multiple of 8) owns;
+// workgroups b, b+8, b+16, ... run on the same XCD and take neighbouring slices
+__device__ __forceinline__ void my_range(int64_t total, int64_t& g0, int64_t& g1) {
+    const int64_t bid = blockIdx.x, S = gridDim.x >> 3;
+    const int64_t xcd = bid & 7, slot = bid >> 3;
+    const int64_t per = (total + 7) >> 3;
+    const int64_t xb = xcd * per;
+    int64_t xe = xb + per;
+    xe = xe > total ? total : xe;
+    const int64_t len = xe > xb ? xe - xb : 0;
+    g0 = xb + len * slot / S;
+    g1 = xb + len * (slot + 1) / S;
+}
+
+template <int kRow0 = 0, int kRow1 = 64>
+__device__ __forceinline__ void load_chunk_cols(float (&v)[64], const Cursor& c, int lane) {
+    load_chunk_rows<kRow0, kRow1>(v, (const void*)(c.base + (c.y * 64) * c.ld + static_cast<int64_t>(c.xc) * 64),
+                                  c.ld, lane);
 }
 
 // =========================================================================================
@@ -250,22 +375,48 @@ __global__ __launch_bounds__(64) void k_topk_rows(const float* __restrict__ coef
     emit_selected(s, lane, k, row, idx12, val);
 }
 
+// Persistent fused encode: every wave walks its slice of the chunk list; the 64 row loads of
+// the next chunk are in flight while the current one is transformed and selected.
 template <bool kTwo, bool kUseDct>
-__global__ __launch_bounds__(64) void k_encode_topk_pack(const float* __restrict__ x, int64_t ld, int64_t X,
-                                                         int64_t n_chunks, int k, uint8_t* __restrict__ idx12,
+__global__ __launch_bounds__(64) void k_encode_topk_pack(const tplr_tensor_desc* __restrict__ table,
+                                                         const tplr_tensor_desc single, int n_tensors,
+                                                         int64_t total, int k, uint8_t* __restrict__ idx12,
                                                          float* __restrict__ val) {
     __shared__ __align__(16) float tile[kTileFloats];
     const int lane = threadIdx.x;
-    const int64_t chunk = xcd_contiguous(blockIdx.x, gridDim.x);
-    if (chunk >= n_chunks) return;
-    const int64_t y = chunk / X, xc = chunk - y * X;
-    float v[64];
-    load_chunk_cols(v, x, ld, y, xc, lane);
-    chunk_forward<kUseDct>(v, tile, lane);
-    regs_to_tile_rows(v, tile, lane);
-    __syncthreads();
-    const Selected s = select_topk<kTwo>(v, tile, lane, k);
-    emit_selected(s, lane, k, chunk, idx12, val);
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
+    Cursor c;
+    cursor_seek(c, table, single, n_tensors, g0);
+    // Loads and stores share one completion counter and complete out of order with respect to
+    // each other, so a wait for the prefetched rows also waits for every store issued before it.
+    // The selection of chunk g is therefore written in the middle of iteration g + 1, a
+    // transform pass away from the waits on either side.
+    float v[64], nx[64];
+    load_chunk_cols(nx, c, lane);
+    Selected prev = {};
+    for (int64_t g = g0; g < g1; ++g) {
+#pragma unroll
+        for (int r = 0; r < 64; ++r) v[r] = nx[r];
+        // at most 63 vector-memory operations can be outstanding: the previous selection is
+        // written, and the last rows requested, after the first transform pass
+        constexpr int kSplit = 56;
+        const bool more = g + 1 < g1;
+        if (more) {
+            cursor_next(c, g + 1);
+            load_chunk_cols<0, kSplit>(nx, c, lane);
+        }
+        chunk_forward<kUseDct>(v, tile, lane, [&]() {
+            if (g > g0) emit_selected(prev, lane, k, g - 1, idx12, val);
+            if (more) load_chunk_cols<kSplit, 64>(nx, c, lane);
+        });
+        regs_to_tile_rows(v, tile, lane);
+        wave_lds_fence();
+        prev = select_topk<kTwo>(v, tile, lane, k);
+        wave_lds_fence();
+    }
+    emit_selected(prev, lane, k, g1 - 1, idx12, val);
 }
 
 // =========================================================================================
@@ -279,44 +430,85 @@ struct PeerPtrs {
 __device__ __forceinline__ int tile_pos(uint32_t idx) { return (idx >> 6) * kLd + (idx & 63); }
 
 // 12-bit index j of a packed row (byte pointer to the row start)
-__device__ __forceinline__ uint32_t load_idx12(const uint8_t* __restrict__ row, int j) {
-    const uint8_t* b = row + 3 * (j >> 1) + (j & 1);
+template <typename BytePtr>
+__device__ __forceinline__ uint32_t load_idx12(BytePtr row, int j) {
+    BytePtr b = row + 3 * (j >> 1) + (j & 1);
     const uint32_t w = b[0] | (static_cast<uint32_t>(b[1]) << 8);
     return (j & 1) ? (w >> 4) : (w & 0xfffu);
 }
 
+// Up to 64 peers keep their (index, value) base pointers in the padding columns of the tile
+// (16 bytes per tile row); beyond that they are read from the kernel arguments.
+struct PeerTable {
+    const PeerPtrs* pp;
+    float* tile;
+    bool in_lds;
+    __device__ __forceinline__ void get(int p, const gbyte*& ip, const gfloat*& vp) const {
+        if (in_lds) {
+            const uint64_t* slot = reinterpret_cast<const uint64_t*>(tile + p * kLd + kChunk);
+            ip = (const gbyte*)slot[0];
+            vp = (const gfloat*)slot[1];
+        } else {
+            ip = (const gbyte*)pp->idx[p];
+            vp = (const gfloat*)pp->val[p];
+        }
+    }
+};
+
+constexpr int kUnitRegs = 16;  // wave-wide batches of one chunk's entries that stay in registers
+
+struct UnitRegs {
+    uint32_t ix[kUnitRegs];
+    float a[kUnitRegs];
+    uint32_t ok;  // bit i: unit i holds an entry for this lane
+};
+
+typedef uint16_t __attribute__((aligned(1))) unaligned_u16;
+using gu16 = __attribute__((address_space(1))) unaligned_u16;
+
+// 12-bit index j of a packed row: the two bytes that hold it, as one unaligned 16-bit load
+__device__ __forceinline__ uint32_t load_idx12_g(const gbyte* row, int j) {
+    const uint32_t w = *(const gu16*)(row + 3 * (j >> 1) + (j & 1));
+    return (j & 1) ? (w >> 4) : (w & 0xfffu);
+}
+
+// Persistent fused decode: per chunk, the peers' entries are accumulated in peer order into an
+// LDS tile (sum) and a byte-per-coefficient contribution count, touched coefficients are
+// divided by their count, and the tile goes through the inverse 2-D DCT.  Because loads and
+// stores complete out of order with respect to each other on one counter, the 64 row stores of
+// chunk g are issued at the top of iteration g + 1, right after the wait for that chunk's
+// payload registers; the payload of chunk g + 1 is requested once chunk g's entries are in the
+// tile and travels during its inverse transform.
 template <bool kUseDct>
-__global__ __launch_bounds__(64) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale,
-                                                         int P, int k, int64_t X, int64_t n_chunks,
-                                                         int reduce_mode, int normalise, float* __restrict__ out,
-                                                         int64_t ld_out, float* __restrict__ sumsq) {
+__global__ __launch_bounds__(64) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
+                                                         int k, const tplr_tensor_desc* __restrict__ table,
+                                                         const tplr_tensor_desc single, int n_tensors, int64_t total,
+                                                         int reduce_mode, int normalise,
+                                                         float* __restrict__ sumsq) {
     __shared__ __align__(16) float tile[kTileFloats];
     __shared__ __align__(16) uint32_t cnt[1024];  // 4096 one-byte contribution counters
     const int lane = threadIdx.x;
-    const int64_t chunk = xcd_contiguous(blockIdx.x, gridDim.x);
-    if (chunk >= n_chunks) return;
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
 
-    {
-        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int c = 0; c < kTileFloats / 256; ++c) reinterpret_cast<float4*>(tile)[c * 64 + lane] = z;
-        const uint4 zi = make_uint4(0, 0, 0, 0);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) reinterpret_cast<uint4*>(cnt)[c * 64 + lane] = zi;
+    PeerTable pt{&pp, tile, P <= 64};
+    if (pt.in_lds && lane < P) {
+        uint64_t* slot = reinterpret_cast<uint64_t*>(tile + lane * kLd + kChunk);
+        slot[0] = reinterpret_cast<uint64_t>(pp.idx[lane]);
+        slot[1] = reinterpret_cast<uint64_t>(pp.val[lane]);
     }
-    __syncthreads();
+    wave_lds_fence();
 
-    // A "unit" is one wave-wide batch of entries of this chunk: for k <= 64 it covers
-    // G = 64 / k whole peers (lane -> peer g_lane, entry j_lane), for k > 64 one 64-entry
-    // slice of one peer.  Peers are applied strictly in order (g loop below).
+    // A "unit" is one wave-wide batch of entries of a chunk: for k <= 64 it covers G = 64 / k
+    // whole peers (lane -> peer g_lane, entry j_lane), for k > 64 one 64-entry slice of one
+    // peer.  Peers are applied strictly in order (gq loop in apply_unit).
     const int G = k >= 64 ? 1 : 64 / k;
     const int S = (k + 63) >> 6;
     const int g_lane = k >= 64 ? 0 : lane / k;
     const int j_lane = k >= 64 ? lane : lane - g_lane * k;
     const int n_units = k >= 64 ? P * S : (P + G - 1) / G;
-    const int64_t idx_row = chunk * (k + (k >> 1));
-    const int64_t val_row = chunk * k;
-    bool collide = false;
+    const int64_t idx_stride = k + (k >> 1);
 
     auto entry = [&](int u, int& p, int& j) -> bool {
         if (k >= 64) {
@@ -329,105 +521,180 @@ __global__ __launch_bounds__(64) void k_decode_aggregate(const PeerPtrs pp, cons
         return g_lane < G && p < P;
     };
 
-    if (normalise) {
-        // per-peer, per-chunk L2 normalisation (compress.py:541-545); simple, unbatched
-        for (int p = 0; p < P; ++p) {
-            float ss = 0.f;
-            for (int j = lane; j < k; j += 64) {
-                const float a = pp.val[p][val_row + j];
-                ss += a * a;
-            }
-            const float nrm = __builtin_sqrtf(wave_sum_f32(ss)) + 1e-8f;
-            for (int j0 = 0; j0 < k; j0 += 64) {
-                const int j = j0 + lane;
-                if (j < k) {
-                    const uint32_t ix = load_idx12(pp.idx[p] + idx_row, j);
-                    const float a = pp.val[p][val_row + j] / nrm;
-                    atomicAdd(&tile[tile_pos(ix)], a);
-                    const uint32_t sh = (ix & 3) * 8;
-                    const uint32_t old = atomicAdd(&cnt[ix >> 2], 1u << sh);
-                    collide |= ((old >> sh) & 0xffu) != 0;
-                }
+    auto load_units = [&](UnitRegs& r, int64_t g, int t) {
+        r.ok = 0;
+#pragma unroll
+        for (int i = 0; i < kUnitRegs; ++i) {
+            int p, j;
+            r.ix[i] = 0;
+            r.a[i] = 0.f;
+            if (i < n_units && entry(i, p, j)) {
+                r.ok |= 1u << i;
+                const gbyte* ip;
+                const gfloat* vp;
+                pt.get(p, ip, vp);
+                r.ix[i] = load_idx12_g(ip + g * idx_stride, j);
+                r.a[i] = vp[g * k + j];
+                if (scale) r.a[i] *= scale[static_cast<int64_t>(t) * P + p];
             }
         }
-    } else {
-        constexpr int kBatch = 8;
-        for (int u0 = 0; u0 < n_units; u0 += kBatch) {
-            uint32_t ix[kBatch];
-            float a[kBatch];
-            bool ok[kBatch];
+    };
+
+    bool collide = false;
+    auto apply_one = [&](uint32_t ix, float a) {
+        atomicAdd(&tile[tile_pos(ix)], a);
+        const uint32_t sh = (ix & 3) * 8;
+        const uint32_t old = atomicAdd(&cnt[ix >> 2], 1u << sh);
+        collide |= ((old >> sh) & 0xffu) != 0;
+    };
+    auto claim_divide = [&](uint32_t ix) {
+        // exactly one entry per destination claims the counter and divides the sum
+        const uint32_t sh = (ix & 3) * 8;
+        const uint32_t old = atomicAnd(&cnt[ix >> 2], ~(0xffu << sh));
+        const uint32_t n = (old >> sh) & 0xffu;
+        if (n > 1) {
+            float* t = &tile[tile_pos(ix)];
+            *t = *t / static_cast<float>(n);
+        }
+    };
+
+    Cursor c;
+    cursor_seek(c, table, single, n_tensors, g0);
+    UnitRegs cur;
+    if (!normalise) load_units(cur, g0, c.t);
+
+    float v[64];  // inverse transform of the previous chunk, stored one iteration late
+    gfloat* prev_chunk0 = nullptr;
+    int64_t prev_ld = 0;
+    float prev_ss = 0.f;
+
+    for (int64_t g = g0; g < g1; ++g) {
+        if (g > g0) {
+            if (kUseDct)
+                store_chunk_rows(v, (void*)prev_chunk0, prev_ld, lane);
+            else
+                tile_to_flat(tile, (float*)prev_chunk0, lane);
+            if (sumsq && lane == 0) sumsq[g - 1] = prev_ss;
+            wave_lds_fence();
+        }
+        // where this chunk's result goes (the cursor moves on before the store)
+        const int t_now = c.t;
+        prev_ld = c.ld;
+        prev_chunk0 = kUseDct ? c.base + (c.y * 64) * c.ld + static_cast<int64_t>(c.xc) * 64
+                              : c.base + (g - c.begin) * 4096;
+
+        {
+            const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+            float4* row = reinterpret_cast<float4*>(tile + lane * kLd);  // data columns only
 #pragma unroll
-            for (int t = 0; t < kBatch; ++t) {
-                int p, j;
-                ok[t] = (u0 + t < n_units) && entry(u0 + t, p, j);
-                ix[t] = 0;
-                a[t] = 0.f;
-                if (ok[t]) {
-                    ix[t] = load_idx12(pp.idx[p] + idx_row, j);
-                    a[t] = pp.val[p][val_row + j];
-                    if (scale) a[t] *= scale[p];
+            for (int q = 0; q < 16; ++q) row[q] = z;
+            const uint4 zi = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
+        }
+        wave_lds_fence();
+        collide = false;
+
+        if (normalise) {
+            // per-peer, per-chunk L2 normalisation (compress.py:541-545); simple, unbatched
+            for (int p = 0; p < P; ++p) {
+                const gbyte* ip;
+                const gfloat* vp;
+                pt.get(p, ip, vp);
+                float ss = 0.f;
+                for (int j = lane; j < k; j += 64) {
+                    const float a = vp[g * k + j];
+                    ss += a * a;
+                }
+                const float nrm = __builtin_sqrtf(wave_sum_f32(ss)) + 1e-8f;
+                for (int j0 = 0; j0 < k; j0 += 64) {
+                    const int j = j0 + lane;
+                    if (j < k) apply_one(load_idx12_g(ip + g * idx_stride, j), vp[g * k + j] / nrm);
                 }
             }
+        } else {
 #pragma unroll
-            for (int t = 0; t < kBatch; ++t) {
-                if (u0 + t >= n_units) break;
-                for (int g = 0; g < G; ++g) {
-                    if (ok[t] && g_lane == g) {
-                        atomicAdd(&tile[tile_pos(ix[t])], a[t]);
-                        const uint32_t sh = (ix[t] & 3) * 8;
-                        const uint32_t old = atomicAdd(&cnt[ix[t] >> 2], 1u << sh);
-                        collide |= ((old >> sh) & 0xffu) != 0;
+            for (int i = 0; i < kUnitRegs; ++i) {
+                if (i < n_units) {
+                    for (int gq = 0; gq < G; ++gq)
+                        if (((cur.ok >> i) & 1u) && g_lane == gq) apply_one(cur.ix[i], cur.a[i]);
+                }
+            }
+            for (int u = kUnitRegs; u < n_units; ++u) {  // more entries than the registers hold
+                int p, j;
+                const bool ok = entry(u, p, j);
+                uint32_t ix = 0;
+                float a = 0.f;
+                if (ok) {
+                    const gbyte* ip;
+                    const gfloat* vp;
+                    pt.get(p, ip, vp);
+                    ix = load_idx12_g(ip + g * idx_stride, j);
+                    a = vp[g * k + j];
+                    if (scale) a *= scale[static_cast<int64_t>(t_now) * P + p];
+                }
+                for (int gq = 0; gq < G; ++gq)
+                    if (ok && g_lane == gq) apply_one(ix, a);
+            }
+        }
+        wave_lds_fence();
+
+        if (reduce_mode == TPLR_REDUCE_MEAN && __any(collide)) {
+            if (normalise) {
+                for (int p = 0; p < P; ++p) {
+                    const gbyte* ip;
+                    const gfloat* vp;
+                    pt.get(p, ip, vp);
+                    for (int j = lane; j < k; j += 64) claim_divide(load_idx12_g(ip + g * idx_stride, j));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < kUnitRegs; ++i)
+                    if (i < n_units && ((cur.ok >> i) & 1u)) claim_divide(cur.ix[i]);
+                for (int u = kUnitRegs; u < n_units; ++u) {
+                    int p, j;
+                    if (entry(u, p, j)) {
+                        const gbyte* ip;
+                        const gfloat* vp;
+                        pt.get(p, ip, vp);
+                        claim_divide(load_idx12_g(ip + g * idx_stride, j));
                     }
                 }
             }
+            wave_lds_fence();
         }
-    }
-    __syncthreads();
 
-    if (reduce_mode == TPLR_REDUCE_MEAN && __any(collide)) {
-        // exactly one entry per destination claims the counter and divides the sum
-        for (int u = 0; u < n_units; ++u) {
-            int p, j;
-            if (entry(u, p, j)) {
-                const uint32_t ix = load_idx12(pp.idx[p] + idx_row, j);
-                const uint32_t sh = (ix & 3) * 8;
-                const uint32_t old = atomicAnd(&cnt[ix >> 2], ~(0xffu << sh));
-                const uint32_t c = (old >> sh) & 0xffu;
-                if (c > 1) {
-                    float* t = &tile[tile_pos(ix)];
-                    *t = *t / static_cast<float>(c);
-                }
+        // the next chunk's payload travels while this one goes through the inverse transform
+        if (g + 1 < g1) {
+            cursor_next(c, g + 1);
+            if (!normalise) load_units(cur, g + 1, c.t);
+        }
+
+        if (kUseDct) {
+            chunk_inverse<true>(v, tile, lane);
+            if (sumsq) {
+                float ss = 0.f;
+#pragma unroll
+                for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
+                prev_ss = wave_sum_f32(ss);
             }
-        }
-        __syncthreads();
-    }
-
-    if (kUseDct) {
-        const int64_t y = chunk / X, xc = chunk - y * X;
-        float v[64];
-        chunk_inverse<true>(v, tile, lane);
-        store_chunk_cols(v, out, ld_out, y, xc, lane);
-        if (sumsq) {
+        } else if (sumsq) {
             float ss = 0.f;
 #pragma unroll
-            for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
-            ss = wave_sum_f32(ss);
-            if (lane == 0) sumsq[chunk] = ss;
-        }
-    } else {
-        tile_to_flat(tile, out + chunk * 4096, lane);
-        if (sumsq) {
-            float ss = 0.f;
-#pragma unroll
-            for (int c = 0; c < 16; ++c) {
-                const int q = c * 64 + lane;
+            for (int q0 = 0; q0 < 16; ++q0) {
+                const int q = q0 * 64 + lane;
                 const float4 t = *reinterpret_cast<const float4*>(tile + (q >> 4) * kLd + ((q & 15) << 2));
                 ss += t.x * t.x + t.y * t.y + t.z * t.z + t.w * t.w;
             }
-            ss = wave_sum_f32(ss);
-            if (lane == 0) sumsq[chunk] = ss;
+            prev_ss = wave_sum_f32(ss);
         }
+        wave_lds_fence();
     }
+    if (kUseDct)
+        store_chunk_rows(v, (void*)prev_chunk0, prev_ld, lane);
+    else
+        tile_to_flat(tile, (float*)prev_chunk0, lane);
+    if (sumsq && lane == 0) sumsq[g1 - 1] = prev_ss;
 }
 
 // generic rows (1-D tensors, un-chunked 2-D rows): exact source-order accumulation
@@ -510,12 +777,32 @@ __global__ __launch_bounds__(1024) void k_peer_sumsq(const ValPtrs vp, int64_t n
     }
 }
 
+// one block per (tensor, peer): sum of squares of that tensor's slice of the peer's values
+__global__ __launch_bounds__(256) void k_segment_sumsq(const ValPtrs vp, int P, int k,
+                                                       const tplr_tensor_desc* __restrict__ table,
+                                                       float* __restrict__ sumsq) {
+    __shared__ float part[4];
+    const int t = blockIdx.x / P, p = blockIdx.x - t * P;
+    const tplr_tensor_desc d = table[t];
+    const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks * k;
+    const float* v = vp.val[p] + d.chunk_begin * k;
+    float s = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += 256) s = __builtin_fmaf(v[i], v[i], s);
+    s = wave_sum_f32(s);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) sumsq[blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+// one block per tensor: scale[t][p] = min(1, med_t / (norm[t][p] + 1e-8))
 __global__ __launch_bounds__(128) void k_clip_scales(const float* __restrict__ norm, int P, int is_sumsq,
                                                      float* __restrict__ scale, float* __restrict__ median) {
     __shared__ float nv[TPLR_MAX_PEERS];
     __shared__ float med;
     const int i = threadIdx.x;
-    if (i < P) nv[i] = is_sumsq ? __builtin_sqrtf(norm[i]) : norm[i];
+    const int64_t off = static_cast<int64_t>(blockIdx.x) * P;
+    if (i < P) nv[i] = is_sumsq ? __builtin_sqrtf(norm[off + i]) : norm[off + i];
+    if (i == 0) med = 0.f;
     __syncthreads();
     if (i < P) {
         int rank = 0;
@@ -526,9 +813,9 @@ __global__ __launch_bounds__(128) void k_clip_scales(const float* __restrict__ n
     __syncthreads();
     if (i < P) {
         const float f = med / (nv[i] + 1e-8f);
-        scale[i] = f > 1.0f ? 1.0f : f;  // clamp(max=1); NaN propagates as in torch.clamp
+        scale[off + i] = f > 1.0f ? 1.0f : f;  // clamp(max=1); NaN propagates as in torch.clamp
     }
-    if (i == 0 && median) *median = med;
+    if (i == 0 && median) median[blockIdx.x] = med;
 }
 
 }  // namespace tplr
@@ -621,9 +908,13 @@ static int check_2d(const void* a, const void* b, int64_t R, int64_t C) {
     return 0;
 }
 
+// chunk rows are addressed with 32-bit byte offsets (63 rows * ld * 4 bytes)
+static inline bool ld_ok(int64_t ld) { return ld > 0 && ld <= (int64_t{1} << 23); }
+
 int tplr_dct2d_fwd(const float* d_x, int64_t R, int64_t C, int64_t ld_x, float* d_coef, void* stream) {
     if (int s = check_2d(d_x, d_coef, R, C)) return s;
     if (ld_x < C) return TPLR_E_BADARG;
+    if (!ld_ok(ld_x)) return TPLR_E_TOOMANY;
     const int64_t n = (R / 64) * (C / 64);
     if (n == 0) return 0;
     hipLaunchKernelGGL(k_dct2d_fwd, dim3(grid8(n)), dim3(64), 0, static_cast<hipStream_t>(stream), d_x, ld_x,
@@ -634,6 +925,7 @@ int tplr_dct2d_fwd(const float* d_x, int64_t R, int64_t C, int64_t ld_x, float* 
 int tplr_dct2d_inv(const float* d_coef, int64_t R, int64_t C, float* d_x, int64_t ld_x, void* stream) {
     if (int s = check_2d(d_x, d_coef, R, C)) return s;
     if (ld_x < C) return TPLR_E_BADARG;
+    if (!ld_ok(ld_x)) return TPLR_E_TOOMANY;
     const int64_t n = (R / 64) * (C / 64);
     if (n == 0) return 0;
     hipLaunchKernelGGL(k_dct2d_inv, dim3(grid8(n)), dim3(64), 0, static_cast<hipStream_t>(stream), d_coef,
@@ -678,55 +970,128 @@ int tplr_topk_pack(const float* d_coef, int64_t n_rows, int64_t row_len, int k, 
     return launch_status();
 }
 
+// persistent grids: one resident set of single-wave workgroups (LDS bounds the residency)
+static int persistent_grid(int64_t total, int waves_per_cu) {
+    static int n_cu = 0;
+    if (n_cu == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            n_cu = v;
+        else
+            n_cu = 256;
+    }
+    int64_t g = static_cast<int64_t>(n_cu) * waves_per_cu;
+    g = (g / 8) * 8;
+    const int64_t need = ((total + 7) / 8) * 8;
+    return static_cast<int>(need < g ? need : g);
+}
+
+static int launch_encode(const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single, int n_tensors,
+                         int64_t total, int k, int use_dct, uint8_t* d_idx12, float* d_val, void* stream) {
+    const dim3 grid(persistent_grid(total, 9)), block(64);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (k > 32) {
+        if (use_dct)
+            hipLaunchKernelGGL((k_encode_topk_pack<true, true>), grid, block, 0, st, d_desc, single, n_tensors, total, k,
+                               d_idx12, d_val);
+        else
+            hipLaunchKernelGGL((k_encode_topk_pack<true, false>), grid, block, 0, st, d_desc, single, n_tensors, total, k,
+                               d_idx12, d_val);
+    } else {
+        if (use_dct)
+            hipLaunchKernelGGL((k_encode_topk_pack<false, true>), grid, block, 0, st, d_desc, single, n_tensors, total, k,
+                               d_idx12, d_val);
+        else
+            hipLaunchKernelGGL((k_encode_topk_pack<false, false>), grid, block, 0, st, d_desc, single, n_tensors, total, k,
+                               d_idx12, d_val);
+    }
+    return launch_status();
+}
+
 int tplr_encode_topk_pack(const float* d_x, int64_t R, int64_t C, int64_t ld_x, int k, int use_dct,
                           uint8_t* d_idx12, float* d_val, void* stream) {
     if (int s = check_2d(d_x, d_val, R, C)) return s;
     if (!d_idx12 || ld_x < C || k < 2 || (k & 1) || k > kCandCap) return TPLR_E_BADARG;
     const int64_t n = (R / 64) * (C / 64);
     if (n == 0) return 0;
-    const dim3 grid(grid8(n)), block(64);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const int64_t X = C / 64;
-    if (k > 32) {
-        if (use_dct)
-            hipLaunchKernelGGL((k_encode_topk_pack<true, true>), grid, block, 0, st, d_x, ld_x, X, n, k, d_idx12, d_val);
-        else
-            hipLaunchKernelGGL((k_encode_topk_pack<true, false>), grid, block, 0, st, d_x, ld_x, X, n, k, d_idx12, d_val);
-    } else {
-        if (use_dct)
-            hipLaunchKernelGGL((k_encode_topk_pack<false, true>), grid, block, 0, st, d_x, ld_x, X, n, k, d_idx12, d_val);
-        else
-            hipLaunchKernelGGL((k_encode_topk_pack<false, false>), grid, block, 0, st, d_x, ld_x, X, n, k, d_idx12, d_val);
-    }
-    return launch_status();
+    if (C / 64 > 0x7fffffff || R / 64 > 0x7fffffff || !ld_ok(ld_x)) return TPLR_E_TOOMANY;
+    tplr_tensor_desc single;
+    single.dense = const_cast<float*>(d_x);
+    single.ld = ld_x;
+    single.chunk_begin = 0;
+    single.x_chunks = static_cast<int32_t>(C / 64);
+    single.y_chunks = static_cast<int32_t>(R / 64);
+    return launch_encode(nullptr, single, 1, n, k, use_dct, d_idx12, d_val, stream);
 }
 
-int tplr_decode_aggregate(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_peer_scale,
-                          int n_peers, int k, int64_t R, int64_t C, int reduce_mode, int normalise, int use_dct,
-                          float* d_out, int64_t ld_out, float* d_sumsq, void* stream) {
-    if (!h_idx12 || !h_val || !d_out || R < 0 || C < 0 || n_peers < 1 || k < 2 || (k & 1) || k > 4096 ||
-        (reduce_mode != TPLR_REDUCE_MEAN && reduce_mode != TPLR_REDUCE_SUM))
+int tplr_encode_topk_pack_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, int k,
+                                int use_dct, uint8_t* d_idx12, float* d_val, void* stream) {
+    if (!d_desc || n_tensors < 1 || total_chunks < 0 || !d_idx12 || !d_val || k < 2 || (k & 1) || k > kCandCap)
         return TPLR_E_BADARG;
-    if ((R % 64) || (C % 64)) return TPLR_E_SHAPE;
-    if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
-    if (use_dct && ld_out < C) return TPLR_E_BADARG;
-    const int64_t n = (R / 64) * (C / 64);
-    if (n == 0) return 0;
+    if (total_chunks == 0) return 0;
+    tplr_tensor_desc none = {};
+    return launch_encode(d_desc, none, n_tensors, total_chunks, k, use_dct, d_idx12, d_val, stream);
+}
+
+static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale, int n_peers,
+                         int k, const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single, int n_tensors,
+                         int64_t total, int reduce_mode, int normalise, int use_dct, float* d_sumsq, void* stream) {
     PeerPtrs pp;
     for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
         pp.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
         pp.val[p] = p < n_peers ? h_val[p] : nullptr;
         if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
     }
-    const dim3 grid(grid8(n)), block(64);
+    const dim3 grid(persistent_grid(total, 7)), block(64);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (use_dct)
-        hipLaunchKernelGGL(k_decode_aggregate<true>, grid, block, 0, st, pp, d_peer_scale, n_peers, k, C / 64, n,
-                           reduce_mode, normalise, d_out, ld_out, d_sumsq);
+        hipLaunchKernelGGL(k_decode_aggregate<true>, grid, block, 0, st, pp, d_scale, n_peers, k, d_desc, single,
+                           n_tensors, total, reduce_mode, normalise, d_sumsq);
     else
-        hipLaunchKernelGGL(k_decode_aggregate<false>, grid, block, 0, st, pp, d_peer_scale, n_peers, k, C / 64, n,
-                           reduce_mode, normalise, d_out, ld_out, d_sumsq);
+        hipLaunchKernelGGL(k_decode_aggregate<false>, grid, block, 0, st, pp, d_scale, n_peers, k, d_desc, single,
+                           n_tensors, total, reduce_mode, normalise, d_sumsq);
     return launch_status();
+}
+
+static int check_decode(const void* a, const void* b, int n_peers, int k, int reduce_mode) {
+    if (!a || !b || n_peers < 1 || k < 2 || (k & 1) || k > 4096 ||
+        (reduce_mode != TPLR_REDUCE_MEAN && reduce_mode != TPLR_REDUCE_SUM))
+        return TPLR_E_BADARG;
+    if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
+    return 0;
+}
+
+int tplr_decode_aggregate(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_peer_scale,
+                          int n_peers, int k, int64_t R, int64_t C, int reduce_mode, int normalise, int use_dct,
+                          float* d_out, int64_t ld_out, float* d_sumsq, void* stream) {
+    if (int s = check_decode(h_idx12, h_val, n_peers, k, reduce_mode)) return s;
+    if (!d_out || R < 0 || C < 0) return TPLR_E_BADARG;
+    if ((R % 64) || (C % 64)) return TPLR_E_SHAPE;
+    if (use_dct && ld_out < C) return TPLR_E_BADARG;
+    const int64_t n = (R / 64) * (C / 64);
+    if (n == 0) return 0;
+    if (C / 64 > 0x7fffffff || R / 64 > 0x7fffffff || (use_dct && !ld_ok(ld_out))) return TPLR_E_TOOMANY;
+    tplr_tensor_desc single;
+    single.dense = d_out;
+    single.ld = ld_out;
+    single.chunk_begin = 0;
+    single.x_chunks = static_cast<int32_t>(C / 64);
+    single.y_chunks = static_cast<int32_t>(R / 64);
+    return launch_decode(h_idx12, h_val, d_peer_scale, n_peers, k, nullptr, single, 1, n, reduce_mode, normalise,
+                         use_dct, d_sumsq, stream);
+}
+
+int tplr_decode_aggregate_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale,
+                                int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
+                                int64_t total_chunks, int reduce_mode, int normalise, int use_dct, float* d_sumsq,
+                                void* stream) {
+    if (int s = check_decode(h_idx12, h_val, n_peers, k, reduce_mode)) return s;
+    if (!d_desc || n_tensors < 1 || total_chunks < 0) return TPLR_E_BADARG;
+    if (total_chunks == 0) return 0;
+    tplr_tensor_desc none = {};
+    return launch_decode(h_idx12, h_val, d_scale, n_peers, k, d_desc, none, n_tensors, total_chunks, reduce_mode,
+                         normalise, use_dct, d_sumsq, stream);
 }
 
 int tplr_scatter_rows(const uint8_t* d_idx12, const int64_t* d_idx64, const float* d_val, int64_t n_rows,
@@ -759,10 +1124,29 @@ int tplr_peer_sumsq(const float* const* h_val, int n_peers, int64_t n, float* d_
 
 int tplr_clip_scales(const float* d_norm, int n_peers, int is_sumsq, float* d_scale, float* d_median,
                      void* stream) {
-    if (!d_norm || !d_scale || n_peers < 1) return TPLR_E_BADARG;
+    return tplr_clip_scales_batch(d_norm, 1, n_peers, is_sumsq, d_scale, d_median, stream);
+}
+
+int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int is_sumsq, float* d_scale,
+                           float* d_median, void* stream) {
+    if (!d_norm || !d_scale || n_peers < 1 || n_tensors < 1) return TPLR_E_BADARG;
     if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
-    hipLaunchKernelGGL(k_clip_scales, dim3(1), dim3(128), 0, static_cast<hipStream_t>(stream), d_norm, n_peers,
+    hipLaunchKernelGGL(k_clip_scales, dim3(n_tensors), dim3(128), 0, static_cast<hipStream_t>(stream), d_norm, n_peers,
                        is_sumsq, d_scale, d_median);
+    return launch_status();
+}
+
+int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
+                       float* d_sumsq, void* stream) {
+    if (!h_val || !d_desc || !d_sumsq || n_peers < 1 || n_tensors < 1 || k < 1) return TPLR_E_BADARG;
+    if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
+    ValPtrs vp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        vp.val[p] = p < n_peers ? h_val[p] : nullptr;
+        if (p < n_peers && !vp.val[p]) return TPLR_E_BADARG;
+    }
+    hipLaunchKernelGGL(k_segment_sumsq, dim3(static_cast<unsigned>(n_tensors) * n_peers), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), vp, n_peers, k, d_desc, d_sumsq);
     return launch_status();
 }
 

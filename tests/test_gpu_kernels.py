@@ -413,3 +413,80 @@ def test_bad_arguments_are_rejected(dev):
     assert lib.tplr_pack12(tc._ptr(o), 3, tc._ptr(b), None, None) == _lib.TPLR_E_ODD
     assert lib.tplr_encode_topk_pack(tc._ptr(x), 64, 64, 32, 32, 1, tc._ptr(b), tc._ptr(o), None) == _lib.TPLR_E_BADARG
     assert b"even" in lib.tplr_status_string(_lib.TPLR_E_ODD)
+
+
+# ---------------------------------------------------------------- persistent loops and batches
+def test_persistent_encode_many_chunks_per_wave(dev):
+    # 4608 chunks: more than one resident set of waves, so every wave walks several chunks
+    x = t3((4608, 4096), 2024, row_scale=True).to(dev)
+    idx_f, val_f, xshape, _ = tc.encode_compress(x, 32)
+    tr = tc.ChunkingTransformer(_Stub([x]), 64)
+    coef = tr.encode(x, use_dct=True)
+    idx_u, val_u = tc._topk_rows(coef.reshape(-1, 4096), 32)
+    assert torch.equal(idx_f, idx_u) and torch.equal(val_f.reshape(-1, 32), val_u)
+    # spot-check chunks against the oracle's selection on the device coefficients
+    rows = coef.reshape(-1, 4096)[::97].cpu().numpy()
+    want_i, want_v = orc.topk_rows(rows, 32)
+    got = orc.unpack12(idx_f.cpu().numpy(), (72 * 64, 32))[::97]
+    assert np.array_equal(got, want_i)
+    assert np.array_equal(val_f.reshape(-1, 32)[::97].cpu().numpy(), want_v)
+    # and the decode side over the same number of chunks
+    full = tc.batch_decompress_decode([idx_f], [val_f], xshape, clip_norm=False)
+    dense = tc.TopKCompressor().decompress(x, idx_f, val_f, xshape, 4096)
+    assert torch.equal(full, tr.decode(dense, use_dct=True))
+
+
+def test_batch_encode_and_aggregate_match_per_tensor(dev):
+    shapes = [(128, 192), (64, 64), (512, 1024), (1536, 2048), (64, 3072), (2048, 64)]
+    k, P = 32, 4
+    grads = [t3(s, 500 + i, row_scale=True).to(dev) for i, s in enumerate(shapes)]
+    batch = tc.TensorBatch(grads)
+    assert batch.total_chunks == sum((a // 64) * (b // 64) for a, b in shapes)
+    idx12, val = tc.encode_compress_batch(batch, k)
+    for i, g in enumerate(grads):
+        want_i, want_v, xshape, _ = tc.encode_compress(g, k)
+        got_i, got_v = batch.payload_slice(i, idx12, val, k)
+        assert torch.equal(got_i, want_i) and torch.equal(got_v, want_v) and tuple(xshape) == batch.xshape(i)
+    # P peers with flat payloads
+    pay = []
+    for p in range(P):
+        pg = [0.5 * g + t3(tuple(g.shape), 9000 + 10 * p + i, row_scale=True).to(dev) * (1 + p)
+              for i, g in enumerate(grads)]
+        pay.append(tc.encode_compress_batch(tc.TensorBatch(pg), k))
+    idxs, vals = [a for a, _ in pay], [b for _, b in pay]
+    scale = tc.peer_clip_scales_batch(batch, vals, k)
+    assert scale.shape == (len(shapes), P)
+    for i in range(len(shapes)):
+        norms = np.array([np.sqrt((batch.payload_slice(i, idxs[p], vals[p], k)[1].double() ** 2).sum().item())
+                          for p in range(P)], np.float32)
+        _, want = orc.clip_scales(norms)
+        assert np.allclose(scale[i].cpu().numpy(), want, rtol=2e-6)
+    outs = [torch.full(s, float("nan"), device=dev) for s in shapes]
+    ss = torch.zeros(batch.total_chunks, device=dev)
+    tc.batch_decompress_decode_batch(tc.TensorBatch(outs), idxs, vals, k, scale=scale, sumsq=ss)
+    for i, o in enumerate(outs):
+        sl = [batch.payload_slice(i, idxs[p], vals[p], k) for p in range(P)]
+        y, x = batch.xshape(i)[:2]
+        want = tc._aggregate_chunks([a.contiguous() for a, _ in sl], [b.contiguous() for _, b in sl],
+                                    scale[i].contiguous(), y, x, k, normalise=False, use_dct=True)
+        assert torch.equal(o, want)
+        b0 = batch.offsets[i]
+        per_chunk = (want.reshape(y, 64, x, 64).double() ** 2).sum((1, 3)).reshape(-1)
+        assert torch.allclose(ss[b0:b0 + y * x].double(), per_chunk, rtol=1e-4)
+    # dense-coefficient output of the batch kernel (no inverse transform)
+    couts = [torch.empty(batch.xshape(i), device=dev) for i in range(len(shapes))]
+    cb = tc.TensorBatch.__new__(tc.TensorBatch)
+    # coefficient tensors are (Y, X, 64, 64): describe them by hand as contiguous chunk lists
+    import numpy as _np
+    desc = _np.zeros(len(shapes), dtype=_np.dtype([("dense", "<u8"), ("ld", "<i8"), ("chunk_begin", "<i8"),
+                                                   ("x_chunks", "<i4"), ("y_chunks", "<i4")]))
+    for i, c in enumerate(couts):
+        desc[i] = (c.data_ptr(), 0, batch.offsets[i], c.shape[1], c.shape[0])
+    cb.tensors, cb.total_chunks, cb.device, cb.offsets = couts, batch.total_chunks, dev, batch.offsets
+    cb.table = torch.from_numpy(desc.view(_np.uint8).copy()).to(dev)
+    tc.batch_decompress_decode_batch(cb, idxs, vals, k, scale=scale, use_dct=False)
+    for i, c in enumerate(couts):
+        sl = [batch.payload_slice(i, idxs[p], vals[p], k) for p in range(P)]
+        want = orc.batch_decompress([a.cpu().numpy() for a, _ in sl], [b.cpu().numpy() for _, b in sl],
+                                    batch.xshape(i), 4096, clip_norm=False)  # unclipped reference for the pattern
+        assert np.array_equal(c.cpu().numpy() != 0, want != 0)
