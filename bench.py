@@ -6,10 +6,12 @@ Workload (BASELINE.json configs[2] and configs[3]): the LLaMA-style 1B gradient 
 294 144 chunks of 64x64, plus 33 norm vectors), synthetic Student-t(df=3) x 1e-3 gradients
 with log-normal row scales, chunk 64, top-k 32.
 
-  step       = one encode + top-k + pack pass over the whole set (fused kernel per tensor)
+  step       = one encode + top-k + pack pass over the whole set (one fused launch for all
+               2-D tensors, one transform + one select launch for the norm vectors)
   value      = algorithmic bytes of that pass / time, in GB/s (inputs resident in HBM)
-  aggregate  = one 15-peer decode-aggregate pass over the same shapes (clip factors, fused
-               unpack + scatter-mean + inverse DCT per tensor), reported as ms and GB/s
+  aggregate  = one 15-peer decode-aggregate pass over the same shapes (per-tensor, per-peer
+               norms and clip factors, then one fused unpack + scatter-mean + inverse DCT launch),
+               reported as ms and GB/s
   roofline   = the same figures against the 8 TB/s HBM peak, per kernel, from HIP events on
                the launch stream
   cpu_baseline = the reference's op sequence in torch on the host cores (oracle port), timed
@@ -39,6 +41,8 @@ def parse():
     ap.add_argument("--workload", default="cfg3_llama1b", help="cfg1_2048x2048 | cfg2_llama150m | cfg3_llama1b | cfg5_72b_block")
     ap.add_argument("--peers", type=int, default=15)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--profile", choices=["encode", "aggregate"], default=None,
+                    help="run only that phase's batched launches --steps times (for rocprofv3) and print nothing")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline sample")
     return ap.parse_args()
 
@@ -148,44 +152,72 @@ def main():
     grads = workloads.gradient_set(args.workload, device=dev)
     two_d = [g for g in grads if g.dim() == 2]
     one_d = [g for g in grads if g.dim() == 1]
+    batch = tc.TensorBatch(two_d)
+    n_chunks = batch.total_chunks
+    idx_buf = torch.empty(n_chunks * (k // 2) * 3, dtype=torch.uint8, device=dev)
+    val_buf = torch.empty((n_chunks, k), dtype=torch.float32, device=dev)
+    # the norm vectors (64-element chunks) as one flat tensor: one transform + one select launch
+    flat_1d = torch.cat(one_d) if one_d else None
+
+    def encode2d_only():
+        tc.encode_compress_batch(batch, k, use_dct=True, idx12=idx_buf, val=val_buf)
 
     def encode_pass():
-        out = [tc.encode_compress(g, k, use_dct=True) for g in two_d]
-        for g in one_d:
-            out.append(comp.compress(tr.encode(g, use_dct=True), k))
-        return out
+        encode2d_only()
+        if flat_1d is not None:
+            comp.compress(tr.encode(flat_1d, use_dct=True), k)
 
-    enc_ms, enc_wall = event_ms(encode_pass, args.steps, args.warmup)
-    enc_bytes = workloads.encode_bytes(shapes, k)
-    # kernel-only figure for the fused 2-D kernel (the dominant one)
-    def encode2d_only():
+    def encode_per_tensor():
         for g in two_d:
             tc.encode_compress(g, k, use_dct=True)
-    enc2d_ms, _ = event_ms(encode2d_only, args.steps, 1)
-    enc2d_bytes = workloads.chunks_2d(shapes) * (16384 + 11 * k // 2)
 
-    # ---- P peers' payloads for the aggregation side (peer p = 0.5 shared + own)
-    payloads = []  # per tensor: (idxs[P], vals[P], xshape)
-    for j, g in enumerate(two_d):
-        idxs, vals = [], []
-        for p in range(P):
-            own = workloads.student_t3(tuple(g.shape), 1000 * (p + 1) + j, row_scale=True, device=dev)
-            own.add_(g, alpha=0.5)
-            i12, v, xshape, _ = tc.encode_compress(own, k, use_dct=True)
-            idxs.append(i12)
-            vals.append(v)
-            del own
-        payloads.append((idxs, vals, xshape))
-    del grads, two_d
-    torch.cuda.empty_cache()
-    outs = [torch.empty(xs[0] * 64, xs[1] * 64, device=dev) for _, _, xs in payloads]
+    if flat_1d is not None:
+        tr.shape_dict[flat_1d.shape[0]] = 64
+    if args.profile == "encode":
+        event_ms(encode2d_only, args.steps, args.warmup)
+        return
+    if args.profile is None:
+        enc_ms, enc_wall = event_ms(encode_pass, args.steps, args.warmup)
+    enc_bytes = workloads.encode_bytes(shapes, k)
+    if args.profile is None:
+        enc2d_ms, _ = event_ms(encode2d_only, args.steps, 1)      # the fused 2-D kernel alone (dominant)
+        enc_pt_ms, _ = event_ms(encode_per_tensor, max(3, args.steps // 2), 1)
+    enc2d_bytes = n_chunks * (16384 + 11 * k // 2)
+
+    # ---- P peers' flat payloads for the aggregation side (peer p = 0.5 shared + own)
+    idxs, vals = [], []
+    for p in range(P):
+        own = [workloads.student_t3(tuple(g.shape), 1000 * (p + 1) + j, row_scale=True, device=dev).add_(g, alpha=0.5)
+               for j, g in enumerate(two_d)]
+        i12, v = tc.encode_compress_batch(tc.TensorBatch(own), k, use_dct=True)
+        torch.cuda.synchronize()
+        idxs.append(i12)
+        vals.append(v)
+        del own
+    outs = two_d  # the gradients are not needed any more: decode into their storage
+    out_batch = batch
 
     def aggregate_pass():
-        for (idxs, vals, xshape), out in zip(payloads, outs):
-            tc.batch_decompress_decode(idxs, vals, xshape, clip_norm=True, use_dct=True, out=out)
+        tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, clip_norm=True, use_dct=True)
 
-    agg_ms, agg_wall = event_ms(aggregate_pass, max(3, args.steps // 2), 2)
-    agg_bytes = workloads.chunks_2d(shapes) * (P * 11 * k // 2 + 16384)
+    scale = tc.peer_clip_scales_batch(out_batch, vals, k)
+
+    def aggregate_kernel_only():
+        tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, scale=scale, use_dct=True)
+
+    def aggregate_per_tensor():
+        for i in range(len(out_batch)):
+            sl = [out_batch.payload_slice(i, idxs[p], vals[p], k) for p in range(P)]
+            tc.batch_decompress_decode([a for a, _ in sl], [b for _, b in sl], out_batch.xshape(i), out=outs[i])
+
+    if args.profile == "aggregate":
+        event_ms(aggregate_pass, args.steps, args.warmup)
+        return
+    agg_steps = max(3, args.steps // 2)
+    agg_ms, agg_wall = event_ms(aggregate_pass, agg_steps, 2)
+    aggk_ms, _ = event_ms(aggregate_kernel_only, agg_steps, 1)
+    agg_pt_ms, _ = event_ms(aggregate_per_tensor, 3, 1)
+    agg_bytes = n_chunks * (P * 11 * k // 2 + 16384)
 
     result = {
         "metric": "encode+topk+pack GB/s and 15-peer decode-aggregate ms, 1B grads, 1 GPU",
@@ -207,17 +239,19 @@ def main():
         "aggregate_ms": round(agg_ms, 4),
         "aggregate_GBps": round(agg_bytes / (agg_ms * 1e-3) / 1e9, 2),
         "aggregate_wall_ms": round(agg_wall, 4),
+        "per_tensor_launches": {"encode_ms": round(enc_pt_ms, 4), "aggregate_ms": round(agg_pt_ms, 4),
+                                "note": "same work as one fused launch per tensor through the reference-shaped API"},
         "roofline": {
             "bound": "hbm", "kernel": "k_encode_topk_pack",
             "achieved": round(enc2d_bytes / (enc2d_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(enc2d_bytes / (enc2d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
-            "launches_per_step": len(payloads), "bytes_per_step": enc2d_bytes, "ms_per_step": round(enc2d_ms, 4),
+            "launches_per_step": 1, "bytes_per_launch": enc2d_bytes, "ms_per_launch": round(enc2d_ms, 4),
         },
         "roofline_aggregate": {
             "bound": "hbm", "kernel": "k_decode_aggregate",
-            "achieved": round(agg_bytes / (agg_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(agg_bytes / (agg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
-            "launches_per_step": len(payloads), "bytes_per_step": agg_bytes,
+            "achieved": round(agg_bytes / (aggk_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(agg_bytes / (aggk_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+            "launches_per_step": 1, "bytes_per_launch": agg_bytes, "ms_per_launch": round(aggk_ms, 4),
         },
     }
     if not args.no_cpu_baseline:

@@ -832,6 +832,34 @@ static inline int launch_status() {
 
 static inline unsigned grid8(int64_t n) { return static_cast<unsigned>(((n + 7) / 8) * 8); }
 
+// persistent grids: exactly one resident set of single-wave workgroups, as the occupancy
+// calculator reports it for the kernel at hand (registers or LDS bound it); a larger grid
+// would leave a second, mostly empty round
+template <typename Kernel>
+static int persistent_grid(Kernel kernel, int64_t total) {
+    int n_cu = 256, per_cu = 0, dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+        n_cu = v;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 64, 0) != hipSuccess || per_cu < 1) per_cu = 4;
+    int64_t g = static_cast<int64_t>(n_cu) * per_cu;
+    g = g < 8 ? 8 : (g / 8) * 8;
+    const int64_t need = ((total + 7) / 8) * 8;
+    return static_cast<int>(need < g ? need : g);
+}
+
+template <typename Kernel>
+static int launch_encode_as(Kernel kernel, const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single,
+                            int n_tensors, int64_t total, int k, uint8_t* d_idx12, float* d_val, void* stream) {
+    static int resident = 0;  // per kernel variant
+    if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
+    const int64_t need = ((total + 7) / 8) * 8;
+    const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
+    hipLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), d_desc, single, n_tensors, total, k,
+                       d_idx12, d_val);
+    return launch_status();
+}
+
 extern "C" {
 
 int tplr_version(void) { return 100; }
@@ -970,43 +998,16 @@ int tplr_topk_pack(const float* d_coef, int64_t n_rows, int64_t row_len, int k, 
     return launch_status();
 }
 
-// persistent grids: one resident set of single-wave workgroups (LDS bounds the residency)
-static int persistent_grid(int64_t total, int waves_per_cu) {
-    static int n_cu = 0;
-    if (n_cu == 0) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-            n_cu = v;
-        else
-            n_cu = 256;
-    }
-    int64_t g = static_cast<int64_t>(n_cu) * waves_per_cu;
-    g = (g / 8) * 8;
-    const int64_t need = ((total + 7) / 8) * 8;
-    return static_cast<int>(need < g ? need : g);
-}
-
 static int launch_encode(const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single, int n_tensors,
                          int64_t total, int k, int use_dct, uint8_t* d_idx12, float* d_val, void* stream) {
-    const dim3 grid(persistent_grid(total, 9)), block(64);
-    hipStream_t st = static_cast<hipStream_t>(stream);
     if (k > 32) {
         if (use_dct)
-            hipLaunchKernelGGL((k_encode_topk_pack<true, true>), grid, block, 0, st, d_desc, single, n_tensors, total, k,
-                               d_idx12, d_val);
-        else
-            hipLaunchKernelGGL((k_encode_topk_pack<true, false>), grid, block, 0, st, d_desc, single, n_tensors, total, k,
-                               d_idx12, d_val);
-    } else {
-        if (use_dct)
-            hipLaunchKernelGGL((k_encode_topk_pack<false, true>), grid, block, 0, st, d_desc, single, n_tensors, total, k,
-                               d_idx12, d_val);
-        else
-            hipLaunchKernelGGL((k_encode_topk_pack<false, false>), grid, block, 0, st, d_desc, single, n_tensors, total, k,
-                               d_idx12, d_val);
+            return launch_encode_as(k_encode_topk_pack<true, true>, d_desc, single, n_tensors, total, k, d_idx12, d_val, stream);
+        return launch_encode_as(k_encode_topk_pack<true, false>, d_desc, single, n_tensors, total, k, d_idx12, d_val, stream);
     }
-    return launch_status();
+    if (use_dct)
+        return launch_encode_as(k_encode_topk_pack<false, true>, d_desc, single, n_tensors, total, k, d_idx12, d_val, stream);
+    return launch_encode_as(k_encode_topk_pack<false, false>, d_desc, single, n_tensors, total, k, d_idx12, d_val, stream);
 }
 
 int tplr_encode_topk_pack(const float* d_x, int64_t R, int64_t C, int64_t ld_x, int k, int use_dct,
@@ -1043,7 +1044,13 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
         pp.val[p] = p < n_peers ? h_val[p] : nullptr;
         if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
     }
-    const dim3 grid(persistent_grid(total, 7)), block(64);
+    static int resident[2] = {0, 0};
+    const int which = use_dct ? 1 : 0;
+    if (resident[which] == 0)
+        resident[which] = use_dct ? persistent_grid(k_decode_aggregate<true>, int64_t{1} << 40)
+                                  : persistent_grid(k_decode_aggregate<false>, int64_t{1} << 40);
+    const int64_t need = ((total + 7) / 8) * 8;
+    const dim3 grid(static_cast<unsigned>(need < resident[which] ? need : resident[which])), block(64);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (use_dct)
         hipLaunchKernelGGL(k_decode_aggregate<true>, grid, block, 0, st, pp, d_scale, n_peers, k, d_desc, single,
