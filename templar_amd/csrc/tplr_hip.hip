@@ -378,7 +378,7 @@ __global__ __launch_bounds__(64) void k_topk_rows(const float* __restrict__ coef
 // Persistent fused encode: every wave walks its slice of the chunk list; the 64 row loads of
 // the next chunk are in flight while the current one is transformed and selected.
 template <bool kTwo, bool kUseDct>
-__global__ __launch_bounds__(64) void k_encode_topk_pack(const tplr_tensor_desc* __restrict__ table,
+__global__ __launch_bounds__(64, 2) void k_encode_topk_pack(const tplr_tensor_desc* __restrict__ table,
                                                          const tplr_tensor_desc single, int n_tensors,
                                                          int64_t total, int k, uint8_t* __restrict__ idx12,
                                                          float* __restrict__ val) {
@@ -437,131 +437,76 @@ __device__ __forceinline__ uint32_t load_idx12(BytePtr row, int j) {
     return (j & 1) ? (w >> 4) : (w & 0xfffu);
 }
 
-// Up to 64 peers keep their (index, value) base pointers in the padding columns of the tile
-// (16 bytes per tile row); beyond that they are read from the kernel arguments.
-struct PeerTable {
-    const PeerPtrs* pp;
-    float* tile;
-    bool in_lds;
-    __device__ __forceinline__ void get(int p, const gbyte*& ip, const gfloat*& vp) const {
-        if (in_lds) {
-            const uint64_t* slot = reinterpret_cast<const uint64_t*>(tile + p * kLd + kChunk);
-            ip = (const gbyte*)slot[0];
-            vp = (const gfloat*)slot[1];
-        } else {
-            ip = (const gbyte*)pp->idx[p];
-            vp = (const gfloat*)pp->val[p];
-        }
-    }
-};
-
-constexpr int kUnitRegs = 16;  // wave-wide batches of one chunk's entries that stay in registers
-
-struct UnitRegs {
-    uint32_t ix[kUnitRegs];
-    float a[kUnitRegs];
-    uint32_t ok;  // bit i: unit i holds an entry for this lane
-};
-
 typedef uint16_t __attribute__((aligned(1))) unaligned_u16;
 using gu16 = __attribute__((address_space(1))) unaligned_u16;
 
-// 12-bit index j of a packed row: the two bytes that hold it, as one unaligned 16-bit load
-__device__ __forceinline__ uint32_t load_idx12_g(const gbyte* row, int j) {
-    const uint32_t w = *(const gu16*)(row + 3 * (j >> 1) + (j & 1));
-    return (j & 1) ? (w >> 4) : (w & 0xfffu);
-}
+constexpr int kCntWords = 1024;  // 4096 one-byte contribution counters
 
-// Persistent fused decode: per chunk, the peers' entries are accumulated in peer order into an
-// LDS tile (sum) and a byte-per-coefficient contribution count, touched coefficients are
-// divided by their count, and the tile goes through the inverse 2-D DCT.  Because loads and
-// stores complete out of order with respect to each other on one counter, the 64 row stores of
-// chunk g are issued at the top of iteration g + 1, right after the wait for that chunk's
-// payload registers; the payload of chunk g + 1 is requested once chunk g's entries are in the
-// tile and travels during its inverse transform.
-template <bool kUseDct>
-__global__ __launch_bounds__(64) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
-                                                         int k, const tplr_tensor_desc* __restrict__ table,
-                                                         const tplr_tensor_desc single, int n_tensors, int64_t total,
-                                                         int reduce_mode, int normalise,
-                                                         float* __restrict__ sumsq) {
+// Persistent fused decode.  Per chunk, the peers' entries are accumulated in peer order into an
+// LDS tile (sums) and a byte-per-coefficient contribution count; touched coefficients are
+// divided by their count; the tile goes through the inverse 2-D DCT.
+//
+// Fast path (kUnits > 0: k <= 64 and at most kUnits peers): lane j handles entry j of every
+// peer, so each address is a scalar base (peer pointer from the kernel arguments + chunk
+// offset) plus one lane-constant offset and each clip factor is a scalar; the whole payload of
+// a chunk sits in 2 * kUnits registers, is requested before the inverse transform of the
+// previous chunk and travels during it.  The scatter is straight-line: unused units (peer
+// index >= P) add 0 to a per-lane dummy slot in the tile's padding instead of branching.
+// Generic path (kUnits == 0): any k and peer count, entries loaded where they are used.
+//
+// Loads and stores complete out of order with respect to each other on one counter, so the 64
+// row stores of chunk g are issued at the top of iteration g + 1, after the wait for that
+// chunk's payload registers and a whole iteration before the next wait.
+template <bool kUseDct, int kUnits>
+__global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
+                                                            int k, const tplr_tensor_desc* __restrict__ table,
+                                                            const tplr_tensor_desc single, int n_tensors,
+                                                            int64_t total, int reduce_mode, int normalise,
+                                                            float* __restrict__ sumsq) {
     __shared__ __align__(16) float tile[kTileFloats];
-    __shared__ __align__(16) uint32_t cnt[1024];  // 4096 one-byte contribution counters
+    __shared__ __align__(16) uint32_t cnt[kCntWords];
+    constexpr bool kFast = kUnits > 0;
+    constexpr int kRegs = kFast ? kUnits : 1;
     const int lane = threadIdx.x;
     int64_t g0, g1;
     my_range(total, g0, g1);
     if (g0 >= g1) return;
 
-    PeerTable pt{&pp, tile, P <= 64};
-    if (pt.in_lds && lane < P) {
-        uint64_t* slot = reinterpret_cast<uint64_t*>(tile + lane * kLd + kChunk);
-        slot[0] = reinterpret_cast<uint64_t>(pp.idx[lane]);
-        slot[1] = reinterpret_cast<uint64_t>(pp.val[lane]);
-    }
-    wave_lds_fence();
-
-    // A "unit" is one wave-wide batch of entries of a chunk: for k <= 64 it covers G = 64 / k
-    // whole peers (lane -> peer g_lane, entry j_lane), for k > 64 one 64-entry slice of one
-    // peer.  Peers are applied strictly in order (gq loop in apply_unit).
-    const int G = k >= 64 ? 1 : 64 / k;
-    const int S = (k + 63) >> 6;
-    const int g_lane = k >= 64 ? 0 : lane / k;
-    const int j_lane = k >= 64 ? lane : lane - g_lane * k;
-    const int n_units = k >= 64 ? P * S : (P + G - 1) / G;
     const int64_t idx_stride = k + (k >> 1);
+    const int lane_ioff = 3 * (lane >> 1) + (lane & 1);  // byte offset of entry `lane` in a packed row
+    const bool lane_on = lane < k;                       // fast path: this lane owns an entry
+    const int dummy_pos = lane * kLd + kChunk;           // per-lane padding slot
 
-    auto entry = [&](int u, int& p, int& j) -> bool {
-        if (k >= 64) {
-            p = u / S;
-            j = (u - p * S) * 64 + lane;
-            return j < k;
-        }
-        p = u * G + g_lane;
-        j = j_lane;
-        return g_lane < G && p < P;
-    };
+    uint32_t ix[kRegs];
+    float a[kRegs], sc[kRegs];
 
-    auto load_units = [&](UnitRegs& r, int64_t g, int t) {
-        r.ok = 0;
+    auto load_payload = [&](int64_t g, int t) {  // fast path only
 #pragma unroll
-        for (int i = 0; i < kUnitRegs; ++i) {
-            int p, j;
-            r.ix[i] = 0;
-            r.a[i] = 0.f;
-            if (i < n_units && entry(i, p, j)) {
-                r.ok |= 1u << i;
-                const gbyte* ip;
-                const gfloat* vp;
-                pt.get(p, ip, vp);
-                r.ix[i] = load_idx12_g(ip + g * idx_stride, j);
-                r.a[i] = vp[g * k + j];
-                if (scale) r.a[i] *= scale[static_cast<int64_t>(t) * P + p];
+        for (int i = 0; i < kRegs; ++i) {
+            const int p = i < P ? i : P - 1;  // unused units read the last peer and are masked later
+            const gbyte* irow = (const gbyte*)pp.idx[p] + g * idx_stride;  // wave-uniform
+            const gfloat* vrow = (const gfloat*)pp.val[p] + g * k;
+            sc[i] = scale ? scale[static_cast<int64_t>(t) * P + p] : 1.0f;
+            ix[i] = 0;
+            a[i] = 0.f;
+            if (lane_on) {
+                ix[i] = *(const gu16*)(irow + lane_ioff);
+                a[i] = vrow[lane];
             }
         }
     };
-
-    bool collide = false;
-    auto apply_one = [&](uint32_t ix, float a) {
-        atomicAdd(&tile[tile_pos(ix)], a);
-        const uint32_t sh = (ix & 3) * 8;
-        const uint32_t old = atomicAdd(&cnt[ix >> 2], 1u << sh);
-        collide |= ((old >> sh) & 0xffu) != 0;
-    };
-    auto claim_divide = [&](uint32_t ix) {
-        // exactly one entry per destination claims the counter and divides the sum
-        const uint32_t sh = (ix & 3) * 8;
-        const uint32_t old = atomicAnd(&cnt[ix >> 2], ~(0xffu << sh));
-        const uint32_t n = (old >> sh) & 0xffu;
-        if (n > 1) {
-            float* t = &tile[tile_pos(ix)];
-            *t = *t / static_cast<float>(n);
-        }
+    // entry j of peer p of chunk g (generic path and normalise)
+    auto load_entry = [&](int p, int j, int64_t g, uint32_t& ixo, float& ao) {
+        const gbyte* irow = (const gbyte*)pp.idx[p] + g * idx_stride;
+        const uint32_t w = *(const gu16*)(irow + (3 * (j >> 1) + (j & 1)));
+        ixo = (j & 1) ? (w >> 4) : (w & 0xfffu);
+        ao = ((const gfloat*)pp.val[p] + g * k)[j];
     };
 
     Cursor c;
     cursor_seek(c, table, single, n_tensors, g0);
-    UnitRegs cur;
-    if (!normalise) load_units(cur, g0, c.t);
+    const bool fast = kFast && !normalise;
+    if (fast) load_payload(g0, c.t);
 
     float v[64];  // inverse transform of the previous chunk, stored one iteration late
     gfloat* prev_chunk0 = nullptr;
@@ -569,6 +514,12 @@ __global__ __launch_bounds__(64) void k_decode_aggregate(const PeerPtrs pp, cons
     float prev_ss = 0.f;
 
     for (int64_t g = g0; g < g1; ++g) {
+        // the payload registers must have arrived BEFORE the previous chunk's stores are issued:
+        // a later wait for them would also wait for those stores
+        if (kFast) {
+#pragma unroll
+            for (int i = 0; i < kRegs; ++i) asm volatile("" : "+v"(ix[i]), "+v"(a[i]));
+        }
         if (g > g0) {
             if (kUseDct)
                 store_chunk_rows(v, (void*)prev_chunk0, prev_ld, lane);
@@ -585,7 +536,7 @@ __global__ __launch_bounds__(64) void k_decode_aggregate(const PeerPtrs pp, cons
 
         {
             const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-            float4* row = reinterpret_cast<float4*>(tile + lane * kLd);  // data columns only
+            float4* row = reinterpret_cast<float4*>(tile + lane * kLd);
 #pragma unroll
             for (int q = 0; q < 16; ++q) row[q] = z;
             const uint4 zi = make_uint4(0, 0, 0, 0);
@@ -593,73 +544,89 @@ __global__ __launch_bounds__(64) void k_decode_aggregate(const PeerPtrs pp, cons
             for (int q = 0; q < 4; ++q) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
         }
         wave_lds_fence();
-        collide = false;
 
-        if (normalise) {
+        // ---- scatter: sums in peer order, contribution counts; `seen` collects the old counts
+        uint32_t seen = 0;
+        auto add_entry = [&](uint32_t ixe, float val) {
+            atomicAdd(&tile[tile_pos(ixe)], val);
+            const uint32_t sh = (ixe & 3) * 8;
+            seen |= (atomicAdd(&cnt[ixe >> 2], 1u << sh) >> sh) & 0xffu;
+        };
+        if (fast) {
+            if (lane_on) {
+                uint32_t old[kRegs];
+#pragma unroll
+                for (int i = 0; i < kRegs; ++i) {
+                    const bool on = i < P;  // wave-uniform
+                    const uint32_t e = (lane & 1) ? (ix[i] >> 4) : (ix[i] & 0xfffu);
+                    ix[i] = e;  // decoded index, kept for the mean pass
+                    const uint32_t sh = (e & 3) * 8;
+                    atomicAdd(&tile[on ? tile_pos(e) : dummy_pos], on ? a[i] * sc[i] : 0.f);
+                    old[i] = (atomicAdd(&cnt[on ? (e >> 2) : lane], on ? (1u << sh) : 0u) >> sh) & (on ? 0xffu : 0u);
+                }
+#pragma unroll
+                for (int i = 0; i < kRegs; ++i) seen |= old[i];
+            }
+        } else if (normalise) {
             // per-peer, per-chunk L2 normalisation (compress.py:541-545); simple, unbatched
             for (int p = 0; p < P; ++p) {
-                const gbyte* ip;
-                const gfloat* vp;
-                pt.get(p, ip, vp);
+                const gfloat* vrow = (const gfloat*)pp.val[p] + g * k;
                 float ss = 0.f;
-                for (int j = lane; j < k; j += 64) {
-                    const float a = vp[g * k + j];
-                    ss += a * a;
-                }
+                for (int j = lane; j < k; j += 64) ss += vrow[j] * vrow[j];
                 const float nrm = __builtin_sqrtf(wave_sum_f32(ss)) + 1e-8f;
-                for (int j0 = 0; j0 < k; j0 += 64) {
-                    const int j = j0 + lane;
-                    if (j < k) apply_one(load_idx12_g(ip + g * idx_stride, j), vp[g * k + j] / nrm);
+                for (int j = lane; j < k; j += 64) {
+                    uint32_t ixe;
+                    float ae;
+                    load_entry(p, j, g, ixe, ae);
+                    add_entry(ixe, ae / nrm);
                 }
             }
         } else {
-#pragma unroll
-            for (int i = 0; i < kUnitRegs; ++i) {
-                if (i < n_units) {
-                    for (int gq = 0; gq < G; ++gq)
-                        if (((cur.ok >> i) & 1u) && g_lane == gq) apply_one(cur.ix[i], cur.a[i]);
+            for (int p = 0; p < P; ++p) {
+                const float s = scale ? scale[static_cast<int64_t>(t_now) * P + p] : 1.0f;
+                for (int j = lane; j < k; j += 64) {
+                    uint32_t ixe;
+                    float ae;
+                    load_entry(p, j, g, ixe, ae);
+                    add_entry(ixe, ae * s);
                 }
-            }
-            for (int u = kUnitRegs; u < n_units; ++u) {  // more entries than the registers hold
-                int p, j;
-                const bool ok = entry(u, p, j);
-                uint32_t ix = 0;
-                float a = 0.f;
-                if (ok) {
-                    const gbyte* ip;
-                    const gfloat* vp;
-                    pt.get(p, ip, vp);
-                    ix = load_idx12_g(ip + g * idx_stride, j);
-                    a = vp[g * k + j];
-                    if (scale) a *= scale[static_cast<int64_t>(t_now) * P + p];
-                }
-                for (int gq = 0; gq < G; ++gq)
-                    if (ok && g_lane == gq) apply_one(ix, a);
             }
         }
         wave_lds_fence();
 
-        if (reduce_mode == TPLR_REDUCE_MEAN && __any(collide)) {
-            if (normalise) {
-                for (int p = 0; p < P; ++p) {
-                    const gbyte* ip;
-                    const gfloat* vp;
-                    pt.get(p, ip, vp);
-                    for (int j = lane; j < k; j += 64) claim_divide(load_idx12_g(ip + g * idx_stride, j));
+        // ---- mean: exactly one entry per destination claims the counter and divides the sum
+        if (reduce_mode == TPLR_REDUCE_MEAN && __any(seen != 0)) {
+            auto claim = [&](uint32_t ixe) -> uint32_t {
+                const uint32_t sh = (ixe & 3) * 8;
+                return (atomicAnd(&cnt[ixe >> 2], ~(0xffu << sh)) >> sh) & 0xffu;
+            };
+            auto divide = [&](uint32_t ixe, uint32_t n) {
+                if (n > 1) {
+                    float* t = &tile[tile_pos(ixe)];
+                    *t = *t / static_cast<float>(n);
+                }
+            };
+            if (fast) {
+                if (lane_on) {
+                    uint32_t n_claimed[kRegs];
+#pragma unroll
+                    for (int i = 0; i < kRegs; ++i) {
+                        const bool on = i < P;
+                        const uint32_t sh = (ix[i] & 3) * 8;
+                        n_claimed[i] = (atomicAnd(&cnt[on ? (ix[i] >> 2) : lane], on ? ~(0xffu << sh) : ~0u) >> sh) &
+                                       (on ? 0xffu : 0u);
+                    }
+#pragma unroll
+                    for (int i = 0; i < kRegs; ++i) divide(ix[i], n_claimed[i]);
                 }
             } else {
-#pragma unroll
-                for (int i = 0; i < kUnitRegs; ++i)
-                    if (i < n_units && ((cur.ok >> i) & 1u)) claim_divide(cur.ix[i]);
-                for (int u = kUnitRegs; u < n_units; ++u) {
-                    int p, j;
-                    if (entry(u, p, j)) {
-                        const gbyte* ip;
-                        const gfloat* vp;
-                        pt.get(p, ip, vp);
-                        claim_divide(load_idx12_g(ip + g * idx_stride, j));
+                for (int p = 0; p < P; ++p)
+                    for (int j = lane; j < k; j += 64) {
+                        uint32_t ixe;
+                        float ae;
+                        load_entry(p, j, g, ixe, ae);
+                        divide(ixe, claim(ixe));
                     }
-                }
             }
             wave_lds_fence();
         }
@@ -667,7 +634,7 @@ __global__ __launch_bounds__(64) void k_decode_aggregate(const PeerPtrs pp, cons
         // the next chunk's payload travels while this one goes through the inverse transform
         if (g + 1 < g1) {
             cursor_next(c, g + 1);
-            if (!normalise) load_units(cur, g + 1, c.t);
+            if (fast) load_payload(g + 1, c.t);
         }
 
         if (kUseDct) {
@@ -860,6 +827,19 @@ static int launch_encode_as(Kernel kernel, const tplr_tensor_desc* d_desc, const
     return launch_status();
 }
 
+template <typename Kernel>
+static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_scale, int n_peers, int k,
+                            const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single, int n_tensors,
+                            int64_t total, int reduce_mode, int normalise, float* d_sumsq, void* stream) {
+    static int resident = 0;  // per kernel variant
+    if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
+    const int64_t need = ((total + 7) / 8) * 8;
+    const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
+    hipLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale, n_peers, k, d_desc,
+                       single, n_tensors, total, reduce_mode, normalise, d_sumsq);
+    return launch_status();
+}
+
 extern "C" {
 
 int tplr_version(void) { return 100; }
@@ -1044,21 +1024,25 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
         pp.val[p] = p < n_peers ? h_val[p] : nullptr;
         if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
     }
-    static int resident[2] = {0, 0};
-    const int which = use_dct ? 1 : 0;
-    if (resident[which] == 0)
-        resident[which] = use_dct ? persistent_grid(k_decode_aggregate<true>, int64_t{1} << 40)
-                                  : persistent_grid(k_decode_aggregate<false>, int64_t{1} << 40);
-    const int64_t need = ((total + 7) / 8) * 8;
-    const dim3 grid(static_cast<unsigned>(need < resident[which] ? need : resident[which])), block(64);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (use_dct)
-        hipLaunchKernelGGL(k_decode_aggregate<true>, grid, block, 0, st, pp, d_scale, n_peers, k, d_desc, single,
-                           n_tensors, total, reduce_mode, normalise, d_sumsq);
-    else
-        hipLaunchKernelGGL(k_decode_aggregate<false>, grid, block, 0, st, pp, d_scale, n_peers, k, d_desc, single,
-                           n_tensors, total, reduce_mode, normalise, d_sumsq);
-    return launch_status();
+    const int units = (k > 64 || normalise) ? 0 : n_peers <= 8 ? 8 : n_peers <= 16 ? 16 : n_peers <= 24 ? 24 : 0;
+#define TPLR_DECODE_CASE(U)                                                                                         \
+    case U:                                                                                                         \
+        return use_dct ? launch_decode_as(k_decode_aggregate<true, U>, pp, d_scale, n_peers, k, d_desc, single,       \
+                                          n_tensors, total, reduce_mode, normalise, d_sumsq, stream)                 \
+                       : launch_decode_as(k_decode_aggregate<false, U>, pp, d_scale, n_peers, k, d_desc, single,      \
+                                          n_tensors, total, reduce_mode, normalise, d_sumsq, stream);
+    switch (units) {
+        TPLR_DECODE_CASE(8)
+        TPLR_DECODE_CASE(16)
+        TPLR_DECODE_CASE(24)
+        default:
+            break;
+    }
+#undef TPLR_DECODE_CASE
+    return use_dct ? launch_decode_as(k_decode_aggregate<true, 0>, pp, d_scale, n_peers, k, d_desc, single, n_tensors,
+                                      total, reduce_mode, normalise, d_sumsq, stream)
+                   : launch_decode_as(k_decode_aggregate<false, 0>, pp, d_scale, n_peers, k, d_desc, single, n_tensors,
+                                      total, reduce_mode, normalise, d_sumsq, stream);
 }
 
 static int check_decode(const void* a, const void* b, int n_peers, int k, int reduce_mode) {
