@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Generate straight-line 64-point orthonormal DCT-II / DCT-III device code.
+"""Generate straight-line 64-point DCT-II / DCT-III device code (dct64_gen.h).
 
 The codec transforms every 64x64 chunk with F^T X F where
 F[i,k] = c_k cos(pi (2i+1) k / 128), c_0 = sqrt(1/64), c_k = sqrt(2/64)
@@ -17,11 +17,20 @@ which one lane owns one 64-vector in registers:
            C4[2j] = P[j] + Q[M/2-j], C4[2j-1] = P[j] - Q[M/2-j]   (j = 1..M/2-1)
 
 Every factor is a butterfly or a plane rotation, so rounding error grows like
-log N.  The orthonormal scale factors are folded into the rotation constants
-(one explicit multiply is left, on the DC term).  The inverse transform is the
-transposed flow graph run backwards.
+log N.  Rotations are three lifting steps (three fused multiply-adds):
+  x1 = x + p y, y1 = y - s x1, x2 = x1 + p y1,  p = tan(theta / 2).
 
-Output: dct64_gen.h next to this file.  Run as a build step
+Scaling.  The generated transforms are sqrt(32) TIMES the orthonormal ones:
+only the DC term carries a multiplier (1/sqrt 2), the common factor sqrt(2/64)
+is left out.  Two passes therefore give 32 times the orthonormal 2-D transform
+and the kernels finish with an exact multiplication by 2^-5, on the selected
+values only (encode) or folded into the scalar clip factor (decode).
+
+The inverse transform is the transposed flow graph run backwards.
+
+Functions written: dct64_fwd_head (the 32 input butterflies, from a separate
+input array - it lets the caller start refilling that array right after),
+dct64_fwd_tail, dct64_fwd (both), dct64_inv.  Run as a build step
 (`python gen_dct64.py`); `--check` only verifies and prints op counts.
 """
 from __future__ import annotations
@@ -33,103 +42,103 @@ import sys
 import numpy as np
 
 N = 64
+GAIN = math.sqrt(N / 2.0)  # generated transform = GAIN * orthonormal transform
 
 
 # --------------------------------------------------------------------------
-# exact linear op list:  ("lin2", i, j, a, b, c, d)  (s_i, s_j) <- (a s_i + b s_j, c s_i + d s_j)
-#                        ("mul", i, a)               s_i <- a s_i
+# exact linear op list
+#   ("bfly", i, j)        (s_i, s_j) <- (s_i + s_j, s_i - s_j)
+#   ("rot", i, j, c, s)   (s_i, s_j) <- (c s_i + s s_j, -s s_i + c s_j)
+#   ("mul", i, a)         s_i <- a s_i          (a = -1: sign flip, free)
 # --------------------------------------------------------------------------
 def build_forward():
-    """Orthonormal DCT-II: the scale sigma = sqrt(2/N) rides down the recursion and is
-    absorbed by the first rotation on every path; only the DC path has none, and gets
-    one multiply by sqrt(1/N)."""
     ops = []
-    sigma = math.sqrt(2.0 / N)
 
-    def bfly(i, j):
-        ops.append(("lin2", i, j, 1.0, 1.0, 1.0, -1.0))
-
-    def c2(slots, scale, dc):
+    def c2(slots, dc):
         n = len(slots)
         if n == 1:
-            s = scale / math.sqrt(2.0) if dc else scale
-            if s != 1.0:
-                ops.append(("mul", slots[0], s))
+            if dc:
+                ops.append(("mul", slots[0], 1.0 / math.sqrt(2.0)))
             return list(slots)
         h = n // 2
         for t in range(h):
-            bfly(slots[t], slots[n - 1 - t])
-        even = c2([slots[t] for t in range(h)], scale, dc)
-        odd = c4([slots[n - 1 - t] for t in range(h)], scale)
+            ops.append(("bfly", slots[t], slots[n - 1 - t]))
+        even = c2([slots[t] for t in range(h)], dc)
+        odd = c4([slots[n - 1 - t] for t in range(h)])
         out = [None] * n
         for m in range(h):
             out[2 * m] = even[m]
             out[2 * m + 1] = odd[m]
         return out
 
-    def c4(slots, scale):
+    def c4(slots):
         m = len(slots)
         if m == 1:
-            ops.append(("mul", slots[0], math.cos(math.pi / 4) * scale))
+            ops.append(("mul", slots[0], math.cos(math.pi / 4)))
             return list(slots)
         half = m // 2
         for t in range(half):
             th = math.pi * (2 * t + 1) / (4 * m)
-            c, s = math.cos(th) * scale, math.sin(th) * scale
-            sg = -1.0 if (t & 1) else 1.0
-            ops.append(("lin2", slots[t], slots[m - 1 - t], c, s, -sg * s, sg * c))
-        p = c2([slots[t] for t in range(half)], 1.0, False)
-        q = c2([slots[m - 1 - t] for t in range(half)], 1.0, False)
+            ops.append(("rot", slots[t], slots[m - 1 - t], math.cos(th), math.sin(th)))
+            if t & 1:
+                ops.append(("mul", slots[m - 1 - t], -1.0))
+        p = c2([slots[t] for t in range(half)], False)
+        q = c2([slots[m - 1 - t] for t in range(half)], False)
         out = [None] * m
         out[0] = p[0]
         ops.append(("mul", q[0], -1.0))
         out[m - 1] = q[0]
         for j in range(1, half):
-            bfly(p[j], q[half - j])
+            ops.append(("bfly", p[j], q[half - j]))
             out[2 * j] = p[j]
             out[2 * j - 1] = q[half - j]
         return out
 
-    out_slots = c2(list(range(N)), sigma, True)
+    out_slots = c2(list(range(N)), True)
     return ops, out_slots
-
-
-def is_pm1(x):
-    return abs(abs(x) - 1.0) < 1e-15
 
 
 def transpose_ops(ops):
     out = []
     for op in reversed(ops):
-        if op[0] == "mul":
-            out.append(op)
+        if op[0] == "rot":
+            _, i, j, c, s = op
+            out.append(("rot", i, j, c, -s))
         else:
-            _, i, j, a, b, c, d = op
-            out.append(("lin2", i, j, a, c, b, d))
+            out.append(op)  # butterflies and diagonal factors are symmetric
     return out
 
 
-def as_matrix(ops, in_slots, out_slots, dtype=np.float64):
-    """Column k of the result = transform of unit vector k (inputs in logical order)."""
-    x = np.zeros((N, N), dtype=dtype)  # slot-major state, one column per probe
-    for n, s in enumerate(in_slots):
-        x[s, n] = 1.0
-    x = run_ops(ops, x, dtype)
-    return np.stack([x[s] for s in out_slots])
-
-
-def run_ops(ops, x, dtype=np.float64):
+def run_ops(ops, x, dtype=np.float64, lifting=False):
+    """Apply the op list to a slot-major state (one column per probe vector)."""
     x = x.astype(dtype).copy()
+    f = dtype
     for op in ops:
         if op[0] == "mul":
-            _, i, a = op
-            x[i] = (x[i] * dtype(a)).astype(dtype)
+            x[op[1]] = x[op[1]] * f(op[2])
+        elif op[0] == "bfly":
+            _, i, j = op
+            a, b = x[i].copy(), x[j].copy()
+            x[i], x[j] = a + b, a - b
         else:
-            _, i, j, a, b, c, d = op
-            xi, xj = x[i].copy(), x[j].copy()
-            x[i] = (dtype(a) * xi + dtype(b) * xj).astype(dtype)
-            x[j] = (dtype(c) * xi + dtype(d) * xj).astype(dtype)
+            _, i, j, c, s = op
+            a, b = x[i].copy(), x[j].copy()
+            if lifting:
+                p = f((1.0 - c) / s)
+                a1 = a + p * b
+                b1 = b - f(s) * a1
+                x[i], x[j] = a1 + p * b1, b1
+            else:
+                x[i], x[j] = f(c) * a + f(s) * b, f(c) * b - f(s) * a
     return x
+
+
+def as_matrix(ops, in_slots, out_slots, **kw):
+    x = np.zeros((N, N))
+    for n, s in enumerate(in_slots):
+        x[s, n] = 1.0
+    x = run_ops(ops, x, **kw)
+    return np.stack([x[s] for s in out_slots])
 
 
 def dense_dct():
@@ -141,98 +150,96 @@ def dense_dct():
 
 
 # --------------------------------------------------------------------------
-# emission with lazy sign tracking and FMA fusion
+# emission with lazy sign tracking
 # --------------------------------------------------------------------------
+def lit(v):
+    return np.format_float_scientific(np.float32(v), unique=True, trim="0") + "f"
+
+
 class Emitter:
-    def __init__(self):
-        self.lines = []
-        self.nops = 0
-        self.ntmp = 0
-
-    def new(self):
-        self.ntmp += 1
-        return f"t{self.ntmp}"
-
-    @staticmethod
-    def lit(v):
-        s = repr(float(np.float32(v)))
-        if "e" not in s and "." not in s:
-            s += ".0"
-        # shortest repr of the float32 value, as a float literal
-        s = np.format_float_scientific(np.float32(v), unique=True, trim="0")
-        return s + "f"
+    def __init__(self, prefix):
+        self.lines, self.nops, self.n, self.prefix = [], 0, 0, prefix
 
     def emit(self, expr):
-        name = self.new()
+        self.n += 1
+        name = f"{self.prefix}{self.n}"
         self.lines.append(f"    const float {name} = {expr};")
         self.nops += 1
         return name
 
 
-def emit_function(name, ops, in_slots, out_slots):
-    """in_slots[n]: slot that input v[n] starts in; out_slots[k]: slot holding output k."""
-    em = Emitter()
-    var = {}
-    sign = {}
-    for n, s in enumerate(in_slots):
-        var[s] = f"v[{n}]"
-        sign[s] = 1.0
+def emit_ops(em, ops, var, sign):
     for op in ops:
         if op[0] == "mul":
             _, i, a = op
-            a = a * sign[i]
-            if is_pm1(a):
+            a *= sign[i]
+            if abs(abs(a) - 1.0) < 1e-15:
                 sign[i] = math.copysign(1.0, a)
-                continue
-            var[i] = em.emit(f"{var[i]} * {em.lit(a)}")
-            sign[i] = 1.0
-            continue
-        _, i, j, a, b, c, d = op
-        a, c = a * sign[i], c * sign[i]
-        b, d = b * sign[j], d * sign[j]
-        xi, xj = var[i], var[j]
-        if all(is_pm1(v) for v in (a, b, c, d)):
-            def row(p, q):
-                # returns (expr, sign) for p*xi + q*xj with p,q in +-1
-                if p > 0 and q > 0:
-                    return f"{xi} + {xj}", 1.0
-                if p > 0 and q < 0:
-                    return f"{xi} - {xj}", 1.0
-                if p < 0 and q > 0:
-                    return f"{xj} - {xi}", 1.0
-                return f"{xi} + {xj}", -1.0
-            e1, s1 = row(a, b)
-            e2, s2 = row(c, d)
-            var[i], sign[i] = em.emit(e1), s1
-            var[j], sign[j] = em.emit(e2), s2
+            else:
+                var[i], sign[i] = em.emit(f"{var[i]} * {lit(a)}"), 1.0
+        elif op[0] == "bfly":
+            _, i, j = op
+            xi, xj, si, sj = var[i], var[j], sign[i], sign[j]
+            if si > 0 and sj > 0:
+                var[i], sign[i] = em.emit(f"{xi} + {xj}"), 1.0
+                var[j], sign[j] = em.emit(f"{xi} - {xj}"), 1.0
+            elif si > 0:
+                var[i], sign[i] = em.emit(f"{xi} - {xj}"), 1.0
+                var[j], sign[j] = em.emit(f"{xi} + {xj}"), 1.0
+            elif sj > 0:
+                var[i], sign[i] = em.emit(f"{xj} - {xi}"), 1.0
+                var[j], sign[j] = em.emit(f"{xi} + {xj}"), -1.0
+            else:
+                var[i], sign[i] = em.emit(f"{xi} + {xj}"), -1.0
+                var[j], sign[j] = em.emit(f"{xj} - {xi}"), 1.0
         else:
-            def row(p, q):
-                # p*xi + q*xj with FMA; a +-1 coefficient saves the multiply
-                if is_pm1(p):
-                    base = xi if p > 0 else f"-{xi}"
-                    return em.emit(f"__builtin_fmaf({xj}, {em.lit(q)}, {base})")
-                if is_pm1(q):
-                    base = xj if q > 0 else f"-{xj}"
-                    return em.emit(f"__builtin_fmaf({xi}, {em.lit(p)}, {base})")
-                t = em.emit(f"{xi} * {em.lit(p)}")
-                return em.emit(f"__builtin_fmaf({xj}, {em.lit(q)}, {t})")
-            n1 = row(a, b)
-            n2 = row(c, d)
-            var[i], sign[i] = n1, 1.0
-            var[j], sign[j] = n2, 1.0
+            _, i, j, c, s = op
+            s = s * sign[i] * sign[j]  # R diag(si, sj) = diag(si, sj) R(s -> s si sj)
+            p = (1.0 - c) / s
+            x1 = em.emit(f"__builtin_fmaf({var[j]}, {lit(p)}, {var[i]})")
+            y1 = em.emit(f"__builtin_fmaf({x1}, {lit(-s)}, {var[j]})")
+            x2 = em.emit(f"__builtin_fmaf({y1}, {lit(p)}, {x1})")
+            var[i], var[j] = x2, y1
+
+
+def finish(em, var, sign, out_slots, dst="v"):
     tail = []
     negs = 0
     for k, s in enumerate(out_slots):
         if sign[s] < 0:
-            tail.append(f"    v[{k}] = -{var[s]};")
+            tail.append(f"    {dst}[{k}] = -{var[s]};")
             negs += 1
         else:
-            tail.append(f"    v[{k}] = {var[s]};")
-    body = "\n".join(em.lines + tail)
-    text = (
-        f"__device__ __forceinline__ void {name}(float (&v)[64]) {{\n{body}\n}}\n"
-    )
-    return text, em.nops, negs
+            tail.append(f"    {dst}[{k}] = {var[s]};")
+    return "\n".join(em.lines + tail), negs
+
+
+def emit_function(name, ops, in_slots, out_slots):
+    em = Emitter("t")
+    var = {s: f"v[{n}]" for n, s in enumerate(in_slots)}
+    sign = {s: 1.0 for s in in_slots}
+    emit_ops(em, ops, var, sign)
+    body, negs = finish(em, var, sign, out_slots)
+    return f"__device__ __forceinline__ void {name}(float (&v)[64]) {{\n{body}\n}}\n", em.nops, negs
+
+
+def emit_split_forward(ops, out_slots, n_head):
+    """head: in[] -> v[] through the first n_head ops (slot order kept); tail: the rest, in place."""
+    em = Emitter("h")
+    var = {s: f"in[{s}]" for s in range(N)}
+    sign = {s: 1.0 for s in range(N)}
+    emit_ops(em, ops[:n_head], var, sign)
+    assert all(sg > 0 for sg in sign.values())
+    body, _ = finish(em, var, sign, list(range(N)))
+    head = ("__device__ __forceinline__ void dct64_fwd_head(const float (&in)[64], float (&v)[64]) {\n"
+            f"{body}\n}}\n")
+    em2 = Emitter("t")
+    var = {s: f"v[{s}]" for s in range(N)}
+    sign = {s: 1.0 for s in range(N)}
+    emit_ops(em2, ops[n_head:], var, sign)
+    body, negs = finish(em2, var, sign, out_slots)
+    tail = f"__device__ __forceinline__ void dct64_fwd_tail(float (&v)[64]) {{\n{body}\n}}\n"
+    return head, tail, em.nops, em2.nops, negs
 
 
 def main():
@@ -240,41 +247,55 @@ def main():
     fwd, out_slots = build_forward()
     inv = transpose_ops(fwd)
     ident = list(range(N))
+    n_head = N // 2
+    assert all(op[0] == "bfly" for op in fwd[:n_head])
 
     f = dense_dct()
-    m_fwd = as_matrix(fwd, ident, out_slots)  # [k, n]
-    err_f = np.abs(m_fwd - f.T).max()
-    m_inv = as_matrix(inv, out_slots, ident)  # inputs logical k live in out_slots[k]
-    err_i = np.abs(m_inv - f).max()
-    assert err_f < 1e-14 and err_i < 1e-14, (err_f, err_i)
+    for lifting in (False, True):
+        m_fwd = as_matrix(fwd, ident, out_slots, lifting=lifting)  # [k, n]
+        m_inv = as_matrix(inv, out_slots, ident, lifting=lifting)
+        err_f = np.abs(m_fwd - GAIN * f.T).max()
+        err_i = np.abs(m_inv - GAIN * f).max()
+        assert err_f < 1e-13 and err_i < 1e-13, (lifting, err_f, err_i)
 
-    # float32 behaviour on heavy-tailed data
+    # float32 behaviour on heavy-tailed data, forward and round trip
     rng = np.random.default_rng(0)
-    x = (rng.standard_t(3, size=(N, 4096)) * 1e-3)
+    x = rng.standard_t(3, size=(N, 4096)) * 1e-3
     st = np.zeros((N, 4096))
     st[ident] = x
-    y32 = run_ops(fwd, st, np.float32)
-    y32 = np.stack([y32[s] for s in out_slots]).astype(np.float64)
+    y32 = run_ops(fwd, st, np.float32, lifting=True)
+    y = np.stack([y32[s] for s in out_slots]).astype(np.float64) / GAIN
     y64 = f.T @ x
-    rel = np.abs(y32 - y64).max() / np.abs(y64).max()
+    rel = np.abs(y - y64).max() / np.abs(y64).max()
+    st2 = np.zeros((N, 4096), np.float32)
+    for k, s in enumerate(out_slots):
+        st2[s] = y32[s]
+    back = run_ops(inv, st2, np.float32, lifting=True)[ident].astype(np.float64) / (GAIN * GAIN)
+    rel_rt = np.abs(back - x).max() / np.abs(x).max()
 
-    t_fwd, n_fwd, neg_f = emit_function("dct64_fwd", fwd, ident, out_slots)
+    head, tail, n_h, n_t, neg_f = emit_split_forward(fwd, out_slots, n_head)
     t_inv, n_inv, neg_i = emit_function("dct64_inv", inv, out_slots, ident)
-    print(f"dct64_fwd: {n_fwd} ops (+{neg_f} negations), dct64_inv: {n_inv} ops (+{neg_i} negations)")
-    print(f"fp64 matrix error fwd {err_f:.2e} inv {err_i:.2e}; fp32 max err / max|y| = {rel:.2e}")
+    print(f"dct64_fwd: {n_h} + {n_t} ops (+{neg_f} negations), dct64_inv: {n_inv} ops (+{neg_i} negations)")
+    print(f"fp64 matrix error fwd {err_f:.2e} inv {err_i:.2e}; fp32 forward err / max|y| = {rel:.2e}, "
+          f"round trip err / max|x| = {rel_rt:.2e}")
     if check_only:
         return
     here = os.path.dirname(os.path.abspath(__file__))
     with open(os.path.join(here, "dct64_gen.h"), "w") as fh:
         fh.write(
             "// Generated by gen_dct64.py - do not edit.\n"
-            "// 64-point orthonormal DCT-II (dct64_fwd) and its inverse, DCT-III (dct64_inv),\n"
-            "// as straight-line butterfly/rotation code on 64 registers of one lane.\n"
-            f"// {n_fwd} / {n_inv} floating-point instructions per transform.\n"
+            "// 64-point DCT-II (dct64_fwd = dct64_fwd_head + dct64_fwd_tail) and DCT-III (dct64_inv) as\n"
+            "// straight-line butterfly / lifting-rotation code on the 64 registers of one lane.\n"
+            "// Both are sqrt(32) times the orthonormal transform: two passes give 32x, and the caller\n"
+            "// finishes with an exact multiplication by kDctPow2Scale.\n"
+            f"// {n_h + n_t} / {n_inv} floating-point instructions per transform.\n"
             "#pragma once\n\n"
+            "constexpr float kDctPow2Scale = 0.03125f;  // 2^-5\n\n"
         )
-        fh.write(t_fwd)
-        fh.write("\n")
+        fh.write(head + "\n" + tail + "\n")
+        fh.write("__device__ __forceinline__ void dct64_fwd(float (&v)[64]) {\n"
+                 "    float t[64];\n    dct64_fwd_head(v, t);\n    dct64_fwd_tail(t);\n"
+                 "#pragma unroll\n    for (int i = 0; i < 64; ++i) v[i] = t[i];\n}\n\n")
         fh.write(t_inv)
 
 

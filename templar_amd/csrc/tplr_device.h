@@ -321,8 +321,11 @@ __device__ __forceinline__ void sort128_step(uint64_t& e0, uint64_t& e1) {
 
 __device__ __forceinline__ void sort128_desc(uint64_t& e0, uint64_t& e1, int) { sort128_step<2, 1>(e0, e1); }
 
+// `out_scale` multiplies the gathered values (an exact power of two left over by the caller's
+// transform; the ordering is taken on the unscaled values).
 template <bool kTwo>
-__device__ __forceinline__ Selected select_topk(const float (&v)[64], float* tile, int lane, int k) {
+__device__ __forceinline__ Selected select_topk(const float (&v)[64], float* tile, int lane, int k,
+                                                float out_scale) {
     uint32_t b1, b2;
     lane_stats<kTwo>(v, b1, b2);
     const uint32_t t0 = stat_threshold<kTwo>(b1, b2, k);
@@ -417,8 +420,8 @@ __device__ __forceinline__ Selected select_topk(const float (&v)[64], float* til
     // lanes beyond k may hold padding (index 0xffffffff - 0 wraps to a huge value): clamp
     out.idx0 &= 4095u;
     out.idx1 &= 4095u;
-    out.val0 = tile[(out.idx0 >> 6) * kLd + (out.idx0 & 63)];
-    if (k > 64) out.val1 = tile[(out.idx1 >> 6) * kLd + (out.idx1 & 63)];
+    out.val0 = tile[(out.idx0 >> 6) * kLd + (out.idx0 & 63)] * out_scale;
+    if (k > 64) out.val1 = tile[(out.idx1 >> 6) * kLd + (out.idx1 & 63)] * out_scale;
     return out;
 }
 

@@ -118,10 +118,25 @@ struct NoHook {
     __device__ __forceinline__ void operator()() const {}
 };
 
-template <bool kUseDct, typename Hook = NoHook>
-__device__ __forceinline__ void chunk_forward(float (&v)[64], float* tile, int lane, Hook between_passes = Hook()) {
-    if (kUseDct) dct64_fwd(v);  // along rows k: v[b] = sum_k X[k][lane] F[k][b]
-    // keep the hook's memory requests behind the first pass: tie them to its last results
+// Forward 2-D transform of a chunk.  `in` holds it column-per-lane (in[r] = X[r][lane]); the
+// result is row-per-lane in v (v[d] = 32 * coef[lane][d] with the transform, X[lane][d]
+// without) and the tile is left free.  `in` is dead after the first butterfly level, which is
+// when after_inputs() runs (the caller starts refilling it there); between_passes() runs after
+// the first pass.
+template <bool kUseDct, typename Hook1 = NoHook, typename Hook2 = NoHook>
+__device__ __forceinline__ void chunk_forward(const float (&in)[64], float (&v)[64], float* tile, int lane,
+                                              Hook1 after_inputs = Hook1(), Hook2 between_passes = Hook2()) {
+    if (kUseDct) {
+        dct64_fwd_head(in, v);  // along rows k: v[b] = sum_k X[k][lane] F[k][b]
+    } else {
+#pragma unroll
+        for (int r = 0; r < 64; ++r) v[r] = in[r];
+    }
+    // pin the hooks' memory requests to their place in the instruction stream
+    asm volatile("" : "+v"(v[0]), "+v"(v[31]), "+v"(v[63])::"memory");
+    after_inputs();
+    asm volatile("" ::: "memory");
+    if (kUseDct) dct64_fwd_tail(v);
     asm volatile("" : "+v"(v[1]), "+v"(v[31]), "+v"(v[63])::"memory");
     between_passes();
     asm volatile("" ::: "memory");
@@ -133,10 +148,16 @@ __device__ __forceinline__ void chunk_forward(float (&v)[64], float* tile, int l
 }
 
 // inverse: tile holds coef rows; result column-per-lane v[k] = x[k][lane]
-template <bool kUseDct>
+// (the tile must hold the coefficients times 2^-5: the two passes multiply by 32; kScaleInput
+// applies that factor here for callers whose tile holds plain coefficients)
+template <bool kUseDct, bool kScaleInput = false>
 __device__ __forceinline__ void chunk_inverse(float (&v)[64], float* tile, int lane) {
     if (kUseDct) {
         tile_rows_to_regs(v, tile, lane);
+        if (kScaleInput) {
+#pragma unroll
+            for (int d = 0; d < 64; ++d) v[d] *= kDctPow2Scale;
+        }
         dct64_inv(v);  // along d: v[l] = sum_d Y[lane][d] F[l][d]
         wave_lds_fence();
         regs_to_tile_rows(v, tile, lane);
@@ -252,9 +273,11 @@ __global__ __launch_bounds__(64) void k_dct2d_fwd(const float* __restrict__ x, i
     const int64_t chunk = xcd_contiguous(blockIdx.x, gridDim.x);
     if (chunk >= n_chunks) return;
     const int64_t y = chunk / X, xc = chunk - y * X;
-    float v[64];
-    load_chunk_cols(v, x, ld, y, xc, lane);
-    chunk_forward<true>(v, tile, lane);
+    float in[64], v[64];
+    load_chunk_cols(in, x, ld, y, xc, lane);
+    chunk_forward<true>(in, v, tile, lane);
+#pragma unroll
+    for (int d = 0; d < 64; ++d) v[d] *= kDctPow2Scale;  // exact: 32x the orthonormal transform so far
     regs_to_tile_rows(v, tile, lane);
     __syncthreads();
     tile_to_flat(tile, coef + chunk * 4096, lane);
@@ -270,7 +293,7 @@ __global__ __launch_bounds__(64) void k_dct2d_inv(const float* __restrict__ coef
     flat_to_tile(coef + chunk * 4096, tile, lane);
     __syncthreads();
     float v[64];
-    chunk_inverse<true>(v, tile, lane);
+    chunk_inverse<true, true>(v, tile, lane);
     store_chunk_cols(v, x, ld, y, xc, lane);
 }
 
@@ -296,6 +319,9 @@ __global__ __launch_bounds__(64) void k_dct1d(const float* __restrict__ in, int6
         dct64_inv(v);
     else
         dct64_fwd(v);
+    // one pass is sqrt(32) times the orthonormal transform
+#pragma unroll
+    for (int d = 0; d < 64; ++d) v[d] *= 0.17677669529663687f;
     __syncthreads();
     regs_to_tile_rows(v, tile, lane);
     __syncthreads();
@@ -371,7 +397,7 @@ __global__ __launch_bounds__(64) void k_topk_rows(const float* __restrict__ coef
     __syncthreads();
     float v[64];
     tile_rows_to_regs(v, tile, lane);
-    const Selected s = select_topk<kTwo>(v, tile, lane, k);
+    const Selected s = select_topk<kTwo>(v, tile, lane, k, 1.0f);
     emit_selected(s, lane, k, row, idx12, val);
 }
 
@@ -392,28 +418,32 @@ __global__ __launch_bounds__(64, 2) void k_encode_topk_pack(const tplr_tensor_de
     // Loads and stores share one completion counter and complete out of order with respect to
     // each other, so a wait for the prefetched rows also waits for every store issued before it.
     // The selection of chunk g is therefore written in the middle of iteration g + 1, a
-    // transform pass away from the waits on either side.
+    // transform pass away from the waits on either side.  The rows of chunk g + 1 land in the
+    // registers chunk g was read from, which its first butterfly level has freed.
     float v[64], nx[64];
     load_chunk_cols(nx, c, lane);
     Selected prev = {};
     for (int64_t g = g0; g < g1; ++g) {
-#pragma unroll
-        for (int r = 0; r < 64; ++r) v[r] = nx[r];
-        // at most 63 vector-memory operations can be outstanding: the previous selection is
-        // written, and the last rows requested, after the first transform pass
+        // at most 63 vector-memory operations can be outstanding: most rows of the next chunk are
+        // requested as soon as the first butterfly level has consumed this chunk's registers, the
+        // previous selection is written and the last rows requested after the first pass
         constexpr int kSplit = 56;
         const bool more = g + 1 < g1;
-        if (more) {
-            cursor_next(c, g + 1);
-            load_chunk_cols<0, kSplit>(nx, c, lane);
-        }
-        chunk_forward<kUseDct>(v, tile, lane, [&]() {
-            if (g > g0) emit_selected(prev, lane, k, g - 1, idx12, val);
-            if (more) load_chunk_cols<kSplit, 64>(nx, c, lane);
-        });
+        chunk_forward<kUseDct>(
+            nx, v, tile, lane,
+            [&]() {
+                if (more) {
+                    cursor_next(c, g + 1);
+                    load_chunk_cols<0, kSplit>(nx, c, lane);
+                }
+            },
+            [&]() {
+                if (g > g0) emit_selected(prev, lane, k, g - 1, idx12, val);
+                if (more) load_chunk_cols<kSplit, 64>(nx, c, lane);
+            });
         regs_to_tile_rows(v, tile, lane);
         wave_lds_fence();
-        prev = select_topk<kTwo>(v, tile, lane, k);
+        prev = select_topk<kTwo>(v, tile, lane, k, kUseDct ? kDctPow2Scale : 1.0f);
         wave_lds_fence();
     }
     emit_selected(prev, lane, k, g1 - 1, idx12, val);
@@ -440,10 +470,20 @@ __device__ __forceinline__ uint32_t load_idx12(BytePtr row, int j) {
 typedef uint16_t __attribute__((aligned(1))) unaligned_u16;
 using gu16 = __attribute__((address_space(1))) unaligned_u16;
 
-constexpr int kCntWords = 1024;  // 4096 one-byte contribution counters
+// Contribution counters, one per coefficient, packed into 32-bit words that LDS atomics update:
+// 4 bits each when at most 15 peers can hit a coefficient (2 KB, so that 8 waves fit the 160 KB
+// of a CU), 8 bits otherwise (4 KB, 7 waves).
+template <int kBits>
+struct Counters {
+    static constexpr int kPerWord = 32 / kBits;
+    static constexpr int kWords = 4096 / kPerWord;
+    static constexpr uint32_t kMask = (1u << kBits) - 1u;
+    __device__ static __forceinline__ uint32_t word(uint32_t e) { return e / kPerWord; }
+    __device__ static __forceinline__ uint32_t shift(uint32_t e) { return (e % kPerWord) * kBits; }
+};
 
 // Persistent fused decode.  Per chunk, the peers' entries are accumulated in peer order into an
-// LDS tile (sums) and a byte-per-coefficient contribution count; touched coefficients are
+// LDS tile (sums) and a per-coefficient contribution count; touched coefficients are
 // divided by their count; the tile goes through the inverse 2-D DCT.
 //
 // Fast path (kUnits > 0: k <= 64 and at most kUnits peers): lane j handles entry j of every
@@ -457,14 +497,15 @@ constexpr int kCntWords = 1024;  // 4096 one-byte contribution counters
 // Loads and stores complete out of order with respect to each other on one counter, so the 64
 // row stores of chunk g are issued at the top of iteration g + 1, after the wait for that
 // chunk's payload registers and a whole iteration before the next wait.
-template <bool kUseDct, int kUnits>
+template <bool kUseDct, int kUnits, int kCntBits>
 __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
                                                             int64_t total, int reduce_mode, int normalise,
                                                             float* __restrict__ sumsq) {
     __shared__ __align__(16) float tile[kTileFloats];
-    __shared__ __align__(16) uint32_t cnt[kCntWords];
+    using Cnt = Counters<kCntBits>;
+    __shared__ __align__(16) uint32_t cnt[Cnt::kWords];
     constexpr bool kFast = kUnits > 0;
     constexpr int kRegs = kFast ? kUnits : 1;
     const int lane = threadIdx.x;
@@ -473,6 +514,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     if (g0 >= g1) return;
 
     const int64_t idx_stride = k + (k >> 1);
+    // the inverse transform below is 32x the orthonormal one: its input carries the exact 2^-5
+    const float out_scale = kUseDct ? kDctPow2Scale : 1.0f;
     const int lane_ioff = 3 * (lane >> 1) + (lane & 1);  // byte offset of entry `lane` in a packed row
     const bool lane_on = lane < k;                       // fast path: this lane owns an entry
     const int dummy_pos = lane * kLd + kChunk;           // per-lane padding slot
@@ -486,7 +529,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             const int p = i < P ? i : P - 1;  // unused units read the last peer and are masked later
             const gbyte* irow = (const gbyte*)pp.idx[p] + g * idx_stride;  // wave-uniform
             const gfloat* vrow = (const gfloat*)pp.val[p] + g * k;
-            sc[i] = scale ? scale[static_cast<int64_t>(t) * P + p] : 1.0f;
+            sc[i] = (scale ? scale[static_cast<int64_t>(t) * P + p] : 1.0f) * out_scale;
             ix[i] = 0;
             a[i] = 0.f;
             if (lane_on) {
@@ -541,7 +584,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             for (int q = 0; q < 16; ++q) row[q] = z;
             const uint4 zi = make_uint4(0, 0, 0, 0);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
+            for (int q = 0; q < Cnt::kWords / 256; ++q) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
         }
         wave_lds_fence();
 
@@ -549,8 +592,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         uint32_t seen = 0;
         auto add_entry = [&](uint32_t ixe, float val) {
             atomicAdd(&tile[tile_pos(ixe)], val);
-            const uint32_t sh = (ixe & 3) * 8;
-            seen |= (atomicAdd(&cnt[ixe >> 2], 1u << sh) >> sh) & 0xffu;
+            const uint32_t sh = Cnt::shift(ixe);
+            seen |= (atomicAdd(&cnt[Cnt::word(ixe)], 1u << sh) >> sh) & Cnt::kMask;
         };
         if (fast) {
             if (lane_on) {
@@ -560,12 +603,14 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                     const bool on = i < P;  // wave-uniform
                     const uint32_t e = (lane & 1) ? (ix[i] >> 4) : (ix[i] & 0xfffu);
                     ix[i] = e;  // decoded index, kept for the mean pass
-                    const uint32_t sh = (e & 3) * 8;
                     atomicAdd(&tile[on ? tile_pos(e) : dummy_pos], on ? a[i] * sc[i] : 0.f);
-                    old[i] = (atomicAdd(&cnt[on ? (e >> 2) : lane], on ? (1u << sh) : 0u) >> sh) & (on ? 0xffu : 0u);
+                    old[i] = atomicAdd(&cnt[on ? Cnt::word(e) : lane], on ? (1u << Cnt::shift(e)) : 0u);
                 }
+                // the returned counts are only looked at once every add has been issued
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int i = 0; i < kRegs; ++i) seen |= old[i];
+                for (int i = 0; i < kRegs; ++i)
+                    if (i < P) seen |= (old[i] >> Cnt::shift(ix[i])) & Cnt::kMask;
             }
         } else if (normalise) {
             // per-peer, per-chunk L2 normalisation (compress.py:541-545); simple, unbatched
@@ -578,7 +623,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                     uint32_t ixe;
                     float ae;
                     load_entry(p, j, g, ixe, ae);
-                    add_entry(ixe, ae / nrm);
+                    add_entry(ixe, (ae / nrm) * out_scale);
                 }
             }
         } else {
@@ -588,7 +633,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                     uint32_t ixe;
                     float ae;
                     load_entry(p, j, g, ixe, ae);
-                    add_entry(ixe, ae * s);
+                    add_entry(ixe, (ae * s) * out_scale);
                 }
             }
         }
@@ -597,8 +642,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         // ---- mean: exactly one entry per destination claims the counter and divides the sum
         if (reduce_mode == TPLR_REDUCE_MEAN && __any(seen != 0)) {
             auto claim = [&](uint32_t ixe) -> uint32_t {
-                const uint32_t sh = (ixe & 3) * 8;
-                return (atomicAnd(&cnt[ixe >> 2], ~(0xffu << sh)) >> sh) & 0xffu;
+                const uint32_t sh = Cnt::shift(ixe);
+                return (atomicAnd(&cnt[Cnt::word(ixe)], ~(Cnt::kMask << sh)) >> sh) & Cnt::kMask;
             };
             auto divide = [&](uint32_t ixe, uint32_t n) {
                 if (n > 1) {
@@ -612,12 +657,13 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
 #pragma unroll
                     for (int i = 0; i < kRegs; ++i) {
                         const bool on = i < P;
-                        const uint32_t sh = (ix[i] & 3) * 8;
-                        n_claimed[i] = (atomicAnd(&cnt[on ? (ix[i] >> 2) : lane], on ? ~(0xffu << sh) : ~0u) >> sh) &
-                                       (on ? 0xffu : 0u);
+                        const uint32_t sh = Cnt::shift(ix[i]);
+                        n_claimed[i] = atomicAnd(&cnt[on ? Cnt::word(ix[i]) : lane], on ? ~(Cnt::kMask << sh) : ~0u);
                     }
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int i = 0; i < kRegs; ++i) divide(ix[i], n_claimed[i]);
+                    for (int i = 0; i < kRegs; ++i)
+                        if (i < P) divide(ix[i], (n_claimed[i] >> Cnt::shift(ix[i])) & Cnt::kMask);
                 }
             } else {
                 for (int p = 0; p < P; ++p)
@@ -744,17 +790,31 @@ __global__ __launch_bounds__(1024) void k_peer_sumsq(const ValPtrs vp, int64_t n
     }
 }
 
-// one block per (tensor, peer): sum of squares of that tensor's slice of the peer's values
+// one block per (tensor, peer): sum of squares of that tensor's slice of the peer's values.
+// The slice starts at an even element (k is even), so it is read as float2 with eight
+// independent accumulators per thread; the reduction order is fixed.
 __global__ __launch_bounds__(256) void k_segment_sumsq(const ValPtrs vp, int P, int k,
                                                        const tplr_tensor_desc* __restrict__ table,
                                                        float* __restrict__ sumsq) {
     __shared__ float part[4];
     const int t = blockIdx.x / P, p = blockIdx.x - t * P;
     const tplr_tensor_desc d = table[t];
-    const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks * k;
-    const float* v = vp.val[p] + d.chunk_begin * k;
-    float s = 0.f;
-    for (int64_t i = threadIdx.x; i < n; i += 256) s = __builtin_fmaf(v[i], v[i], s);
+    const int64_t n2 = static_cast<int64_t>(d.x_chunks) * d.y_chunks * k / 2;
+    const float2* v = reinterpret_cast<const float2*>(vp.val[p] + d.chunk_begin * k);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    int64_t i = threadIdx.x;
+    for (; i + 7 * 256 < n2; i += 8 * 256) {
+        float2 x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = v[i + u * 256];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc[u] = __builtin_fmaf(x[u].y, x[u].y, __builtin_fmaf(x[u].x, x[u].x, acc[u]));
+    }
+    for (; i < n2; i += 256) {
+        const float2 x = v[i];
+        acc[0] = __builtin_fmaf(x.y, x.y, __builtin_fmaf(x.x, x.x, acc[0]));
+    }
+    float s = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
     s = wave_sum_f32(s);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
     __syncthreads();
@@ -1024,25 +1084,26 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
         pp.val[p] = p < n_peers ? h_val[p] : nullptr;
         if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
     }
-    const int units = (k > 64 || normalise) ? 0 : n_peers <= 8 ? 8 : n_peers <= 16 ? 16 : n_peers <= 24 ? 24 : 0;
-#define TPLR_DECODE_CASE(U)                                                                                         \
+    // register-resident fast path: k <= 64 and at most 24 peers; 4-bit counters up to 15 peers
+    const int units = (k > 64 || normalise) ? 0 : n_peers <= 8 ? 8 : n_peers <= 15 ? 16 : n_peers <= 24 ? 24 : 0;
+#define TPLR_DECODE_CASE(U, BITS)                                                                                   \
     case U:                                                                                                         \
-        return use_dct ? launch_decode_as(k_decode_aggregate<true, U>, pp, d_scale, n_peers, k, d_desc, single,       \
-                                          n_tensors, total, reduce_mode, normalise, d_sumsq, stream)                 \
-                       : launch_decode_as(k_decode_aggregate<false, U>, pp, d_scale, n_peers, k, d_desc, single,      \
-                                          n_tensors, total, reduce_mode, normalise, d_sumsq, stream);
+        return use_dct ? launch_decode_as(k_decode_aggregate<true, U, BITS>, pp, d_scale, n_peers, k, d_desc,         \
+                                          single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream)         \
+                       : launch_decode_as(k_decode_aggregate<false, U, BITS>, pp, d_scale, n_peers, k, d_desc,        \
+                                          single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream);
     switch (units) {
-        TPLR_DECODE_CASE(8)
-        TPLR_DECODE_CASE(16)
-        TPLR_DECODE_CASE(24)
+        TPLR_DECODE_CASE(8, 4)
+        TPLR_DECODE_CASE(16, 4)
+        TPLR_DECODE_CASE(24, 8)
         default:
             break;
     }
 #undef TPLR_DECODE_CASE
-    return use_dct ? launch_decode_as(k_decode_aggregate<true, 0>, pp, d_scale, n_peers, k, d_desc, single, n_tensors,
-                                      total, reduce_mode, normalise, d_sumsq, stream)
-                   : launch_decode_as(k_decode_aggregate<false, 0>, pp, d_scale, n_peers, k, d_desc, single, n_tensors,
-                                      total, reduce_mode, normalise, d_sumsq, stream);
+    return use_dct ? launch_decode_as(k_decode_aggregate<true, 0, 8>, pp, d_scale, n_peers, k, d_desc, single,
+                                      n_tensors, total, reduce_mode, normalise, d_sumsq, stream)
+                   : launch_decode_as(k_decode_aggregate<false, 0, 8>, pp, d_scale, n_peers, k, d_desc, single,
+                                      n_tensors, total, reduce_mode, normalise, d_sumsq, stream);
 }
 
 static int check_decode(const void* a, const void* b, int n_peers, int k, int reduce_mode) {
