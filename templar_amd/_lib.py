@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtplr_hip.so")
+# TPLR_HIP_LIB selects another build of the same library (e.g. an instrumented one)
+LIB_PATH = os.environ.get("TPLR_HIP_LIB") or os.path.join(_HERE, "libtplr_hip.so")
 
 TPLR_E_BADARG, TPLR_E_ODD, TPLR_E_SHAPE, TPLR_E_TOOMANY = -1, -2, -3, -4
 TPLR_MAX_PEERS = 128
