@@ -17,8 +17,10 @@ namespace tplr {
 
 constexpr int kChunk = 64;
 constexpr int kLd = 68;                    // tile row stride in floats
-constexpr int kTileFloats = kChunk * kLd;  // 4352 floats = 17408 bytes
-constexpr int kCandCap = 128;              // candidate slots hidden in the tile padding
+constexpr int kTileFloats = kChunk * kLd;  // 4352 floats = 17408 bytes: a whole chunk
+constexpr int kHalfRows = 32;
+constexpr int kHalfFloats = kHalfRows * kLd;  // 8704 bytes: the encode side stages half a chunk at a time
+constexpr int kCandCap = 128;                 // top-k candidate slots (8 bytes each)
 
 // Workgroups are dealt round-robin to the 8 XCDs; give every XCD one contiguous range of
 // work items so that neighbouring chunks (which share output cache lines) meet in one L2.
@@ -34,10 +36,6 @@ __device__ __forceinline__ int64_t xcd_contiguous(int64_t bid, int64_t grid) {
 __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
-}
-
-__device__ __forceinline__ uint64_t* cand_slot(float* tile, int s) {
-    return reinterpret_cast<uint64_t*>(tile + (s >> 1) * kLd + kChunk + ((s & 1) << 1));
 }
 
 // All NaNs share the top key so that they tie and fall back to index order.
@@ -58,6 +56,19 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
         const uint32_t o = __shfl_xor(x, off);
         x = o > x ? o : x;
     }
+    return x;
+}
+
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (no LDS round
+// trips): four shifted adds inside each row of 16 lanes, then the row totals are broadcast
+// into the following rows.
+__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t x) {
+    x += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x111, 0xf, 0xf, false));  // row_shr:1
+    x += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x112, 0xf, 0xf, false));  // row_shr:2
+    x += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x114, 0xf, 0xf, false));  // row_shr:4
+    x += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x118, 0xf, 0xf, false));  // row_shr:8
+    x += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x142, 0xa, 0xf, false));  // row_bcast:15
+    x += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x143, 0xc, 0xf, false));  // row_bcast:31
     return x;
 }
 
@@ -119,17 +130,19 @@ __device__ __forceinline__ void tile_to_flat(const float* tile, float* __restric
 // ---------------------------------------------------------------------------------------
 // Top-k of the 4096 values of one chunk by magnitude.
 //
-// On entry lane L holds v[d] = value with flat index L*64 + d, and the same values are in
-// the tile (rows).  On exit lanes hold the k selected elements in canonical order
-// (descending magnitude, lowest index first on ties): element i < 64 in lane i (idx0/val0),
-// element 64 + i in lane i (idx1/val1, only when k > 64).
+// On entry lane L holds w[d] = value with flat index L*64 + d.  On exit lanes hold the k
+// selected elements in canonical order (descending magnitude, lowest index first on ties):
+// element i < 64 in lane i (idx0/val0), element 64 + i in lane i (idx1/val1, only for k > 64).
 //
-// Method: a cheap lower bound T0 for the k-th largest magnitude comes from per-lane
-// maxima (k <= 32) or per-lane top-2 (k <= 128): the k-th largest of those is met by at
-// least k elements.  Everything >= T0 (typically 1.1-1.4 k elements) is compacted into the
-// candidate slots and bitonic-sorted on the 64-bit key (magnitude bits, ~index).  If more
-// than 128 elements pass, an exact bitwise search for the k-th largest magnitude runs
-// instead (rare: constant or all-zero chunks, pathological ties).
+// Method: a cheap lower bound T0 for the k-th largest magnitude comes from per-lane maxima
+// (k <= 32) or per-lane top-2 (k <= 128): the k-th largest of those is met by at least k
+// elements.  Everything
+// >= T0 (typically 1.1-1.5 k elements) is compacted into 8-byte candidate slots - (magnitude
+// bits, 4095 - index, sign) - and bitonic-sorted.  If more than 128 elements pass, an exact
+// bitwise search for the k-th largest magnitude runs instead (rare: constant or all-zero
+// chunks, pathological ties).  The only LDS needed besides the 128 slots is a 32-row staging
+// buffer through which each half of the wave reads its own row with a run-time index.
+// NaN payload bits are not kept: a selected NaN comes out as the quiet NaN of its sign.
 // ---------------------------------------------------------------------------------------
 struct Selected {
     uint32_t idx0, idx1;
@@ -323,105 +336,107 @@ __device__ __forceinline__ void sort128_desc(uint64_t& e0, uint64_t& e1, int) { 
 
 // `out_scale` multiplies the gathered values (an exact power of two left over by the caller's
 // transform; the ordering is taken on the unscaled values).
+// `buf` is a kHalfFloats staging buffer, `cand` kCandCap slots; both are free on return.
 template <bool kTwo>
-__device__ __forceinline__ Selected select_topk(const float (&v)[64], float* tile, int lane, int k,
+__device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf, uint64_t* cand, int lane, int k,
                                                 float out_scale) {
-    uint32_t b1, b2;
-    lane_stats<kTwo>(v, b1, b2);
-    const uint32_t t0 = stat_threshold<kTwo>(b1, b2, k);
-    uint32_t mhi, mlo;
-    filter_masks(v, __uint_as_float(t0), mhi, mlo);
-    uint32_t cnt = __popc(mhi) + __popc(mlo);
-    uint32_t total = wave_sum_u32(cnt);
+    uint32_t mhi = 0, mlo = 0, cnt = 0, incl = 0, total = 0;
+    {
+        uint32_t b1, b2;
+        lane_stats<kTwo>(w, b1, b2);
+        const uint32_t t0 = stat_threshold<kTwo>(b1, b2, k);
+        filter_masks(w, __uint_as_float(t0), mhi, mlo);
+        cnt = __popc(mhi) + __popc(mlo);
+        incl = wave_incl_scan_u32(cnt);
+        total = __builtin_amdgcn_readlane(incl, 63);
 
-    if (total > static_cast<uint32_t>(kCandCap) || total < static_cast<uint32_t>(k)) {
-        // Exact search for the k-th largest key, from the bits t0 and the maximum share.
-        const uint32_t vmax = wave_max_u32(mag_key(b1));
-        uint32_t t = mag_key(t0);
-        uint32_t n_ge = count_ge(v, t);
-        if (n_ge > static_cast<uint32_t>(kCandCap)) {
-            const uint32_t diff = t ^ vmax;
-            const int top = diff ? 31 - __builtin_clz(diff) : -1;
-            t = top >= 0 ? (t & ~((2u << top) - 1u)) : t;
+        if (total > static_cast<uint32_t>(kCandCap) || total < static_cast<uint32_t>(k)) {
+            // Exact search for the k-th largest key, from the bits t0 and the maximum share.
+            const uint32_t vmax = wave_max_u32(mag_key(b1));
+            uint32_t t = mag_key(t0);
+            uint32_t n_ge = count_ge(w, t);
+            if (n_ge > static_cast<uint32_t>(kCandCap)) {
+                const uint32_t diff = t ^ vmax;
+                const int top = diff ? 31 - __builtin_clz(diff) : -1;
+                t = top >= 0 ? (t & ~((2u << top) - 1u)) : t;
 #pragma nounroll
-            for (int bit = top; bit >= 0; --bit) {
-                const uint32_t c = t | (1u << bit);
-                const uint32_t n = count_ge(v, c);
-                if (n >= static_cast<uint32_t>(k)) {
-                    t = c;
-                    n_ge = n;
-                    if (n <= static_cast<uint32_t>(kCandCap)) break;
+                for (int bit = top; bit >= 0; --bit) {
+                    const uint32_t c = t | (1u << bit);
+                    const uint32_t n = count_ge(w, c);
+                    if (n >= static_cast<uint32_t>(k)) {
+                        t = c;
+                        n_ge = n;
+                        if (n <= static_cast<uint32_t>(kCandCap)) break;
+                    }
                 }
             }
-        }
-        uint32_t ghi, glo, ehi, elo;
-        exact_masks(v, t, ghi, glo, ehi, elo);
-        if (n_ge > static_cast<uint32_t>(kCandCap)) {
-            // more ties at the threshold than slots: take the lowest-index ties only
-            const uint32_t g = wave_sum_u32(__popc(ghi) + __popc(glo));
-            const uint32_t ties = __popc(ehi) + __popc(elo);
-            uint32_t incl = ties;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const uint32_t o = __shfl_up(incl, off);
-                if (lane >= off) incl += o;
+            uint32_t ghi, glo, ehi, elo;
+            exact_masks(w, t, ghi, glo, ehi, elo);
+            if (n_ge > static_cast<uint32_t>(kCandCap)) {
+                // more ties at the threshold than slots: take the lowest-index ties only
+                const uint32_t g = wave_sum_u32(__popc(ghi) + __popc(glo));
+                const uint32_t ties = __popc(ehi) + __popc(elo);
+                const uint32_t tincl = wave_incl_scan_u32(ties);
+                const int need = k - static_cast<int>(g);
+                const int before = static_cast<int>(tincl - ties);
+                int keep = need - before;
+                keep = keep < 0 ? 0 : keep;
+                keep_first(ehi, elo, keep);
             }
-            const int need = k - static_cast<int>(g);
-            const int before = static_cast<int>(incl - ties);
-            int keep = need - before;
-            keep = keep < 0 ? 0 : keep;
-            keep_first(ehi, elo, keep);
+            mhi = ghi | ehi;
+            mlo = glo | elo;
+            cnt = __popc(mhi) + __popc(mlo);
+            incl = wave_incl_scan_u32(cnt);
+            total = __builtin_amdgcn_readlane(incl, 63);
         }
-        mhi = ghi | ehi;
-        mlo = glo | elo;
-        cnt = __popc(mhi) + __popc(mlo);
-        total = wave_sum_u32(cnt);
     }
+    uint32_t slot = incl - cnt;  // exclusive prefix of the per-lane counts
 
-    // exclusive prefix of the per-lane counts
-    uint32_t incl = cnt;
+    // compaction: each half of the wave in turn parks its rows in the staging buffer, so that a
+    // lane can fetch its own candidates with a run-time column index
+    float* row = buf + (lane & 31) * kLd;
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const uint32_t o = __shfl_up(incl, off);
-        if (lane >= off) incl += o;
+    for (int half = 0; half < 2; ++half) {
+        if ((lane >> 5) == half) {
+            regs_to_tile_rows(w, buf, lane & 31);
+            while (mhi | mlo) {
+                const bool hi = mhi != 0;
+                const uint32_t m = hi ? mhi : mlo;
+                const int z = __builtin_clz(m);
+                const uint32_t cleared = m & ~(0x80000000u >> z);
+                mhi = hi ? cleared : mhi;
+                mlo = hi ? mlo : cleared;
+                const int d = hi ? z : 32 + z;
+                const uint32_t bits = __float_as_uint(row[d]);
+                const uint32_t ix = lane * 64 + d;
+                cand[slot++] = (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - ix) << 1) | (bits >> 31);
+            }
+        }
+        wave_lds_fence();
     }
-    uint32_t slot = incl - cnt;
-
-    // compaction: (magnitude key, ~index) into the candidate slots
-    const float* row = tile + lane * kLd;
-    while (mhi) {
-        const int d = __builtin_clz(mhi);
-        mhi &= ~(0x80000000u >> d);
-        const uint32_t key = mag_key(__float_as_uint(row[d]));
-        *cand_slot(tile, slot++) = (static_cast<uint64_t>(key) << 32) | (0xffffffffu - (lane * 64 + d));
-    }
-    while (mlo) {
-        const int d = 32 + __builtin_clz(mlo);
-        mlo &= ~(0x80000000u >> (d - 32));
-        const uint32_t key = mag_key(__float_as_uint(row[d]));
-        *cand_slot(tile, slot++) = (static_cast<uint64_t>(key) << 32) | (0xffffffffu - (lane * 64 + d));
-    }
-    wave_lds_fence();
 
     Selected out;
     out.idx1 = 0;
     out.val1 = 0.0f;
+    uint64_t e0, e1 = 0ull;
     if (total <= 64) {
-        uint64_t e = lane < static_cast<int>(total) ? *cand_slot(tile, lane) : 0ull;
-        sort64_desc(e, lane);
-        out.idx0 = 0xffffffffu - static_cast<uint32_t>(e);
+        e0 = lane < static_cast<int>(total) ? cand[lane] : 0ull;
+        sort64_desc(e0, lane);
     } else {
-        uint64_t e0 = *cand_slot(tile, lane);
-        uint64_t e1 = lane + 64 < static_cast<int>(total) ? *cand_slot(tile, lane + 64) : 0ull;
+        e0 = cand[lane];
+        e1 = lane + 64 < static_cast<int>(total) ? cand[lane + 64] : 0ull;
         sort128_desc(e0, e1, lane);
-        out.idx0 = 0xffffffffu - static_cast<uint32_t>(e0);
-        out.idx1 = 0xffffffffu - static_cast<uint32_t>(e1);
     }
-    // lanes beyond k may hold padding (index 0xffffffff - 0 wraps to a huge value): clamp
-    out.idx0 &= 4095u;
-    out.idx1 &= 4095u;
-    out.val0 = tile[(out.idx0 >> 6) * kLd + (out.idx0 & 63)] * out_scale;
-    if (k > 64) out.val1 = tile[(out.idx1 >> 6) * kLd + (out.idx1 & 63)] * out_scale;
+    // a slot unpacks to index, and to the value itself: sign bit on top of the magnitude bits
+    auto unpack = [&](uint64_t e, uint32_t& ix, float& val) {
+        const uint32_t lo = static_cast<uint32_t>(e), key = static_cast<uint32_t>(e >> 32);
+        ix = 4095u - ((lo >> 1) & 4095u);
+        const uint32_t mag = key == 0x7fffffffu ? 0x7fc00000u : key;
+        val = __uint_as_float(mag | (lo << 31)) * out_scale;
+    };
+    unpack(e0, out.idx0, out.val0);
+    if (k > 64) unpack(e1, out.idx1, out.val1);
+    wave_lds_fence();
     return out;
 }
 

@@ -114,37 +114,28 @@ __device__ __forceinline__ void store_chunk_cols(const float (&v)[64], float* __
 
 // forward 2-D transform of the chunk held column-per-lane; result row-per-lane:
 // v[d] = coef[lane][d], and the tile is left free
-struct NoHook {
-    __device__ __forceinline__ void operator()() const {}
-};
-
-// Forward 2-D transform of a chunk.  `in` holds it column-per-lane (in[r] = X[r][lane]); the
-// result is row-per-lane in v (v[d] = 32 * coef[lane][d] with the transform, X[lane][d]
-// without) and the tile is left free.  `in` is dead after the first butterfly level, which is
-// when after_inputs() runs (the caller starts refilling it there); between_passes() runs after
-// the first pass.
-template <bool kUseDct, typename Hook1 = NoHook, typename Hook2 = NoHook>
-__device__ __forceinline__ void chunk_forward(const float (&in)[64], float (&v)[64], float* tile, int lane,
-                                              Hook1 after_inputs = Hook1(), Hook2 between_passes = Hook2()) {
-    if (kUseDct) {
-        dct64_fwd_head(in, v);  // along rows k: v[b] = sum_k X[k][lane] F[k][b]
-    } else {
+// registers column-per-lane (v[r] = M[r][lane]) -> registers row-per-lane (w[c] = M[lane][c])
+// through a 32-row staging buffer: rows 0..31 go first and lanes 0..31 pick theirs up, then rows
+// 32..63 for lanes 32..63.  Half the LDS of a whole-chunk tile, which is what lets twice as many
+// waves stay resident.
+__device__ __forceinline__ void transpose_via_half(const float (&v)[64], float (&w)[64], float* buf, int lane) {
 #pragma unroll
-        for (int r = 0; r < 64; ++r) v[r] = in[r];
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+        for (int r = 0; r < kHalfRows; ++r) buf[r * kLd + lane] = v[half * kHalfRows + r];
+        wave_lds_fence();
+        if ((lane >> 5) == half) tile_rows_to_regs(w, buf, lane & 31);
+        wave_lds_fence();
     }
-    // pin the hooks' memory requests to their place in the instruction stream
-    asm volatile("" : "+v"(v[0]), "+v"(v[31]), "+v"(v[63])::"memory");
-    after_inputs();
-    asm volatile("" ::: "memory");
-    if (kUseDct) dct64_fwd_tail(v);
-    asm volatile("" : "+v"(v[1]), "+v"(v[31]), "+v"(v[63])::"memory");
-    between_passes();
-    asm volatile("" ::: "memory");
-    regs_to_tile_cols(v, tile, lane);
-    wave_lds_fence();
-    tile_rows_to_regs(v, tile, lane);
-    if (kUseDct) dct64_fwd(v);  // along columns l: v[d] = sum_l T[lane][l] F[l][d]
-    wave_lds_fence();
+}
+
+// Forward 2-D transform of a chunk held column-per-lane (v[r] = X[r][lane]); the result is
+// row-per-lane: w[d] = 32 * coef[lane][d] with the transform, X[lane][d] without.
+template <bool kUseDct>
+__device__ __forceinline__ void chunk_forward(float (&v)[64], float (&w)[64], float* buf, int lane) {
+    if (kUseDct) dct64_fwd(v);  // along rows k: v[b] = sum_k X[k][lane] F[k][b]
+    transpose_via_half(v, w, buf, lane);
+    if (kUseDct) dct64_fwd(w);  // along columns l: w[d] = sum_l T[lane][l] F[l][d]
 }
 
 // inverse: tile holds coef rows; result column-per-lane v[k] = x[k][lane]
@@ -273,12 +264,12 @@ __global__ __launch_bounds__(64) void k_dct2d_fwd(const float* __restrict__ x, i
     const int64_t chunk = xcd_contiguous(blockIdx.x, gridDim.x);
     if (chunk >= n_chunks) return;
     const int64_t y = chunk / X, xc = chunk - y * X;
-    float in[64], v[64];
-    load_chunk_cols(in, x, ld, y, xc, lane);
-    chunk_forward<true>(in, v, tile, lane);
+    float v[64], w[64];
+    load_chunk_cols(v, x, ld, y, xc, lane);
+    chunk_forward<true>(v, w, tile, lane);
 #pragma unroll
-    for (int d = 0; d < 64; ++d) v[d] *= kDctPow2Scale;  // exact: 32x the orthonormal transform so far
-    regs_to_tile_rows(v, tile, lane);
+    for (int d = 0; d < 64; ++d) w[d] *= kDctPow2Scale;  // exact: 32x the orthonormal transform so far
+    regs_to_tile_rows(w, tile, lane);
     __syncthreads();
     tile_to_flat(tile, coef + chunk * 4096, lane);
 }
@@ -381,6 +372,7 @@ template <bool kTwo>
 __global__ __launch_bounds__(64) void k_topk_rows(const float* __restrict__ coef, int64_t n_rows, int row_len,
                                                   int k, uint8_t* __restrict__ idx12, float* __restrict__ val) {
     __shared__ __align__(16) float tile[kTileFloats];
+    __shared__ uint64_t cand[kCandCap];
     const int lane = threadIdx.x;
     const int64_t row = xcd_contiguous(blockIdx.x, gridDim.x);
     if (row >= n_rows) return;
@@ -395,58 +387,38 @@ __global__ __launch_bounds__(64) void k_topk_rows(const float* __restrict__ coef
         }
     }
     __syncthreads();
-    float v[64];
-    tile_rows_to_regs(v, tile, lane);
-    const Selected s = select_topk<kTwo>(v, tile, lane, k, 1.0f);
+    float w[64];
+    tile_rows_to_regs(w, tile, lane);
+    __syncthreads();
+    const Selected s = select_topk<kTwo>(w, tile, cand, lane, k, 1.0f);
     emit_selected(s, lane, k, row, idx12, val);
 }
 
-// Persistent fused encode: every wave walks its slice of the chunk list; the 64 row loads of
-// the next chunk are in flight while the current one is transformed and selected.
+// Persistent fused encode: every wave walks its slice of the chunk list.  The kernel is bound by
+// vector-ALU issue and by the latencies between its phases, so it is shaped for residency -
+// 8.5 KB + 1 KB of LDS and a register budget that admits three to four waves per SIMD - and
+// leaves the overlap of one wave's row loads with the other waves' arithmetic to the hardware.
 template <bool kTwo, bool kUseDct>
-__global__ __launch_bounds__(64, 2) void k_encode_topk_pack(const tplr_tensor_desc* __restrict__ table,
-                                                         const tplr_tensor_desc single, int n_tensors,
-                                                         int64_t total, int k, uint8_t* __restrict__ idx12,
-                                                         float* __restrict__ val) {
-    __shared__ __align__(16) float tile[kTileFloats];
+__global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_desc* __restrict__ table,
+                                                            const tplr_tensor_desc single, int n_tensors,
+                                                            int64_t total, int k, uint8_t* __restrict__ idx12,
+                                                            float* __restrict__ val) {
+    __shared__ __align__(16) float buf[kHalfFloats];
+    __shared__ uint64_t cand[kCandCap];
     const int lane = threadIdx.x;
     int64_t g0, g1;
     my_range(total, g0, g1);
     if (g0 >= g1) return;
     Cursor c;
     cursor_seek(c, table, single, n_tensors, g0);
-    // Loads and stores share one completion counter and complete out of order with respect to
-    // each other, so a wait for the prefetched rows also waits for every store issued before it.
-    // The selection of chunk g is therefore written in the middle of iteration g + 1, a
-    // transform pass away from the waits on either side.  The rows of chunk g + 1 land in the
-    // registers chunk g was read from, which its first butterfly level has freed.
-    float v[64], nx[64];
-    load_chunk_cols(nx, c, lane);
-    Selected prev = {};
     for (int64_t g = g0; g < g1; ++g) {
-        // at most 63 vector-memory operations can be outstanding: most rows of the next chunk are
-        // requested as soon as the first butterfly level has consumed this chunk's registers, the
-        // previous selection is written and the last rows requested after the first pass
-        constexpr int kSplit = 56;
-        const bool more = g + 1 < g1;
-        chunk_forward<kUseDct>(
-            nx, v, tile, lane,
-            [&]() {
-                if (more) {
-                    cursor_next(c, g + 1);
-                    load_chunk_cols<0, kSplit>(nx, c, lane);
-                }
-            },
-            [&]() {
-                if (g > g0) emit_selected(prev, lane, k, g - 1, idx12, val);
-                if (more) load_chunk_cols<kSplit, 64>(nx, c, lane);
-            });
-        regs_to_tile_rows(v, tile, lane);
-        wave_lds_fence();
-        prev = select_topk<kTwo>(v, tile, lane, k, kUseDct ? kDctPow2Scale : 1.0f);
-        wave_lds_fence();
+        float v[64], w[64];
+        load_chunk_cols(v, c, lane);
+        if (g + 1 < g1) cursor_next(c, g + 1);
+        chunk_forward<kUseDct>(v, w, buf, lane);
+        const Selected s = select_topk<kTwo>(w, buf, cand, lane, k, kUseDct ? kDctPow2Scale : 1.0f);
+        emit_selected(s, lane, k, g, idx12, val);
     }
-    emit_selected(prev, lane, k, g1 - 1, idx12, val);
 }
 
 // =========================================================================================
