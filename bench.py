@@ -36,13 +36,14 @@ HBM_PEAK_GBPS = 8000.0
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg3_llama1b", help="cfg1_2048x2048 | cfg2_llama150m | cfg3_llama1b | cfg5_72b_block")
     ap.add_argument("--peers", type=int, default=15)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--profile", choices=["encode", "aggregate"], default=None,
-                    help="run only that phase's batched launches --steps times (for rocprofv3) and print nothing")
+    ap.add_argument("--profile", choices=["encode", "aggregate", "copy"], default=None,
+                    help="run only that phase's batched launches --steps times (for rocprofv3) and print nothing; "
+                         "'copy' runs the library's calibration copy of 1 GiB instead (counter scaling)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline sample")
     return ap.parse_args()
 
@@ -144,6 +145,17 @@ def main():
     import workloads
 
     dev = torch.device("cuda:0")
+    if args.profile == "copy":
+        from templar_amd import _lib
+
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB
+        dst = torch.empty_like(src)
+        lib = _lib.load()
+        event_ms(lambda: _lib.check(lib.tplr_calib_copy(src.data_ptr(), dst.data_ptr(), src.numel() * 4,
+                                                        torch.cuda.current_stream().cuda_stream), "calib_copy"),
+                 args.steps, args.warmup)
+        assert torch.equal(src, dst)
+        return
     cfg = workloads.CONFIGS[args.workload]
     k, shapes = cfg["k"], cfg["shapes"]
     P = args.peers

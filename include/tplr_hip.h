@@ -185,6 +185,11 @@ int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr
 int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int is_sumsq, float* d_scale,
                            float* d_median, void* stream);
 
+/* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes
+ * (a multiple of 16, both pointers 16-byte aligned) that moves exactly n_bytes each way.
+ * Profilers' HBM traffic counters are scaled by what they report for this kernel. */
+int tplr_calib_copy(const void* d_src, void* d_dst, int64_t n_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -29,7 +29,7 @@ values only (encode) or folded into the scalar clip factor (decode).
 The inverse transform is the transposed flow graph run backwards.
 
 Functions written: dct64_fwd_head (the 32 input butterflies, from a separate
-input array - it lets the caller start refilling that array right after),
+input array),
 dct64_fwd_tail, dct64_fwd (both), dct64_inv.  Run as a build step
 (`python gen_dct64.py`); `--check` only verifies and prints op counts.
 """

@@ -817,6 +817,14 @@ __global__ __launch_bounds__(128) void k_clip_scales(const float* __restrict__ n
     if (i == 0 && median) median[blockIdx.x] = med;
 }
 
+// Plain streaming copy (16 bytes per lane per step, grid-stride).  It exists so that hardware
+// traffic counters can be calibrated: it moves exactly n16 * 16 bytes each way.
+typedef float v4f __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void k_calib_copy(const v4f* __restrict__ src, v4f* __restrict__ dst, int64_t n16) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
 }  // namespace tplr
 
 // =========================================================================================
@@ -1171,6 +1179,15 @@ int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr
     }
     hipLaunchKernelGGL(k_segment_sumsq, dim3(static_cast<unsigned>(n_tensors) * n_peers), dim3(256), 0,
                        static_cast<hipStream_t>(stream), vp, n_peers, k, d_desc, d_sumsq);
+    return launch_status();
+}
+
+int tplr_calib_copy(const void* d_src, void* d_dst, int64_t n_bytes, void* stream) {
+    if (!d_src || !d_dst || n_bytes < 0 || (n_bytes & 15)) return TPLR_E_BADARG;
+    if ((reinterpret_cast<uintptr_t>(d_src) | reinterpret_cast<uintptr_t>(d_dst)) & 15) return TPLR_E_BADARG;
+    if (n_bytes == 0) return 0;
+    hipLaunchKernelGGL(k_calib_copy, dim3(256 * 16), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const v4f*>(d_src), static_cast<v4f*>(d_dst), n_bytes >> 4);
     return launch_status();
 }
 

@@ -415,6 +415,17 @@ def test_bad_arguments_are_rejected(dev):
     assert b"even" in lib.tplr_status_string(_lib.TPLR_E_ODD)
 
 
+def test_calibration_copy(dev):
+    lib = _lib.load()
+    src = torch.arange(1 << 20, dtype=torch.float32, device=dev)
+    dst = torch.zeros_like(src)
+    assert lib.tplr_calib_copy(tc._ptr(src), tc._ptr(dst), src.numel() * 4, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst)
+    assert lib.tplr_calib_copy(tc._ptr(src), tc._ptr(dst), 24, None) == _lib.TPLR_E_BADARG
+    assert lib.tplr_calib_copy(tc._ptr(src), tc._ptr(dst), 0, None) == 0
+
+
 # ---------------------------------------------------------------- persistent loops and batches
 def test_persistent_encode_many_chunks_per_wave(dev):
     # 4608 chunks: more than one resident set of waves, so every wave walks several chunks
