@@ -462,8 +462,7 @@ struct Counters {
 // peer, so each address is a scalar base (peer pointer from the kernel arguments + chunk
 // offset) plus one lane-constant offset and each clip factor is a scalar; the whole payload of
 // a chunk sits in 2 * kUnits registers, is requested before the inverse transform of the
-// previous chunk and travels during it.  The scatter is straight-line: unused units (peer
-// index >= P) add 0 to a per-lane dummy slot in the tile's padding instead of branching.
+// previous chunk and travels during it.
 // Generic path (kUnits == 0): any k and peer count, entries loaded where they are used.
 //
 // Loads and stores complete out of order with respect to each other on one counter, so the 64
@@ -490,7 +489,6 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     const float out_scale = kUseDct ? kDctPow2Scale : 1.0f;
     const int lane_ioff = 3 * (lane >> 1) + (lane & 1);  // byte offset of entry `lane` in a packed row
     const bool lane_on = lane < k;                       // fast path: this lane owns an entry
-    const int dummy_pos = lane * kLd + kChunk;           // per-lane padding slot
 
     uint32_t ix[kRegs];
     float a[kRegs], sc[kRegs];
@@ -560,29 +558,23 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
         wave_lds_fence();
 
-        // ---- scatter: sums in peer order, contribution counts; `seen` collects the old counts
-        uint32_t seen = 0;
+        // ---- scatter: sums in peer order and contribution counts.  One instruction carries one
+        // peer's entries, whose destinations are distinct, and LDS instructions of a wave execute in
+        // order, so every destination receives its contributions in peer order.  Nothing is
+        // returned: the adds are fire-and-forget.
         auto add_entry = [&](uint32_t ixe, float val) {
             atomicAdd(&tile[tile_pos(ixe)], val);
-            const uint32_t sh = Cnt::shift(ixe);
-            seen |= (atomicAdd(&cnt[Cnt::word(ixe)], 1u << sh) >> sh) & Cnt::kMask;
+            atomicAdd(&cnt[Cnt::word(ixe)], 1u << Cnt::shift(ixe));
         };
         if (fast) {
             if (lane_on) {
-                uint32_t old[kRegs];
 #pragma unroll
                 for (int i = 0; i < kRegs; ++i) {
-                    const bool on = i < P;  // wave-uniform
-                    const uint32_t e = (lane & 1) ? (ix[i] >> 4) : (ix[i] & 0xfffu);
-                    ix[i] = e;  // decoded index, kept for the mean pass
-                    atomicAdd(&tile[on ? tile_pos(e) : dummy_pos], on ? a[i] * sc[i] : 0.f);
-                    old[i] = atomicAdd(&cnt[on ? Cnt::word(e) : lane], on ? (1u << Cnt::shift(e)) : 0u);
+                    if (i < P) {  // wave-uniform
+                        const uint32_t e = (lane & 1) ? (ix[i] >> 4) : (ix[i] & 0xfffu);
+                        add_entry(e, a[i] * sc[i]);
+                    }
                 }
-                // the returned counts are only looked at once every add has been issued
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int i = 0; i < kRegs; ++i)
-                    if (i < P) seen |= (old[i] >> Cnt::shift(ix[i])) & Cnt::kMask;
             }
         } else if (normalise) {
             // per-peer, per-chunk L2 normalisation (compress.py:541-545); simple, unbatched
@@ -611,40 +603,35 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
         wave_lds_fence();
 
-        // ---- mean: exactly one entry per destination claims the counter and divides the sum
-        if (reduce_mode == TPLR_REDUCE_MEAN && __any(seen != 0)) {
-            auto claim = [&](uint32_t ixe) -> uint32_t {
-                const uint32_t sh = Cnt::shift(ixe);
-                return (atomicAnd(&cnt[Cnt::word(ixe)], ~(Cnt::kMask << sh)) >> sh) & Cnt::kMask;
-            };
-            auto divide = [&](uint32_t ixe, uint32_t n) {
-                if (n > 1) {
-                    float* t = &tile[tile_pos(ixe)];
-                    *t = *t / static_cast<float>(n);
-                }
-            };
-            if (fast) {
-                if (lane_on) {
-                    uint32_t n_claimed[kRegs];
+        // ---- mean: lane r scans the counters of row r and divides the coefficients that received
+        // more than one contribution (a few per row), one per trip of a lane-divergent loop
+        if (reduce_mode == TPLR_REDUCE_MEAN) {
+            constexpr int kRowWords = kChunk / Cnt::kPerWord;
+            constexpr uint32_t kMulti = kCntBits == 4 ? 0xEEEEEEEEu : 0xFEFEFEFEu;  // count >= 2
+            const uint32_t* crow = cnt + lane * kRowWords;
+            uint32_t todo = 0;  // bit q: word q of the row holds such a counter
 #pragma unroll
-                    for (int i = 0; i < kRegs; ++i) {
-                        const bool on = i < P;
-                        const uint32_t sh = Cnt::shift(ix[i]);
-                        n_claimed[i] = atomicAnd(&cnt[on ? Cnt::word(ix[i]) : lane], on ? ~(Cnt::kMask << sh) : ~0u);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int i = 0; i < kRegs; ++i)
-                        if (i < P) divide(ix[i], (n_claimed[i] >> Cnt::shift(ix[i])) & Cnt::kMask);
+            for (int q4 = 0; q4 < kRowWords / 4; ++q4) {
+                const uint4 t = reinterpret_cast<const uint4*>(crow)[q4];
+                todo |= ((t.x & kMulti) ? 1u : 0u) << (4 * q4);
+                todo |= ((t.y & kMulti) ? 2u : 0u) << (4 * q4);
+                todo |= ((t.z & kMulti) ? 4u : 0u) << (4 * q4);
+                todo |= ((t.w & kMulti) ? 8u : 0u) << (4 * q4);
+            }
+            uint32_t word = 0, m = 0;
+            int q = 0;
+            while (todo | m) {
+                if (m == 0) {
+                    q = __builtin_ctz(todo);
+                    todo &= todo - 1;
+                    word = crow[q];
+                    m = word & kMulti;
                 }
-            } else {
-                for (int p = 0; p < P; ++p)
-                    for (int j = lane; j < k; j += 64) {
-                        uint32_t ixe;
-                        float ae;
-                        load_entry(p, j, g, ixe, ae);
-                        divide(ixe, claim(ixe));
-                    }
+                const int slot = __builtin_ctz(m) / kCntBits;
+                const uint32_t n = (word >> (slot * kCntBits)) & Cnt::kMask;
+                m &= ~(Cnt::kMask << (slot * kCntBits));
+                float* t = &tile[lane * kLd + q * Cnt::kPerWord + slot];
+                *t = *t / static_cast<float>(n);
             }
             wave_lds_fence();
         }
