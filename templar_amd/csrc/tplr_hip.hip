@@ -455,19 +455,14 @@ struct Counters {
 };
 
 // Persistent fused decode.  Per chunk, the peers' entries are accumulated in peer order into an
-// LDS tile (sums) and a per-coefficient contribution count; touched coefficients are
-// divided by their count; the tile goes through the inverse 2-D DCT.
+// LDS tile (sums) and a per-coefficient contribution count; coefficients with several
+// contributions are divided by their count; the tile goes through the inverse 2-D DCT.
 //
 // Fast path (kUnits > 0: k <= 64 and at most kUnits peers): lane j handles entry j of every
 // peer, so each address is a scalar base (peer pointer from the kernel arguments + chunk
 // offset) plus one lane-constant offset and each clip factor is a scalar; the whole payload of
-// a chunk sits in 2 * kUnits registers, is requested before the inverse transform of the
-// previous chunk and travels during it.
+// a chunk sits in 2 * kUnits registers and is requested a whole transform pass before it is used.
 // Generic path (kUnits == 0): any k and peer count, entries loaded where they are used.
-//
-// Loads and stores complete out of order with respect to each other on one counter, so the 64
-// row stores of chunk g are issued at the top of iteration g + 1, after the wait for that
-// chunk's payload registers and a whole iteration before the next wait.
 template <bool kUseDct, int kUnits, int kCntBits>
 __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
@@ -487,25 +482,39 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     const int64_t idx_stride = k + (k >> 1);
     // the inverse transform below is 32x the orthonormal one: its input carries the exact 2^-5
     const float out_scale = kUseDct ? kDctPow2Scale : 1.0f;
-    const int lane_ioff = 3 * (lane >> 1) + (lane & 1);  // byte offset of entry `lane` in a packed row
-    const bool lane_on = lane < k;                       // fast path: this lane owns an entry
+    const bool lane_on = lane < k;       // fast path: this lane owns an entry
+    const int le = lane_on ? lane : 0;   // the other lanes reload entry 0 and stay out of the scatter
+    const int lane_ioff = 3 * (le >> 1) + (le & 1);  // byte offset of entry `le` in a packed row
+
+    // Fast path: lane p keeps peer p's two payload pointers and its clip factor for the current
+    // tensor in registers; unit i gets them as scalars through v_readlane, so that the steady
+    // state of the loop contains no scalar memory load (whose wait would also drain the LDS queue).
+    const int pl = lane < P ? lane : P - 1;
+    const uint64_t my_idx = kFast ? reinterpret_cast<uint64_t>(pp.idx[pl]) : 0;
+    const uint64_t my_val = kFast ? reinterpret_cast<uint64_t>(pp.val[pl]) : 0;
+    float my_scale = out_scale;
+    int t_scale = -1;  // tensor whose clip factors my_scale holds
+    auto lane_bcast64 = [&](uint64_t mine, int i) -> uint64_t {
+        const uint32_t lo = __builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(mine)), i);
+        const uint32_t hi = __builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(mine >> 32)), i);
+        return (static_cast<uint64_t>(hi) << 32) | lo;
+    };
 
     uint32_t ix[kRegs];
-    float a[kRegs], sc[kRegs];
+    float a[kRegs];
 
     auto load_payload = [&](int64_t g, int t) {  // fast path only
+        if (scale && t != t_scale) {  // wave-uniform, once per tensor
+            my_scale = scale[static_cast<int64_t>(t) * P + pl] * out_scale;
+            t_scale = t;
+        }
 #pragma unroll
         for (int i = 0; i < kRegs; ++i) {
-            const int p = i < P ? i : P - 1;  // unused units read the last peer and are masked later
-            const gbyte* irow = (const gbyte*)pp.idx[p] + g * idx_stride;  // wave-uniform
-            const gfloat* vrow = (const gfloat*)pp.val[p] + g * k;
-            sc[i] = (scale ? scale[static_cast<int64_t>(t) * P + p] : 1.0f) * out_scale;
-            ix[i] = 0;
-            a[i] = 0.f;
-            if (lane_on) {
-                ix[i] = *(const gu16*)(irow + lane_ioff);
-                a[i] = vrow[lane];
-            }
+            const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
+            const gbyte* irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
+            const gfloat* vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
+            ix[i] = *(const gu16*)(irow + lane_ioff);
+            a[i] = vrow[le];
         }
     };
     // entry j of peer p of chunk g (generic path and normalise)
@@ -516,63 +525,42 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         ao = ((const gfloat*)pp.val[p] + g * k)[j];
     };
 
-    Cursor c;
-    cursor_seek(c, table, single, n_tensors, g0);
     const bool fast = kFast && !normalise;
-    if (fast) load_payload(g0, c.t);
 
-    float v[64];  // inverse transform of the previous chunk, stored one iteration late
-    gfloat* prev_chunk0 = nullptr;
-    int64_t prev_ld = 0;
-    float prev_ss = 0.f;
-
-    for (int64_t g = g0; g < g1; ++g) {
-        // the payload registers must have arrived BEFORE the previous chunk's stores are issued:
-        // a later wait for them would also wait for those stores
-        if (kFast) {
+    auto zero_tile = [&]() {
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        float4* row = reinterpret_cast<float4*>(tile + lane * kLd);
 #pragma unroll
-            for (int i = 0; i < kRegs; ++i) asm volatile("" : "+v"(ix[i]), "+v"(a[i]));
-        }
-        if (g > g0) {
-            if (kUseDct)
-                store_chunk_rows(v, (void*)prev_chunk0, prev_ld, lane);
-            else
-                tile_to_flat(tile, (float*)prev_chunk0, lane);
-            if (sumsq && lane == 0) sumsq[g - 1] = prev_ss;
-            wave_lds_fence();
-        }
-        // where this chunk's result goes (the cursor moves on before the store)
-        const int t_now = c.t;
-        prev_ld = c.ld;
-        prev_chunk0 = kUseDct ? c.base + (c.y * 64) * c.ld + static_cast<int64_t>(c.xc) * 64
-                              : c.base + (g - c.begin) * 4096;
-
-        {
-            const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-            float4* row = reinterpret_cast<float4*>(tile + lane * kLd);
+        for (int q = 0; q < 16; ++q) row[q] = z;
+        const uint4 zi = make_uint4(0, 0, 0, 0);
 #pragma unroll
-            for (int q = 0; q < 16; ++q) row[q] = z;
-            const uint4 zi = make_uint4(0, 0, 0, 0);
-#pragma unroll
-            for (int q = 0; q < Cnt::kWords / 256; ++q) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
-        }
+        for (int q = 0; q < Cnt::kWords / 256; ++q) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
         wave_lds_fence();
+    };
 
-        // ---- scatter: sums in peer order and contribution counts.  One instruction carries one
-        // peer's entries, whose destinations are distinct, and LDS instructions of a wave execute in
-        // order, so every destination receives its contributions in peer order.  Nothing is
-        // returned: the adds are fire-and-forget.
-        auto add_entry = [&](uint32_t ixe, float val) {
-            atomicAdd(&tile[tile_pos(ixe)], val);
-            atomicAdd(&cnt[Cnt::word(ixe)], 1u << Cnt::shift(ixe));
-        };
+    // ---- scatter: sums in peer order and contribution counts.  One instruction carries one
+    // peer's entries, whose destinations are distinct (a top-k selection has no duplicates), and
+    // LDS instructions of a wave execute in order, so every destination receives its
+    // contributions in peer order.  The fast path therefore needs no atomic for the sums; the
+    // generic path keeps them.
+    auto add_entry = [&](uint32_t ixe, float val) {
+        atomicAdd(&tile[tile_pos(ixe)], val);
+        atomicAdd(&cnt[Cnt::word(ixe)], 1u << Cnt::shift(ixe));
+    };
+    auto scatter = [&](int64_t g, int t_now) {
         if (fast) {
             if (lane_on) {
 #pragma unroll
                 for (int i = 0; i < kRegs; ++i) {
                     if (i < P) {  // wave-uniform
                         const uint32_t e = (lane & 1) ? (ix[i] >> 4) : (ix[i] & 0xfffu);
-                        add_entry(e, a[i] * sc[i]);
+                        const float x = a[i] * __builtin_bit_cast(float, __builtin_amdgcn_readlane(
+                                                   __builtin_bit_cast(int, my_scale), i));
+                        // plain read-add-write: the floating-point LDS atomic costs about 3 cycles
+                        // per lane, six times this sequence
+                        float* t = &tile[tile_pos(e)];
+                        *t = *t + x;
+                        atomicAdd(&cnt[Cnt::word(e)], 1u << Cnt::shift(e));
                     }
                 }
             }
@@ -601,72 +589,130 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 }
             }
         }
+    };
+
+    // ---- mean: lane r scans the counters of row r and divides the coefficients that received
+    // more than one contribution (a few per row), one per trip of a lane-divergent loop
+    auto mean_pass = [&]() {
         wave_lds_fence();
-
-        // ---- mean: lane r scans the counters of row r and divides the coefficients that received
-        // more than one contribution (a few per row), one per trip of a lane-divergent loop
-        if (reduce_mode == TPLR_REDUCE_MEAN) {
-            constexpr int kRowWords = kChunk / Cnt::kPerWord;
-            constexpr uint32_t kMulti = kCntBits == 4 ? 0xEEEEEEEEu : 0xFEFEFEFEu;  // count >= 2
-            const uint32_t* crow = cnt + lane * kRowWords;
-            uint32_t todo = 0;  // bit q: word q of the row holds such a counter
+        if (reduce_mode != TPLR_REDUCE_MEAN) return;
+        constexpr int kRowWords = kChunk / Cnt::kPerWord;
+        constexpr uint32_t kMulti = kCntBits == 4 ? 0xEEEEEEEEu : 0xFEFEFEFEu;  // count >= 2
+        const uint32_t* crow = cnt + lane * kRowWords;
+        uint32_t todo = 0;  // bit q: word q of the row holds such a counter
 #pragma unroll
-            for (int q4 = 0; q4 < kRowWords / 4; ++q4) {
-                const uint4 t = reinterpret_cast<const uint4*>(crow)[q4];
-                todo |= ((t.x & kMulti) ? 1u : 0u) << (4 * q4);
-                todo |= ((t.y & kMulti) ? 2u : 0u) << (4 * q4);
-                todo |= ((t.z & kMulti) ? 4u : 0u) << (4 * q4);
-                todo |= ((t.w & kMulti) ? 8u : 0u) << (4 * q4);
-            }
-            uint32_t word = 0, m = 0;
-            int q = 0;
-            while (todo | m) {
-                if (m == 0) {
-                    q = __builtin_ctz(todo);
-                    todo &= todo - 1;
-                    word = crow[q];
-                    m = word & kMulti;
-                }
-                const int slot = __builtin_ctz(m) / kCntBits;
-                const uint32_t n = (word >> (slot * kCntBits)) & Cnt::kMask;
-                m &= ~(Cnt::kMask << (slot * kCntBits));
-                float* t = &tile[lane * kLd + q * Cnt::kPerWord + slot];
-                *t = *t / static_cast<float>(n);
-            }
-            wave_lds_fence();
+        for (int q4 = 0; q4 < kRowWords / 4; ++q4) {
+            const uint4 t = reinterpret_cast<const uint4*>(crow)[q4];
+            todo |= ((t.x & kMulti) ? 1u : 0u) << (4 * q4);
+            todo |= ((t.y & kMulti) ? 2u : 0u) << (4 * q4);
+            todo |= ((t.z & kMulti) ? 4u : 0u) << (4 * q4);
+            todo |= ((t.w & kMulti) ? 8u : 0u) << (4 * q4);
         }
-
-        // the next chunk's payload travels while this one goes through the inverse transform
-        if (g + 1 < g1) {
-            cursor_next(c, g + 1);
-            if (fast) load_payload(g + 1, c.t);
+        uint32_t word = 0, m = 0;
+        int q = 0;
+        while (todo | m) {
+            if (m == 0) {
+                q = __builtin_ctz(todo);
+                todo &= todo - 1;
+                word = crow[q];
+                m = word & kMulti;
+            }
+            const int slot = __builtin_ctz(m) / kCntBits;
+            const uint32_t n = (word >> (slot * kCntBits)) & Cnt::kMask;
+            m &= ~(Cnt::kMask << (slot * kCntBits));
+            float* t = &tile[lane * kLd + q * Cnt::kPerWord + slot];
+            *t = *t / static_cast<float>(n);
         }
+        wave_lds_fence();
+    };
 
+    // where a chunk's result goes
+    struct Out {
+        gfloat* chunk0;
+        int64_t ld;
+    };
+    auto out_of = [&](const Cursor& cu, int64_t g) -> Out {
+        return Out{kUseDct ? cu.base + (cu.y * 64) * cu.ld + static_cast<int64_t>(cu.xc) * 64
+                           : cu.base + (g - cu.begin) * 4096,
+                   cu.ld};
+    };
+
+    // The loop is software-pipelined over three chunks.  While chunk g is in registers for the
+    // second pass of its inverse transform (vector ALU only), the tile already receives the
+    // scatter of chunk g + 1, and the payload of chunk g + 2 is on its way from memory.
+    Cursor c;
+    cursor_seek(c, table, single, n_tensors, g0);
+    Out out_cur = out_of(c, g0), out_next = out_cur;
+    int t_next = c.t;
+    if (fast) load_payload(g0, c.t);
+    zero_tile();
+    scatter(g0, c.t);
+    mean_pass();
+    if (g0 + 1 < g1) {
+        cursor_next(c, g0 + 1);
+        out_next = out_of(c, g0 + 1);
+        t_next = c.t;
+        if (fast) load_payload(g0 + 1, c.t);
+    }
+
+    for (int64_t g = g0; g < g1; ++g) {
+        float v[64];
+        // ---- first half: everything that needs chunk g's coefficients in the tile
         if (kUseDct) {
-            chunk_inverse<true>(v, tile, lane);
-            if (sumsq) {
-                float ss = 0.f;
-#pragma unroll
-                for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
-                prev_ss = wave_sum_f32(ss);
-            }
-        } else if (sumsq) {
-            float ss = 0.f;
+            tile_rows_to_regs(v, tile, lane);
+            dct64_inv(v);  // along d: v[l] = sum_d Y[lane][d] F[l][d]
+            wave_lds_fence();
+            regs_to_tile_rows(v, tile, lane);
+            wave_lds_fence();
+            tile_cols_to_regs(v, tile, lane);
+        } else {
 #pragma unroll
             for (int q0 = 0; q0 < 16; ++q0) {
                 const int q = q0 * 64 + lane;
                 const float4 t = *reinterpret_cast<const float4*>(tile + (q >> 4) * kLd + ((q & 15) << 2));
-                ss += t.x * t.x + t.y * t.y + t.z * t.z + t.w * t.w;
+                v[4 * q0] = t.x, v[4 * q0 + 1] = t.y, v[4 * q0 + 2] = t.z, v[4 * q0 + 3] = t.w;
             }
-            prev_ss = wave_sum_f32(ss);
         }
         wave_lds_fence();
+
+        // ---- the tile is free: chunk g + 1 moves in, chunk g + 2 is requested
+        const bool more = g + 1 < g1;
+        Out out_after = out_next;
+        int t_after = t_next;
+        if (more) {
+            zero_tile();
+            scatter(g + 1, t_next);
+            if (g + 2 < g1) {
+                cursor_next(c, g + 2);
+                out_after = out_of(c, g + 2);
+                t_after = c.t;
+                if (fast) load_payload(g + 2, c.t);
+            }
+        }
+
+        // ---- second half of chunk g, in registers
+        if (kUseDct) dct64_inv(v);  // along b: v[k] = sum_b Z[b][lane] F[k][b]
+        float ss = 0.f;
+        if (sumsq) {
+#pragma unroll
+            for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
+            ss = wave_sum_f32(ss);
+        }
+        if (more) mean_pass();
+
+        if (kUseDct) {
+            store_chunk_rows(v, (void*)out_cur.chunk0, out_cur.ld, lane);
+        } else {
+#pragma unroll
+            for (int q0 = 0; q0 < 16; ++q0)
+                reinterpret_cast<float4*>((float*)out_cur.chunk0)[q0 * 64 + lane] =
+                    make_float4(v[4 * q0], v[4 * q0 + 1], v[4 * q0 + 2], v[4 * q0 + 3]);
+        }
+        if (sumsq && lane == 0) sumsq[g] = ss;
+        out_cur = out_next;
+        out_next = out_after;
+        t_next = t_after;
     }
-    if (kUseDct)
-        store_chunk_rows(v, (void*)prev_chunk0, prev_ld, lane);
-    else
-        tile_to_flat(tile, (float*)prev_chunk0, lane);
-    if (sumsq && lane == 0) sumsq[g1 - 1] = prev_ss;
 }
 
 // generic rows (1-D tensors, un-chunked 2-D rows): exact source-order accumulation
