@@ -700,12 +700,15 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
         if (more) mean_pass();
 
+        // (the loop-carried destination may have been parked in vector registers: make it scalar
+        // again, or every store becomes a loop over distinct descriptors)
+        gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0));
         if (kUseDct) {
-            store_chunk_rows(v, (void*)out_cur.chunk0, out_cur.ld, lane);
+            store_chunk_rows(v, (void*)dst, uniform64(out_cur.ld), lane);
         } else {
 #pragma unroll
             for (int q0 = 0; q0 < 16; ++q0)
-                reinterpret_cast<float4*>((float*)out_cur.chunk0)[q0 * 64 + lane] =
+                reinterpret_cast<float4*>((float*)dst)[q0 * 64 + lane] =
                     make_float4(v[4 * q0], v[4 * q0 + 1], v[4 * q0 + 2], v[4 * q0 + 3]);
         }
         if (sumsq && lane == 0) sumsq[g] = ss;
