@@ -30,7 +30,8 @@ The inverse transform is the transposed flow graph run backwards.
 
 Functions written: dct64_fwd_head (the 32 input butterflies, from a separate
 input array),
-dct64_fwd_tail, dct64_fwd (both), dct64_inv.  Run as a build step
+dct64_fwd_tail, dct64_fwd (both), dct64_inv, and dct64_inv_hooked (dct64_inv
+with call-outs to a caller-supplied functor between its instructions).  Run as a build step
 (`python gen_dct64.py`); `--check` only verifies and prints op counts.
 """
 from __future__ import annotations
@@ -157,19 +158,31 @@ def lit(v):
 
 
 class Emitter:
-    def __init__(self, prefix):
-        self.lines, self.nops, self.n, self.prefix = [], 0, 0, prefix
+    def __init__(self, prefix, decl="const float"):
+        self.lines, self.nops, self.n, self.prefix, self.decl = [], 0, 0, prefix, decl
 
     def emit(self, expr):
         self.n += 1
         name = f"{self.prefix}{self.n}"
-        self.lines.append(f"    const float {name} = {expr};")
+        self.lines.append(f"    {self.decl} {name} = {expr};")
         self.nops += 1
         return name
 
 
-def emit_ops(em, ops, var, sign):
-    for op in ops:
+N_HOOKS = 48  # call-outs spread evenly through dct64_inv_hooked
+
+
+def emit_ops(em, ops, var, sign, hooks=0):
+    hook_at = {(h * len(ops)) // hooks: h for h in range(hooks)} if hooks else {}
+    for n_op, op in enumerate(ops):
+        if n_op in hook_at:
+            # Arithmetic has no ordering of its own against the memory operations of the hook, and
+            # the compiler would slide all of it to one side.  Passing the 64 live values through an
+            # empty asm statement (no instruction) before the hook keeps them where they are written.
+            live = sorted(set(var.values()))
+            for i in range(0, len(live), 16):
+                em.lines.append("    asm volatile(\"\" : " + ", ".join(f'"+v"({x})' for x in live[i:i + 16]) + ");")
+            em.lines.append(f"    hook(DctHook<{hook_at[n_op]}>{{}});")
         if op[0] == "mul":
             _, i, a = op
             a *= sign[i]
@@ -214,13 +227,17 @@ def finish(em, var, sign, out_slots, dst="v"):
     return "\n".join(em.lines + tail), negs
 
 
-def emit_function(name, ops, in_slots, out_slots):
-    em = Emitter("t")
+def emit_function(name, ops, in_slots, out_slots, hooks=0):
+    em = Emitter("t", "float" if hooks else "const float")
     var = {s: f"v[{n}]" for n, s in enumerate(in_slots)}
     sign = {s: 1.0 for s in in_slots}
-    emit_ops(em, ops, var, sign)
+    emit_ops(em, ops, var, sign, hooks)
     body, negs = finish(em, var, sign, out_slots)
-    return f"__device__ __forceinline__ void {name}(float (&v)[64]) {{\n{body}\n}}\n", em.nops, negs
+    if hooks:
+        head = (f"template <typename Hook>\n__device__ __forceinline__ void {name}(float (&v)[64], Hook&& hook) {{")
+    else:
+        head = f"__device__ __forceinline__ void {name}(float (&v)[64]) {{"
+    return f"{head}\n{body}\n}}\n", em.nops, negs
 
 
 def emit_split_forward(ops, out_slots, n_head):
@@ -275,6 +292,7 @@ def main():
 
     head, tail, n_h, n_t, neg_f = emit_split_forward(fwd, out_slots, n_head)
     t_inv, n_inv, neg_i = emit_function("dct64_inv", inv, out_slots, ident)
+    t_inv_hooked, _, _ = emit_function("dct64_inv_hooked", inv, out_slots, ident, hooks=N_HOOKS)
     print(f"dct64_fwd: {n_h} + {n_t} ops (+{neg_f} negations), dct64_inv: {n_inv} ops (+{neg_i} negations)")
     print(f"fp64 matrix error fwd {err_f:.2e} inv {err_i:.2e}; fp32 forward err / max|y| = {rel:.2e}, "
           f"round trip err / max|x| = {rel_rt:.2e}")
@@ -297,6 +315,12 @@ def main():
                  "    float t[64];\n    dct64_fwd_head(v, t);\n    dct64_fwd_tail(t);\n"
                  "#pragma unroll\n    for (int i = 0; i < 64; ++i) v[i] = t[i];\n}\n\n")
         fh.write(t_inv)
+        fh.write("\n// The same instructions with call-outs: hook(DctHook<h>{}) for h = 0 .. kDctHooks - 1, evenly spread,\n"
+                 "// the first before any arithmetic.  A caller threads latency-bound work (LDS round trips, loads)\n"
+                 "// through the transform that way; the results are bitwise those of dct64_inv.\n"
+                 "template <int I>\nstruct DctHook {\n    static constexpr int value = I;\n};\n"
+                 f"constexpr int kDctHooks = {N_HOOKS};\n\n")
+        fh.write(t_inv_hooked)
 
 
 if __name__ == "__main__":

@@ -165,6 +165,51 @@ __device__ __forceinline__ void chunk_inverse(float (&v)[64], float* tile, int l
 // Pointers that come out of descriptor tables are not kernel arguments, so the compiler
 // cannot tell that they are global memory; say so, or it emits FLAT accesses (which also
 // count as LDS traffic and serialise against the tile).
+// The same 64 rows as 16 stores of 16 bytes per lane.  A wave can have 63 vector-memory
+// instructions in flight, and stores complete slowly when the memory system is saturated with
+// them, so a chunk that leaves as 64 store instructions blocks the issue of the next loads.
+// Lane c holds column c (v[r] = x[r][c]); a 4x4 transpose inside every quad of lanes (two
+// exchange stages, each one v_cndmask with a quad-permuted operand per register) gives lane
+// 4q + i the four values x[4b + i][4q .. 4q + 3] of every row block b.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_chunk_rows_x4(const float (&v)[64], void* chunk0, int64_t ld, int lane) {
+    const __amdgpu_buffer_rsrc_t rs = chunk_rsrc(chunk0, ld);
+    const int ld4 = static_cast<int>(ld) * 4;
+    const bool odd = lane & 1, hi = lane & 2;
+    const int voff = (lane & 3) * ld4 + (lane >> 2) * 16;
+    auto x1 = [](float f) {  // value of the lane whose id differs in bit 0
+        return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, f), 0xB1, 0xf, 0xf, true));
+    };
+    auto x2 = [](float f) {  // ... in bit 1
+        return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, f), 0x4E, 0xf, 0xf, true));
+    };
+    v4u w[16];
+#pragma unroll
+    for (int b = 0; b < 16; ++b) {
+        const float a0 = v[4 * b], a1 = v[4 * b + 1], a2 = v[4 * b + 2], a3 = v[4 * b + 3];
+        // (the cross-lane moves are evaluated by all lanes, outside the selects: inside a
+        // conditional operand only the selecting lanes would run them and read idle neighbours)
+        const float n0 = x1(a0), n1 = x1(a1), n2 = x1(a2), n3 = x1(a3);
+        const float u0 = odd ? n1 : a0, u1 = odd ? a1 : n0;
+        const float u2 = odd ? n3 : a2, u3 = odd ? a3 : n2;
+        const float m0 = x2(u0), m1 = x2(u1), m2 = x2(u2), m3 = x2(u3);
+        w[b].x = __builtin_bit_cast(unsigned, hi ? m2 : u0);
+        w[b].y = __builtin_bit_cast(unsigned, hi ? m3 : u1);
+        w[b].z = __builtin_bit_cast(unsigned, hi ? u2 : m0);
+        w[b].w = __builtin_bit_cast(unsigned, hi ? u3 : m1);
+    }
+    // All 16 stores go out back to back, with no vector ALU instruction between or right after
+    // them.  With the transposes in between, a store's first data register was rewritten for the
+    // next block by the instruction after it, and now and then the store picked up the new
+    // value in a few lanes: a 16-byte store reads its data registers a little after it issues
+    // (no wait states are inserted for the form with a scalar offset).
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int b = 0; b < 16; ++b) __builtin_amdgcn_raw_buffer_store_b128(w[b], rs, voff, 4 * b * ld4, 2);
+    asm volatile("s_nop 3");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 using gfloat = __attribute__((address_space(1))) float;
 using gbyte = __attribute__((address_space(1))) uint8_t;
 
@@ -503,19 +548,25 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     uint32_t ix[kRegs];
     float a[kRegs];
 
-    auto load_payload = [&](int64_t g, int t) {  // fast path only
-        if (scale && t != t_scale) {  // wave-uniform, once per tensor
+    // clip factors of tensor t into my_scale (wave-uniform branch, taken once per tensor)
+    auto load_scale = [&](int t) {
+        if (scale && t != t_scale) {
             my_scale = scale[static_cast<int64_t>(t) * P + pl] * out_scale;
             t_scale = t;
         }
+    };
+    // unit i's entries of chunk g into its two registers
+    auto load_unit = [&](int i, int64_t g) {
+        const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
+        const gbyte* irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
+        const gfloat* vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
+        ix[i] = *(const gu16*)(irow + lane_ioff);
+        a[i] = vrow[le];
+    };
+    auto load_payload = [&](int64_t g, int t) {  // fast path only
+        load_scale(t);
 #pragma unroll
-        for (int i = 0; i < kRegs; ++i) {
-            const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
-            const gbyte* irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
-            const gfloat* vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
-            ix[i] = *(const gu16*)(irow + lane_ioff);
-            a[i] = vrow[le];
-        }
+        for (int i = 0; i < kRegs; ++i) load_unit(i, g);
     };
     // entry j of peer p of chunk g (generic path and normalise)
     auto load_entry = [&](int p, int j, int64_t g, uint32_t& ixo, float& ao) {
@@ -525,7 +576,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         ao = ((const gfloat*)pp.val[p] + g * k)[j];
     };
 
-    const bool fast = kFast && !normalise;
+    const bool fast = kFast;  // (normalise is served by the generic instantiation only)
 
     auto zero_tile = [&]() {
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -637,6 +688,169 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                    cu.ld};
     };
 
+    // =====================================================================================
+    // Fast path with the transform: four chunks in flight per wave.
+    //   chunk g      second transform pass in registers, then 64 row stores
+    //   chunk g + 1  scattered into the tile, threaded through that pass
+    //   chunk g + 2  payload in the other register set, on its way or arrived
+    //   chunk g + 3  payload requested into the registers the scatter has just released
+    // The scatter is a chain of LDS round trips (read, add, write, one peer after the other: a
+    // later peer may hit the same coefficient), far too slow to sit in the open.  Step s of it,
+    // at one of the pass's call-outs, completes unit s - 1 (write back, reload its registers) and
+    // starts unit s (read).  Everything in there is branch-free: lanes and units without an entry
+    // work on a per-lane slot in the tile's padding, and past the end of the wave's range the
+    // same (valid) data is scattered into a tile that nobody reads.
+    // Payload loads queue behind every store of the compute unit's eight waves, which takes
+    // about as long as one chunk; two chunks of distance keep the wave from waiting for them.
+    // =====================================================================================
+    if constexpr (kFast && kUseDct) {
+        struct Set {
+            uint32_t ix[kRegs];
+            float a[kRegs];
+            float sc;  // lane p: clip factor of peer p for tensor t, times 2^-5
+            int t;
+        };
+        Set s0, s1;
+#pragma unroll
+        for (int i = 0; i < kRegs; ++i) s0.ix[i] = s1.ix[i] = 0, s0.a[i] = s1.a[i] = 0.f;
+        s0.sc = s1.sc = out_scale;
+        s0.t = s1.t = -1;
+        auto set_scale = [&](Set& st, int t) {  // wave-uniform branch, taken once per tensor
+            if (scale && t != st.t) {
+                st.sc = scale[static_cast<int64_t>(t) * P + pl] * out_scale;
+                st.t = t;
+            }
+        };
+        auto set_load_unit = [&](Set& st, int i, int64_t g) {
+            const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
+            const gbyte* irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
+            const gfloat* vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
+            st.ix[i] = *(const gu16*)(irow + lane_ioff);
+            st.a[i] = vrow[le];
+        };
+        auto set_load = [&](Set& st, int64_t g, int t) {
+            set_scale(st, t);
+#pragma unroll
+            for (int i = 0; i < kRegs; ++i) set_load_unit(st, i, g);
+        };
+        auto unit_scale = [&](float sc, int u) {
+            return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sc), u));
+        };
+
+        Cursor c;
+        cursor_seek(c, table, single, n_tensors, g0);
+        Out o0 = out_of(c, g0), o1 = o0, o2 = o0;  // destinations of chunks g, g + 1, g + 2
+        // the first chunk: plain serial scatter
+        set_load(s0, g0, c.t);
+        zero_tile();
+        if (lane_on) {
+#pragma unroll
+            for (int i = 0; i < kRegs; ++i) {
+                if (i < P) {  // wave-uniform
+                    const uint32_t e = (lane & 1) ? (s0.ix[i] >> 4) : (s0.ix[i] & 0xfffu);
+                    float* t = &tile[tile_pos(e)];
+                    *t = *t + s0.a[i] * unit_scale(s0.sc, i);
+                    atomicAdd(&cnt[Cnt::word(e)], 1u << Cnt::shift(e));
+                }
+            }
+        }
+        mean_pass();
+        if (g0 + 1 < g1) {
+            cursor_next(c, g0 + 1);
+            o1 = out_of(c, g0 + 1);
+            set_load(s1, g0 + 1, c.t);
+        }
+        if (g0 + 2 < g1) {
+            cursor_next(c, g0 + 2);
+            o2 = out_of(c, g0 + 2);
+            set_load(s0, g0 + 2, c.t);
+        }
+        {
+            // The memory counter completes in order, and the compiler sizes every wait for the
+            // worse of the ways into the loop.  From the back edge, payload loads are followed by
+            // the 16 stores of a chunk, so a wait for a load needs none of the stores behind it;
+            // coming from here there would be no stores, every wait would shrink to "all but the
+            // loads behind me", and on the back edge that means "all stores drained".  Give this
+            // entry the same shape with 16 stores that write nothing: their descriptor has a
+            // range of zero bytes, so the bounds check of the buffer instruction drops them.
+            // (Real stores to the first chunk's rows would not do: two stores of one wave to one
+            // address were seen to land in either order.)
+            const __amdgpu_buffer_rsrc_t nowhere =
+                __builtin_amdgcn_make_buffer_rsrc((void*)o0.chunk0, 0, 0, 0x00020000);
+            const v4u z = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int b = 0; b < 16; ++b) __builtin_amdgcn_raw_buffer_store_b128(z, nowhere, lane * 16, b * 1024, 2);
+        }
+
+        const int dummy_pos = lane * kLd + kChunk;
+        // one chunk: `st` holds chunk g + 1 and is refilled with chunk g + 3
+        auto step = [&](int64_t g, Set& st) {
+            float v[64];
+            tile_rows_to_regs(v, tile, lane);
+            dct64_inv(v);  // along d: v[l] = sum_d Y[lane][d] F[l][d]
+            wave_lds_fence();
+            regs_to_tile_rows(v, tile, lane);
+            wave_lds_fence();
+            tile_cols_to_regs(v, tile, lane);
+            wave_lds_fence();
+
+            zero_tile();
+            const float sc_now = st.sc;
+            const bool more3 = g + 3 < g1;
+            Out o3 = o2;
+            if (more3) {
+                cursor_next(c, g + 3);
+                o3 = out_of(c, g + 3);
+                set_scale(st, c.t);
+            }
+            const int64_t g_load = more3 ? g + 3 : g1 - 1;
+            constexpr int kSteps = kUnits + 1;
+            constexpr int kAlways = kUnits > 8 ? kUnits - 8 : 1;  // units every served peer count uses
+            int pos = dummy_pos;
+            float cur = 0.f, add = 0.f;
+            // along b: v[k] = sum_b Z[b][lane] F[k][b]
+            dct64_inv_hooked(v, [&](auto tag) {
+                constexpr int h = decltype(tag)::value;
+                // step s runs at call-out (s * kDctHooks) / kSteps
+                constexpr int s = (h * kSteps + kDctHooks - 1) / kDctHooks;
+                if constexpr (s < kSteps && (s * kDctHooks) / kSteps == h) {
+                    if constexpr (s > 0) {
+                        tile[pos] = cur + add;
+                        set_load_unit(st, s - 1, g_load);
+                    }
+                    if constexpr (s < kUnits) {
+                        constexpr int u = s;
+                        const bool on = lane_on && (u < kAlways || u < P);
+                        const uint32_t e = (lane & 1) ? (st.ix[u] >> 4) : (st.ix[u] & 0xfffu);
+                        pos = on ? tile_pos(e) : dummy_pos;
+                        add = st.a[u] * unit_scale(sc_now, u);
+                        cur = tile[pos];
+                        atomicAdd(&cnt[on ? Cnt::word(e) : lane], on ? 1u << Cnt::shift(e) : 0u);
+                    }
+                }
+            });
+            float ss = 0.f;
+            if (sumsq) {
+#pragma unroll
+                for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
+                ss = wave_sum_f32(ss);
+            }
+            mean_pass();
+            // (the loop-carried destination may have been parked in vector registers: make it
+            // scalar again, or every store becomes a loop over distinct descriptors)
+            store_chunk_rows_x4(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane);
+            if (sumsq && lane == 0) sumsq[g] = ss;
+            o0 = o1;
+            o1 = o2;
+            o2 = o3;
+        };
+        for (int64_t g = g0; g < g1; g += 2) {
+            step(g, s1);
+            if (g + 1 < g1) step(g + 1, s0);
+        }
+        return;
+    }
+
     // The loop is software-pipelined over three chunks.  While chunk g is in registers for the
     // second pass of its inverse transform (vector ALU only), the tile already receives the
     // scatter of chunk g + 1, and the payload of chunk g + 2 is on its way from memory.
@@ -654,7 +868,6 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         t_next = c.t;
         if (fast) load_payload(g0 + 1, c.t);
     }
-
     for (int64_t g = g0; g < g1; ++g) {
         float v[64];
         // ---- first half: everything that needs chunk g's coefficients in the tile
@@ -689,7 +902,6 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 if (fast) load_payload(g + 2, c.t);
             }
         }
-
         // ---- second half of chunk g, in registers
         if (kUseDct) dct64_inv(v);  // along b: v[k] = sum_b Z[b][lane] F[k][b]
         float ss = 0.f;
