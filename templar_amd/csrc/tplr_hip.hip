@@ -1012,34 +1012,47 @@ __global__ __launch_bounds__(1024) void k_peer_sumsq(const ValPtrs vp, int64_t n
 }
 
 // one block per (tensor, peer): sum of squares of that tensor's slice of the peer's values.
-// The slice starts at an even element (k is even), so it is read as float2 with eight
-// independent accumulators per thread; the reduction order is fixed.
-__global__ __launch_bounds__(256) void k_segment_sumsq(const ValPtrs vp, int P, int k,
-                                                       const tplr_tensor_desc* __restrict__ table,
-                                                       float* __restrict__ sumsq) {
-    __shared__ float part[4];
+// The slice starts at an even element (k is even), so it is read as float2.  The largest slice
+// sets the duration of the launch, so a block keeps a lot in flight: 1024 threads with sixteen
+// independent loads and accumulators each (128 KB per trip).  The reduction order is fixed.
+__global__ __launch_bounds__(1024) void k_segment_sumsq(const ValPtrs vp, int P, int k,
+                                                        const tplr_tensor_desc* __restrict__ table,
+                                                        float* __restrict__ sumsq) {
+    constexpr int kT = 1024, kU = 16;
+    __shared__ float part[kT / 64];
     const int t = blockIdx.x / P, p = blockIdx.x - t * P;
     const tplr_tensor_desc d = table[t];
     const int64_t n2 = static_cast<int64_t>(d.x_chunks) * d.y_chunks * k / 2;
-    const float2* v = reinterpret_cast<const float2*>(vp.val[p] + d.chunk_begin * k);
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    typedef float v2f __attribute__((ext_vector_type(2)));
+    const v2f* v = reinterpret_cast<const v2f*>(vp.val[p] + d.chunk_begin * k);
+    float acc[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) acc[u] = 0.f;
     int64_t i = threadIdx.x;
-    for (; i + 7 * 256 < n2; i += 8 * 256) {
-        float2 x[8];
+    for (; i + (kU - 1) * kT < n2; i += kU * kT) {
+        v2f x[kU];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) x[u] = v[i + u * 256];
+        for (int u = 0; u < kU; ++u) x[u] = __builtin_nontemporal_load(v + i + u * kT);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) acc[u] = __builtin_fmaf(x[u].y, x[u].y, __builtin_fmaf(x[u].x, x[u].x, acc[u]));
+        for (int u = 0; u < kU; ++u) acc[u] = __builtin_fmaf(x[u].y, x[u].y, __builtin_fmaf(x[u].x, x[u].x, acc[u]));
     }
-    for (; i < n2; i += 256) {
-        const float2 x = v[i];
+    for (; i < n2; i += kT) {
+        const v2f x = v[i];
         acc[0] = __builtin_fmaf(x.y, x.y, __builtin_fmaf(x.x, x.x, acc[0]));
     }
-    float s = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
-    s = wave_sum_f32(s);
+#pragma unroll
+    for (int w = kU / 2; w > 0; w >>= 1)
+#pragma unroll
+        for (int u = 0; u < w; ++u) acc[u] += acc[u + w];
+    const float s = wave_sum_f32(acc[0]);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
     __syncthreads();
-    if (threadIdx.x == 0) sumsq[blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
+    if (threadIdx.x == 0) {
+        float tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < kT / 64; ++w) tot += part[w];
+        sumsq[blockIdx.x] = tot;
+    }
 }
 
 // one block per tensor: scale[t][p] = min(1, med_t / (norm[t][p] + 1e-8))
@@ -1426,7 +1439,7 @@ int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr
         vp.val[p] = p < n_peers ? h_val[p] : nullptr;
         if (p < n_peers && !vp.val[p]) return TPLR_E_BADARG;
     }
-    hipLaunchKernelGGL(k_segment_sumsq, dim3(static_cast<unsigned>(n_tensors) * n_peers), dim3(256), 0,
+    hipLaunchKernelGGL(k_segment_sumsq, dim3(static_cast<unsigned>(n_tensors) * n_peers), dim3(1024), 0,
                        static_cast<hipStream_t>(stream), vp, n_peers, k, d_desc, d_sumsq);
     return launch_status();
 }
