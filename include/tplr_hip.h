@@ -172,17 +172,22 @@ int tplr_scatter_rows(const uint8_t* d_idx12, const int64_t* d_idx64, const floa
 int tplr_peer_sumsq(const float* const* h_val, int n_peers, int64_t n, float* d_sumsq, void* stream);
 
 /* d_scale[p] = min(1, med / (norm_p + 1e-8)), med = lower median of the norms
- * (torch.median), norm_p = d_norm[p] (is_sumsq == 0) or sqrt(d_norm[p]) (is_sumsq != 0).
- * d_median (nullable) receives med. */
-int tplr_clip_scales(const float* d_norm, int n_peers, int is_sumsq, float* d_scale, float* d_median,
+ * (torch.median).  n_partials == 0: d_norm[p] is the norm itself; n_partials >= 1: d_norm holds
+ * n_partials partial sums of squares per peer (peer-major), norm_p = sqrt of their sum taken in
+ * order.  d_median (nullable) receives med. */
+int tplr_clip_scales(const float* d_norm, int n_peers, int n_partials, float* d_scale, float* d_median,
                      void* stream);
 
-/* Batch forms for flat payloads: d_sumsq[t * n_peers + p] = sum of squares of peer p's values
- * that belong to tensor t (the per-peer, per-parameter norms of src/tplr/neurons.py:346);
- * d_scale[t * n_peers + p] from the lower median over the peers of tensor t. */
+/* Batch forms for flat payloads (the per-peer, per-parameter norms of src/tplr/neurons.py:346
+ * and the clip of src/tplr/compress.py:526-556 for every parameter at once).
+ * tplr_segment_sumsq: d_sumsq[(t * n_peers + p) * n_slices + s] = sum of squares of slice s of
+ * peer p's values that belong to tensor t; a tensor's chunks are cut into n_slices runs so that
+ * a few very large tensors still fill the device (n_slices = 1: one sum per tensor and peer).
+ * tplr_clip_scales_batch: d_scale[t * n_peers + p] from the lower median over the peers of
+ * tensor t, d_norm laid out as above with n_partials = n_slices (or 0 for plain norms). */
 int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr_tensor_desc* d_desc,
-                       int n_tensors, float* d_sumsq, void* stream);
-int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int is_sumsq, float* d_scale,
+                       int n_tensors, int n_slices, float* d_sumsq, void* stream);
+int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int n_partials, float* d_scale,
                            float* d_median, void* stream);
 
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes

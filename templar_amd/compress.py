@@ -819,13 +819,15 @@ def peer_clip_scales_batch(batch: TensorBatch, vals: Sequence[torch.Tensor], k: 
     if P > _lib.TPLR_MAX_PEERS:
         raise NotImplementedError(f"{P} peers: the HIP aggregate kernel takes up to {_lib.TPLR_MAX_PEERS}")
     dev = batch.device
-    ss = torch.empty((len(batch), P), dtype=torch.float32, device=dev)
-    scale = torch.empty_like(ss)
+    # enough blocks to fill the device even when the set is a few very large tensors
+    slices = max(1, min(64, 4096 // (len(batch) * P)))
+    ss = torch.empty((len(batch), P, slices), dtype=torch.float32, device=dev)
+    scale = torch.empty((len(batch), P), dtype=torch.float32, device=dev)
     vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
     with torch.cuda.device(dev):
-        _lib.check(lib.tplr_segment_sumsq(vp, P, k, _ptr(batch.table), len(batch), _ptr(ss), _stream(dev)),
+        _lib.check(lib.tplr_segment_sumsq(vp, P, k, _ptr(batch.table), len(batch), slices, _ptr(ss), _stream(dev)),
                    "tplr_segment_sumsq")
-        _lib.check(lib.tplr_clip_scales_batch(_ptr(ss), len(batch), P, 1, _ptr(scale), None, _stream(dev)),
+        _lib.check(lib.tplr_clip_scales_batch(_ptr(ss), len(batch), P, slices, _ptr(scale), None, _stream(dev)),
                    "tplr_clip_scales_batch")
     return scale
 

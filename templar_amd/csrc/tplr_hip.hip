@@ -1011,20 +1011,25 @@ __global__ __launch_bounds__(1024) void k_peer_sumsq(const ValPtrs vp, int64_t n
     }
 }
 
-// one block per (tensor, peer): sum of squares of that tensor's slice of the peer's values.
-// The slice starts at an even element (k is even), so it is read as float2.  The largest slice
-// sets the duration of the launch, so a block keeps a lot in flight: 1024 threads with sixteen
-// independent loads and accumulators each (128 KB per trip).  The reduction order is fixed.
-__global__ __launch_bounds__(1024) void k_segment_sumsq(const ValPtrs vp, int P, int k,
+// Sum of squares of a tensor's part of a peer's values, in S slices: one block per (tensor,
+// peer, slice), partial sums at sumsq[(t * P + p) * S + slice] (the consumer adds them in
+// order).  A part starts at an even element (k is even), so it is read as float2.  The largest
+// slice sets the duration of the launch, so a block keeps a lot in flight: 1024 threads with
+// sixteen independent loads and accumulators each (128 KB per trip).  The reduction order is fixed.
+__global__ __launch_bounds__(1024) void k_segment_sumsq(const ValPtrs vp, int P, int k, int S,
                                                         const tplr_tensor_desc* __restrict__ table,
                                                         float* __restrict__ sumsq) {
     constexpr int kT = 1024, kU = 16;
     __shared__ float part[kT / 64];
-    const int t = blockIdx.x / P, p = blockIdx.x - t * P;
+    // block = (tensor t, peer p, slice sl); a slice is a run of whole chunks
+    const int tp = blockIdx.x / S, sl = blockIdx.x - tp * S;
+    const int t = tp / P, p = tp - t * P;
     const tplr_tensor_desc d = table[t];
-    const int64_t n2 = static_cast<int64_t>(d.x_chunks) * d.y_chunks * k / 2;
+    const int64_t n_chunks = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
+    const int64_t c0 = n_chunks * sl / S, c1 = n_chunks * (sl + 1) / S;
+    const int64_t n2 = (c1 - c0) * k / 2;
     typedef float v2f __attribute__((ext_vector_type(2)));
-    const v2f* v = reinterpret_cast<const v2f*>(vp.val[p] + d.chunk_begin * k);
+    const v2f* v = reinterpret_cast<const v2f*>(vp.val[p] + (d.chunk_begin + c0) * k);
     float acc[kU];
 #pragma unroll
     for (int u = 0; u < kU; ++u) acc[u] = 0.f;
@@ -1056,13 +1061,22 @@ __global__ __launch_bounds__(1024) void k_segment_sumsq(const ValPtrs vp, int P,
 }
 
 // one block per tensor: scale[t][p] = min(1, med_t / (norm[t][p] + 1e-8))
-__global__ __launch_bounds__(128) void k_clip_scales(const float* __restrict__ norm, int P, int is_sumsq,
+__global__ __launch_bounds__(128) void k_clip_scales(const float* __restrict__ norm, int P, int n_partials,
                                                      float* __restrict__ scale, float* __restrict__ median) {
     __shared__ float nv[TPLR_MAX_PEERS];
     __shared__ float med;
     const int i = threadIdx.x;
     const int64_t off = static_cast<int64_t>(blockIdx.x) * P;
-    if (i < P) nv[i] = is_sumsq ? __builtin_sqrtf(norm[off + i]) : norm[off + i];
+    if (i < P) {
+        if (n_partials > 0) {  // partial sums of squares, added in order
+            const float* ps = norm + (off + i) * n_partials;
+            float tot = 0.f;
+            for (int s = 0; s < n_partials; ++s) tot += ps[s];
+            nv[i] = __builtin_sqrtf(tot);
+        } else {
+            nv[i] = norm[off + i];
+        }
+    }
     if (i == 0) med = 0.f;
     __syncthreads();
     if (i < P) {
@@ -1416,31 +1430,33 @@ int tplr_peer_sumsq(const float* const* h_val, int n_peers, int64_t n, float* d_
     return launch_status();
 }
 
-int tplr_clip_scales(const float* d_norm, int n_peers, int is_sumsq, float* d_scale, float* d_median,
+int tplr_clip_scales(const float* d_norm, int n_peers, int n_partials, float* d_scale, float* d_median,
                      void* stream) {
-    return tplr_clip_scales_batch(d_norm, 1, n_peers, is_sumsq, d_scale, d_median, stream);
+    return tplr_clip_scales_batch(d_norm, 1, n_peers, n_partials, d_scale, d_median, stream);
 }
 
-int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int is_sumsq, float* d_scale,
+int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int n_partials, float* d_scale,
                            float* d_median, void* stream) {
-    if (!d_norm || !d_scale || n_peers < 1 || n_tensors < 1) return TPLR_E_BADARG;
+    if (!d_norm || !d_scale || n_peers < 1 || n_tensors < 1 || n_partials < 0) return TPLR_E_BADARG;
     if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
     hipLaunchKernelGGL(k_clip_scales, dim3(n_tensors), dim3(128), 0, static_cast<hipStream_t>(stream), d_norm, n_peers,
-                       is_sumsq, d_scale, d_median);
+                       n_partials, d_scale, d_median);
     return launch_status();
 }
 
 int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
-                       float* d_sumsq, void* stream) {
-    if (!h_val || !d_desc || !d_sumsq || n_peers < 1 || n_tensors < 1 || k < 1) return TPLR_E_BADARG;
+                       int n_slices, float* d_sumsq, void* stream) {
+    if (!h_val || !d_desc || !d_sumsq || n_peers < 1 || n_tensors < 1 || k < 2 || (k & 1) || n_slices < 1)
+        return TPLR_E_BADARG;
+    if (static_cast<int64_t>(n_tensors) * n_peers * n_slices > 0x7fffffff) return TPLR_E_TOOMANY;
     if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
     ValPtrs vp;
     for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
         vp.val[p] = p < n_peers ? h_val[p] : nullptr;
         if (p < n_peers && !vp.val[p]) return TPLR_E_BADARG;
     }
-    hipLaunchKernelGGL(k_segment_sumsq, dim3(static_cast<unsigned>(n_tensors) * n_peers), dim3(1024), 0,
-                       static_cast<hipStream_t>(stream), vp, n_peers, k, d_desc, d_sumsq);
+    hipLaunchKernelGGL(k_segment_sumsq, dim3(static_cast<unsigned>(n_tensors) * n_peers * n_slices), dim3(1024), 0,
+                       static_cast<hipStream_t>(stream), vp, n_peers, k, n_slices, d_desc, d_sumsq);
     return launch_status();
 }
 
