@@ -1,0 +1,155 @@
+"""Full-size checks on the GPU: the 1B gradient set (294 144 chunks, BASELINE.json configs 3 and 4)
+and the 72B block (config 5, k = 64) through the batch entry points of the C ABI.
+
+The CPU oracle cannot cover these sizes in test time, so the checks are properties that do not
+depend on size (plus a strided sample that does go through the oracle):
+
+  * selection: every row has k distinct indices < 4096, magnitudes in descending order, lowest
+    index first on ties; fused encode == transform followed by select, bitwise, on the largest
+    tensor; a strided sample of chunks equals the oracle's selection on the device's coefficients;
+  * Parseval: the energy of the reconstruction of one payload equals the energy of its values
+    (the transform is orthonormal), per chunk and in total;
+  * mean of identical peers: P copies of one payload aggregate to the one-peer result (exactly
+    for two peers, within a few ulp for more: sums of equal terms round);
+  * linearity: the sum-mode aggregate of two different peers equals the sum of their one-peer
+    decodes within fp32 tolerance;
+  * round trip: encode(decode(payload)) selects the same index sets.
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+from oracle import codec as orc  # noqa: E402  (the checker)
+import templar_amd.compress as tc  # noqa: E402
+import workloads  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no HIP device")
+    return torch.device("cuda:0")
+
+
+def _set(name, dev):
+    grads = [g for g in workloads.gradient_set(name, device=dev) if g.dim() == 2]
+    return grads, workloads.CONFIGS[name]["k"]
+
+
+def _check_rows(idx12, val, n, k):
+    """Structure of a flat payload: distinct in-range indices, canonical order."""
+    idx = tc.unpack_12bit_indices(idx12, (n, k))
+    assert int(idx.max()) < 4096 and int(idx.min()) >= 0
+    srt = idx.sort(dim=1).values
+    assert bool((srt[:, 1:] != srt[:, :-1]).all()), "duplicate index inside a row"
+    mag = val.abs()
+    assert bool((mag[:, :-1] >= mag[:, 1:]).all()), "magnitudes not descending"
+    tie = mag[:, :-1] == mag[:, 1:]
+    assert bool((idx[:, :-1][tie] < idx[:, 1:][tie]).all()), "ties not in index order"
+    return idx
+
+
+@pytest.mark.parametrize("name", ["cfg3_llama1b", "cfg5_72b_block"])
+def test_full_set_encode_properties(dev, name):
+    grads, k = _set(name, dev)
+    batch = tc.TensorBatch(grads)
+    n = batch.total_chunks
+    idx12, val = tc.encode_compress_batch(batch, k, use_dct=True)
+    assert idx12.numel() == n * k * 3 // 2 and val.shape == (n, k)
+    idx = _check_rows(idx12, val, n, k)
+
+    # fused == transform then select, bitwise, on the largest tensor of the set
+    big = max(range(len(grads)), key=lambda i: grads[i].numel())
+    x = grads[big]
+
+    class M:
+        def named_parameters(self):
+            from types import SimpleNamespace
+            yield "w", SimpleNamespace(requires_grad=True, shape=tuple(x.shape), dtype=torch.float32, device=dev)
+
+    tr = tc.ChunkingTransformer(M(), 64)
+    coef = tr.encode(x, use_dct=True).reshape(-1, 4096)
+    i_u, v_u = tc._topk_rows(coef, k)
+    i_f, v_f = batch.payload_slice(big, idx12, val, k)
+    assert torch.equal(i_f, i_u) and torch.equal(v_f.reshape(-1, k), v_u)
+
+    # a strided sample of that tensor's chunks against the oracle's selection
+    step = max(1, coef.shape[0] // 64)
+    rows = coef[::step].cpu().numpy()
+    want_i, want_v = orc.topk_rows(rows, k)
+    b0 = batch.offsets[big]
+    assert np.array_equal(idx[b0:b0 + coef.shape[0]][::step].cpu().numpy(), want_i)
+    assert np.array_equal(v_u[::step].cpu().numpy(), want_v)
+    # the selection is a top-k: nothing left out is larger than the smallest value kept
+    kept = torch.zeros_like(coef, dtype=torch.bool).scatter_(1, idx[b0:b0 + coef.shape[0]], True)
+    left = coef.abs().masked_fill(kept, 0.0).max(dim=1).values
+    assert bool((left <= v_u.abs().min(dim=1).values).all())
+    # transform tolerance on the sample, against the oracle's closed-form transform
+    y, xx = x.shape[0] // 64, x.shape[1] // 64
+    for g in range(0, coef.shape[0], step * 8):
+        cy, cx = divmod(g, xx)
+        blk = x[cy * 64:(cy + 1) * 64, cx * 64:(cx + 1) * 64].cpu().numpy()
+        want = orc.encode2d(blk).reshape(-1)
+        assert np.abs(coef[g].cpu().numpy() - want).max() <= TOL * np.abs(want).max()
+
+
+def test_full_set_aggregate_properties(dev):
+    grads, k = _set("cfg3_llama1b", dev)
+    batch = tc.TensorBatch(grads)
+    n = batch.total_chunks
+    idx_a, val_a = tc.encode_compress_batch(batch, k, use_dct=True)
+    # a second, different payload on the same shapes
+    others = [workloads.student_t3(tuple(g.shape), 7000 + j, row_scale=True, device=dev) for j, g in enumerate(grads)]
+    idx_b, val_b = tc.encode_compress_batch(tc.TensorBatch(others), k, use_dct=True)
+    del others
+    outs = [torch.empty_like(g) for g in grads]
+    ob = tc.TensorBatch(outs)
+
+    # one peer, no clip: Parseval per chunk and in total
+    ss = torch.empty(n, device=dev)
+    tc.batch_decompress_decode_batch(ob, [idx_a], [val_a], k, clip_norm=False, sumsq=ss)
+    one = [o.clone() for o in outs]
+    e_val = (val_a.double() ** 2).sum(dim=1)
+    assert torch.allclose(ss.double(), e_val, rtol=1e-4, atol=1e-30)
+    e_out = sum(float((o.double() ** 2).sum()) for o in one)
+    assert abs(e_out - float(e_val.sum())) <= 1e-5 * float(e_val.sum())
+
+    # P identical peers: the mean is the one-peer result (x + x halves back exactly; longer sums of
+    # equal terms round, so 8 and 15 peers are held to a few ulp)
+    for P in (2, 8, 15):
+        tc.batch_decompress_decode_batch(ob, [idx_a] * P, [val_a] * P, k, clip_norm=False)
+        for o, w in zip(outs, one):
+            if P == 2:
+                assert torch.equal(o, w)
+            else:
+                assert float((o - w).abs().max()) <= 1e-6 * float(w.abs().max()), f"P={P}"
+
+    # clip factors of identical peers are min(1, n / (n + 1e-8)): 1 to within an ulp
+    tc.batch_decompress_decode_batch(ob, [idx_a] * 4, [val_a] * 4, k, clip_norm=True)
+    for o, w in zip(outs, one):
+        assert float((o - w).abs().max()) <= 1e-6 * float(w.abs().max())
+
+    # sum mode is linear: aggregate(a, b) == decode(a) + decode(b)
+    tc.batch_decompress_decode_batch(ob, [idx_b], [val_b], k, clip_norm=False)
+    two = [o.clone() for o in outs]
+    tc.batch_decompress_decode_batch(ob, [idx_a, idx_b], [val_a, val_b], k, clip_norm=False, mean=False)
+    for o, a, b in zip(outs, one, two):
+        ref = a + b
+        assert float((o - ref).abs().max()) <= TOL * float(ref.abs().max())
+
+    # round trip: the reconstruction of a payload encodes to the same index sets
+    idx_r, val_r = tc.encode_compress_batch(tc.TensorBatch(one), k, use_dct=True)
+    ia = tc.unpack_12bit_indices(idx_a, (n, k)).sort(dim=1).values
+    ir = tc.unpack_12bit_indices(idx_r, (n, k)).sort(dim=1).values
+    same = (ia == ir).all(dim=1)
+    # a row may differ only where the k-th and a dropped coefficient (a rounding-level zero) tie
+    assert float(same.float().mean()) > 0.999
+    assert float((val_r.abs().sum(dim=1) - val_a.abs().sum(dim=1)).abs().max()) <= 1e-4 * float(val_a.abs().sum(dim=1).max())
