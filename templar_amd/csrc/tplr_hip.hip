@@ -165,51 +165,6 @@ __device__ __forceinline__ void chunk_inverse(float (&v)[64], float* tile, int l
 // Pointers that come out of descriptor tables are not kernel arguments, so the compiler
 // cannot tell that they are global memory; say so, or it emits FLAT accesses (which also
 // count as LDS traffic and serialise against the tile).
-// The same 64 rows as 16 stores of 16 bytes per lane.  A wave can have 63 vector-memory
-// instructions in flight, and stores complete slowly when the memory system is saturated with
-// them, so a chunk that leaves as 64 store instructions blocks the issue of the next loads.
-// Lane c holds column c (v[r] = x[r][c]); a 4x4 transpose inside every quad of lanes (two
-// exchange stages, each one v_cndmask with a quad-permuted operand per register) gives lane
-// 4q + i the four values x[4b + i][4q .. 4q + 3] of every row block b.
-typedef unsigned v4u __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void store_chunk_rows_x4(const float (&v)[64], void* chunk0, int64_t ld, int lane) {
-    const __amdgpu_buffer_rsrc_t rs = chunk_rsrc(chunk0, ld);
-    const int ld4 = static_cast<int>(ld) * 4;
-    const bool odd = lane & 1, hi = lane & 2;
-    const int voff = (lane & 3) * ld4 + (lane >> 2) * 16;
-    auto x1 = [](float f) {  // value of the lane whose id differs in bit 0
-        return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, f), 0xB1, 0xf, 0xf, true));
-    };
-    auto x2 = [](float f) {  // ... in bit 1
-        return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, f), 0x4E, 0xf, 0xf, true));
-    };
-    v4u w[16];
-#pragma unroll
-    for (int b = 0; b < 16; ++b) {
-        const float a0 = v[4 * b], a1 = v[4 * b + 1], a2 = v[4 * b + 2], a3 = v[4 * b + 3];
-        // (the cross-lane moves are evaluated by all lanes, outside the selects: inside a
-        // conditional operand only the selecting lanes would run them and read idle neighbours)
-        const float n0 = x1(a0), n1 = x1(a1), n2 = x1(a2), n3 = x1(a3);
-        const float u0 = odd ? n1 : a0, u1 = odd ? a1 : n0;
-        const float u2 = odd ? n3 : a2, u3 = odd ? a3 : n2;
-        const float m0 = x2(u0), m1 = x2(u1), m2 = x2(u2), m3 = x2(u3);
-        w[b].x = __builtin_bit_cast(unsigned, hi ? m2 : u0);
-        w[b].y = __builtin_bit_cast(unsigned, hi ? m3 : u1);
-        w[b].z = __builtin_bit_cast(unsigned, hi ? u2 : m0);
-        w[b].w = __builtin_bit_cast(unsigned, hi ? u3 : m1);
-    }
-    // All 16 stores go out back to back, with no vector ALU instruction between or right after
-    // them.  With the transposes in between, a store's first data register was rewritten for the
-    // next block by the instruction after it, and now and then the store picked up the new
-    // value in a few lanes: a 16-byte store reads its data registers a little after it issues
-    // (no wait states are inserted for the form with a scalar offset).
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int b = 0; b < 16; ++b) __builtin_amdgcn_raw_buffer_store_b128(w[b], rs, voff, 4 * b * ld4, 2);
-    asm volatile("s_nop 3");
-    __builtin_amdgcn_sched_barrier(0);
-}
-
 using gfloat = __attribute__((address_space(1))) float;
 using gbyte = __attribute__((address_space(1))) uint8_t;
 
@@ -769,18 +724,17 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         {
             // The memory counter completes in order, and the compiler sizes every wait for the
             // worse of the ways into the loop.  From the back edge, payload loads are followed by
-            // the 16 stores of a chunk, so a wait for a load needs none of the stores behind it;
+            // the 64 row stores of a chunk, so a wait for a load needs few of the stores behind it;
             // coming from here there would be no stores, every wait would shrink to "all but the
             // loads behind me", and on the back edge that means "all stores drained".  Give this
-            // entry the same shape with 16 stores that write nothing: their descriptor has a
+            // entry the same shape with 64 stores that write nothing: their descriptor has a
             // range of zero bytes, so the bounds check of the buffer instruction drops them.
             // (Real stores to the first chunk's rows would not do: two stores of one wave to one
             // address were seen to land in either order.)
             const __amdgpu_buffer_rsrc_t nowhere =
                 __builtin_amdgcn_make_buffer_rsrc((void*)o0.chunk0, 0, 0, 0x00020000);
-            const v4u z = {0u, 0u, 0u, 0u};
 #pragma unroll
-            for (int b = 0; b < 16; ++b) __builtin_amdgcn_raw_buffer_store_b128(z, nowhere, lane * 16, b * 1024, 2);
+            for (int r = 0; r < 64; ++r) __builtin_amdgcn_raw_buffer_store_b32(0, nowhere, lane * 4, r * 256, 2);
         }
 
         const int dummy_pos = lane * kLd + kChunk;
@@ -839,7 +793,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             mean_pass();
             // (the loop-carried destination may have been parked in vector registers: make it
             // scalar again, or every store becomes a loop over distinct descriptors)
-            store_chunk_rows_x4(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane);
+            store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane);
             if (sumsq && lane == 0) sumsq[g] = ss;
             o0 = o1;
             o1 = o2;
