@@ -738,6 +738,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
 
         const int dummy_pos = lane * kLd + kChunk;
+        const uint32_t nib_shift = (lane & 1) * 4;  // odd entries sit in the upper 12 bits of their 16
         // one chunk: `st` holds chunk g + 1 and is refilled with chunk g + 3
         auto step = [&](int64_t g, Set& st) {
             float v[64];
@@ -776,8 +777,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                     if constexpr (s < kUnits) {
                         constexpr int u = s;
                         const bool on = lane_on && (u < kAlways || u < P);
-                        const uint32_t e = (lane & 1) ? (st.ix[u] >> 4) : (st.ix[u] & 0xfffu);
-                        pos = on ? tile_pos(e) : dummy_pos;
+                        const uint32_t e = __builtin_amdgcn_ubfe(st.ix[u], nib_shift, 12);
+                        pos = on ? static_cast<int>(e + ((e >> 6) << 2)) : dummy_pos;
                         add = st.a[u] * unit_scale(sc_now, u);
                         cur = tile[pos];
                         atomicAdd(&cnt[on ? Cnt::word(e) : lane], on ? 1u << Cnt::shift(e) : 0u);
