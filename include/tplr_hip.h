@@ -190,6 +190,27 @@ int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr
 int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int n_partials, float* d_scale,
                            float* d_median, void* stream);
 
+/* ---- miner side: error-feedback step (src/tplr/neurons.py:147-171) ------------------
+ * The reference runs, per parameter: ef.mul_(decay); ef.add_(grad); encode(ef); compress;
+ * decompress; decode; ef.sub_(decoded).  Two launches over a whole gradient set do the same:
+ *
+ * tplr_ef_encode_topk_pack_batch: for every chunk, ef <- ef * decay + grad (two roundings, as
+ * mul_ then add_), written back in place, and the payload of the updated ef as in
+ * tplr_encode_topk_pack_batch.  d_ef_desc and d_grad_desc are DEVICE arrays of n_tensors
+ * descriptors with the same shapes and chunk_begin; `dense` points to the error-feedback
+ * tensor and to the gradient respectively.  (A null round, neurons.py:148-149, is ef.zero_()
+ * followed by the plain tplr_encode_topk_pack_batch.)
+ *
+ * tplr_ef_subtract_batch: ef <- ef - decode(decompress(payload)) (neurons.py:162-171).  d_val
+ * holds the values the reference would decompress: the payload's own values, or the
+ * de-quantised ones when the compressor quantises.  use_dct != 0: inverse transform per chunk,
+ * k <= 64; use_dct == 0: only the k payload positions of each chunk change. */
+int tplr_ef_encode_topk_pack_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc* d_grad_desc,
+                                   int n_tensors, int64_t total_chunks, float decay, int k, int use_dct,
+                                   uint8_t* d_idx12, float* d_val, void* stream);
+int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, const tplr_tensor_desc* d_ef_desc,
+                           int n_tensors, int64_t total_chunks, int use_dct, void* stream);
+
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes
  * (a multiple of 16, both pointers 16-byte aligned) that moves exactly n_bytes each way.
  * Profilers' HBM traffic counters are scaled by what they report for this kernel. */

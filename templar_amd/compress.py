@@ -859,6 +859,56 @@ def batch_decompress_decode_batch(out: TensorBatch, idxs: Sequence[torch.Tensor]
     _lib.check(st, "tplr_decode_aggregate_batch")
 
 
+@torch.no_grad()
+def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, topk: int, *, use_dct: bool = True,
+                              compressor: "TopKCompressor | None" = None, null_round: bool = False):
+    """The miner's per-parameter loop of src/tplr/neurons.py:147-171 for a whole set of 2-D
+    parameters in two launches:
+
+        ef <- ef * decay + grad (or 0 on a null round), in place          (:148-152)
+        payload = compress(encode(ef))                                     (:155-159)
+        ef <- ef - decode(decompress(payload))                             (:162-171)
+
+    `ef` and `grad` describe the error-feedback tensors and the gradients (same shapes, same
+    order).  Returns (idx12, val, quant): the flat payload by global chunk id, and, when
+    `compressor` quantises, quant = list of (uint8 values, quant_params) per tensor (what the
+    reference's compress returns per parameter), the subtraction then using the de-quantised
+    values exactly as the reference's decompress does; otherwise quant is None."""
+    lib = _lib.load()
+    if len(ef) != len(grad) or ef.offsets != grad.offsets or ef.total_chunks != grad.total_chunks:
+        raise ValueError("error-feedback and gradient sets differ in shape")
+    k = _clamp_k(_CH * _CH, topk)
+    if k > 64:
+        raise NotImplementedError(f"top-{k}: the fused error-feedback step handles k up to 64")
+    dev, n = ef.device, ef.total_chunks
+    idx12 = torch.empty(n * (k // 2) * 3, dtype=torch.uint8, device=dev)
+    val = torch.empty((n, k), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        if null_round:
+            for t in ef.tensors:
+                t.zero_()
+            st = lib.tplr_encode_topk_pack_batch(_ptr(ef.table), len(ef), n, k, int(use_dct), _ptr(idx12), _ptr(val),
+                                                 _stream(dev))
+        else:
+            st = lib.tplr_ef_encode_topk_pack_batch(_ptr(ef.table), _ptr(grad.table), len(ef), n, C.c_float(decay), k,
+                                                    int(use_dct), _ptr(idx12), _ptr(val), _stream(dev))
+    _lib.check(st, "tplr_ef_encode_topk_pack_batch")
+    quant, sent = None, val
+    if compressor is not None and compressor.use_quantization:
+        quant, sent = [], torch.empty_like(val)
+        for i in range(len(ef)):
+            y, x, _, _ = ef.xshape(i)
+            b = ef.offsets[i]
+            q, qp = compressor._quantize_values(val[b:b + y * x].reshape(y, x, k))
+            quant.append((q, qp))
+            sent[b:b + y * x] = compressor._dequantize_values(q, qp).reshape(y * x, k)
+    with torch.cuda.device(dev):
+        st = lib.tplr_ef_subtract_batch(_ptr(idx12), _ptr(sent), k, _ptr(ef.table), len(ef), n, int(use_dct),
+                                        _stream(dev))
+    _lib.check(st, "tplr_ef_subtract_batch")
+    return idx12, val, quant
+
+
 # the names BASELINE.json's north star uses (DeMo-era)
 TransformDCT = ChunkingTransformer
 CompressDCT = TopKCompressor
@@ -866,6 +916,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

@@ -398,22 +398,38 @@ __global__ __launch_bounds__(64) void k_topk_rows(const float* __restrict__ coef
 // vector-ALU issue and by the latencies between its phases, so it is shaped for residency -
 // 8.5 KB + 1 KB of LDS and a register budget that admits three to four waves per SIMD - and
 // leaves the overlap of one wave's row loads with the other waves' arithmetic to the hardware.
-template <bool kTwo, bool kUseDct>
+// kEf: the miner's momentum update rides on the load (src/tplr/neurons.py:151-152): the chunk of
+// the error-feedback tensor becomes ef * decay + grad (two roundings, as mul_ then add_), is
+// written back in place and is what gets encoded.
+template <bool kTwo, bool kUseDct, bool kEf = false>
 __global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
                                                             int64_t total, int k, uint8_t* __restrict__ idx12,
-                                                            float* __restrict__ val) {
+                                                            float* __restrict__ val,
+                                                            const tplr_tensor_desc* __restrict__ grad_table,
+                                                            float decay) {
     __shared__ __align__(16) float buf[kHalfFloats];
     __shared__ uint64_t cand[kCandCap];
     const int lane = threadIdx.x;
     int64_t g0, g1;
     my_range(total, g0, g1);
     if (g0 >= g1) return;
-    Cursor c;
+    Cursor c, cg;
     cursor_seek(c, table, single, n_tensors, g0);
+    if (kEf) cursor_seek(cg, grad_table, single, n_tensors, g0);
     for (int64_t g = g0; g < g1; ++g) {
         float v[64], w[64];
         load_chunk_cols(v, c, lane);
+        if (kEf) {
+            load_chunk_cols(w, cg, lane);
+#pragma unroll
+            for (int r = 0; r < 64; ++r) {
+                const float m = v[r] * decay;
+                v[r] = m + w[r];
+            }
+            store_chunk_cols(v, (float*)c.base, c.ld, c.y, c.xc, lane);
+            if (g + 1 < g1) cursor_next(cg, g + 1);
+        }
         if (g + 1 < g1) cursor_next(c, g + 1);
         chunk_forward<kUseDct>(v, w, buf, lane);
         const Selected s = select_topk<kTwo>(w, buf, cand, lane, k, kUseDct ? kDctPow2Scale : 1.0f);
@@ -463,7 +479,10 @@ struct Counters {
 // offset) plus one lane-constant offset and each clip factor is a scalar; the whole payload of
 // a chunk sits in 2 * kUnits registers and is requested a whole transform pass before it is used.
 // Generic path (kUnits == 0): any k and peer count, entries loaded where they are used.
-template <bool kUseDct, int kUnits, int kCntBits>
+// kSubtract (fast path with the transform only): the destination receives destination - result
+// instead of the result (the error-feedback update of src/tplr/neurons.py:171); its rows are
+// requested before the second pass and arrive during it.
+template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false>
 __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
@@ -767,6 +786,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             constexpr int kAlways = kUnits > 8 ? kUnits - 8 : 1;  // units every served peer count uses
             int pos = dummy_pos;
             float cur = 0.f, add = 0.f;
+            float before[kSubtract ? 64 : 1];
+            if constexpr (kSubtract)
+                load_chunk_rows(before, (const void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane);
             // along b: v[k] = sum_b Z[b][lane] F[k][b]
             dct64_inv_hooked(v, [&](auto tag) {
                 constexpr int h = decltype(tag)::value;
@@ -788,6 +810,10 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                     }
                 }
             });
+            if constexpr (kSubtract) {
+#pragma unroll
+                for (int r = 0; r < 64; ++r) v[r] = before[r] - v[r];
+            }
             float ss = 0.f;
             if (sumsq) {
 #pragma unroll
@@ -886,6 +912,32 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         out_cur = out_next;
         out_next = out_after;
         t_next = t_after;
+    }
+}
+
+// ef <- ef - (the payload's entries) for chunks that are not transformed (use_dct = 0): the
+// reconstruction is the payload itself, so only k elements per chunk change
+// (src/tplr/neurons.py:162-171 with decode a pure re-layout).
+__global__ __launch_bounds__(64) void k_ef_subtract_sparse(const uint8_t* __restrict__ idx12,
+                                                           const float* __restrict__ val, int k,
+                                                           const tplr_tensor_desc* __restrict__ table,
+                                                           const tplr_tensor_desc single, int n_tensors,
+                                                           int64_t total) {
+    const int lane = threadIdx.x;
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
+    Cursor c;
+    cursor_seek(c, table, single, n_tensors, g0);
+    const int64_t idx_stride = k + (k >> 1);
+    for (int64_t g = g0; g < g1; ++g) {
+        gfloat* chunk0 = c.base + (c.y * 64) * c.ld + static_cast<int64_t>(c.xc) * 64;
+        for (int j = lane; j < k; j += 64) {
+            const uint32_t e = load_idx12(idx12 + g * idx_stride, j);
+            gfloat* t = chunk0 + static_cast<int64_t>(e >> 6) * c.ld + (e & 63);
+            *t = *t - val[g * k + j];
+        }
+        if (g + 1 < g1) cursor_next(c, g + 1);
     }
 }
 
@@ -1091,13 +1143,14 @@ static int persistent_grid(Kernel kernel, int64_t total) {
 
 template <typename Kernel>
 static int launch_encode_as(Kernel kernel, const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single,
-                            int n_tensors, int64_t total, int k, uint8_t* d_idx12, float* d_val, void* stream) {
+                            int n_tensors, int64_t total, int k, uint8_t* d_idx12, float* d_val, void* stream,
+                            const tplr_tensor_desc* d_grad_desc = nullptr, float decay = 0.f) {
     static int resident = 0;  // per kernel variant
     if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
     const int64_t need = ((total + 7) / 8) * 8;
     const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
     hipLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), d_desc, single, n_tensors, total, k,
-                       d_idx12, d_val);
+                       d_idx12, d_val, d_grad_desc, decay);
     return launch_status();
 }
 
@@ -1287,6 +1340,51 @@ int tplr_encode_topk_pack_batch(const tplr_tensor_desc* d_desc, int n_tensors, i
     if (total_chunks == 0) return 0;
     tplr_tensor_desc none = {};
     return launch_encode(d_desc, none, n_tensors, total_chunks, k, use_dct, d_idx12, d_val, stream);
+}
+
+int tplr_ef_encode_topk_pack_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc* d_grad_desc,
+                                   int n_tensors, int64_t total_chunks, float decay, int k, int use_dct,
+                                   uint8_t* d_idx12, float* d_val, void* stream) {
+    if (!d_ef_desc || !d_grad_desc || n_tensors < 1 || total_chunks < 0 || !d_idx12 || !d_val || k < 2 || (k & 1) ||
+        k > kCandCap)
+        return TPLR_E_BADARG;
+    if (total_chunks == 0) return 0;
+    tplr_tensor_desc none = {};
+    if (k > 32) {
+        if (use_dct)
+            return launch_encode_as(k_encode_topk_pack<true, true, true>, d_ef_desc, none, n_tensors, total_chunks, k,
+                                    d_idx12, d_val, stream, d_grad_desc, decay);
+        return launch_encode_as(k_encode_topk_pack<true, false, true>, d_ef_desc, none, n_tensors, total_chunks, k,
+                                d_idx12, d_val, stream, d_grad_desc, decay);
+    }
+    if (use_dct)
+        return launch_encode_as(k_encode_topk_pack<false, true, true>, d_ef_desc, none, n_tensors, total_chunks, k,
+                                d_idx12, d_val, stream, d_grad_desc, decay);
+    return launch_encode_as(k_encode_topk_pack<false, false, true>, d_ef_desc, none, n_tensors, total_chunks, k,
+                            d_idx12, d_val, stream, d_grad_desc, decay);
+}
+
+int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, const tplr_tensor_desc* d_ef_desc,
+                           int n_tensors, int64_t total_chunks, int use_dct, void* stream) {
+    if (!d_idx12 || !d_val || !d_ef_desc || n_tensors < 1 || total_chunks < 0 || k < 2 || (k & 1)) return TPLR_E_BADARG;
+    if (k > 64) return TPLR_E_TOOMANY;  // the register-resident decode path
+    if (total_chunks == 0) return 0;
+    tplr_tensor_desc none = {};
+    if (!use_dct) {
+        static int resident = 0;
+        if (resident == 0) resident = persistent_grid(k_ef_subtract_sparse, int64_t{1} << 40);
+        const int64_t need = ((total_chunks + 7) / 8) * 8;
+        hipLaunchKernelGGL(k_ef_subtract_sparse, dim3(static_cast<unsigned>(need < resident ? need : resident)),
+                           dim3(64), 0, static_cast<hipStream_t>(stream), d_idx12, d_val, k, d_ef_desc, none, n_tensors,
+                           total_chunks);
+        return launch_status();
+    }
+    PeerPtrs pp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) pp.idx[p] = nullptr, pp.val[p] = nullptr;
+    pp.idx[0] = d_idx12;
+    pp.val[0] = d_val;
+    return launch_decode_as(k_decode_aggregate<true, 8, 4, true>, pp, nullptr, 1, k, d_ef_desc, none, n_tensors,
+                            total_chunks, TPLR_REDUCE_MEAN, 0, nullptr, stream);
 }
 
 static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale, int n_peers,

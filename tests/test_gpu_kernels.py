@@ -501,3 +501,64 @@ def test_batch_encode_and_aggregate_match_per_tensor(dev):
         want = orc.batch_decompress([a.cpu().numpy() for a, _ in sl], [b.cpu().numpy() for _, b in sl],
                                     batch.xshape(i), 4096, clip_norm=False)  # unclipped reference for the pattern
         assert np.array_equal(c.cpu().numpy() != 0, want != 0)
+
+
+# ---------------------------------------------------------------- miner side: error-feedback step
+@pytest.mark.parametrize("use_dct,k,bins", [(True, 32, 0), (True, 64, 0), (False, 32, 0), (True, 32, 4), (False, 64, 256)])
+def test_error_feedback_step_matches_reference_sequence(dev, use_dct, k, bins):
+    # three tensors of different shapes, walked as one batch (src/tplr/neurons.py:147-171 per parameter)
+    shapes = [(128, 192), (64, 64), (256, 128)]
+    decay = 0.95
+    efs = [t3(s, 400 + i, row_scale=True) for i, s in enumerate(shapes)]
+    grads = [t3(s, 500 + i, row_scale=True) * 0.5 for i, s in enumerate(shapes)]
+    d_ef = [e.clone().to(dev) for e in efs]
+    d_gr = [g.to(dev) for g in grads]
+    comp = tc.TopKCompressor(use_quantization=bins > 0, quantization_bins=bins or 256, quantization_range=6)
+    eb, gb = tc.TensorBatch(d_ef), tc.TensorBatch(d_gr)
+    idx12, val, quant = tc.error_feedback_step_batch(eb, gb, decay, k, use_dct=use_dct, compressor=comp)
+    assert (quant is None) == (bins == 0)
+    tr = tc.ChunkingTransformer(_Stub(d_ef), 64)
+    for i, s in enumerate(shapes):
+        # the accumulated momentum is exact: two roundings, as mul_ then add_
+        acc = (efs[i] * decay) + grads[i]
+        # selection on the device's own coefficients of that exact tensor, values bit-exact
+        coef = tr.encode(acc.to(dev), use_dct=use_dct).cpu().numpy()
+        ef_acc, want_i, want_v, want_new = orc.error_feedback_step(efs[i].numpy(), grads[i].numpy(), decay, k,
+                                                                   use_dct=use_dct, quant_bins=bins, coef_override=coef)
+        assert np.array_equal(ef_acc, acc.numpy())
+        got_i, got_v = eb.payload_slice(i, idx12, val, k)
+        assert np.array_equal(got_i.cpu().numpy(), want_i)
+        assert np.array_equal(got_v.cpu().numpy(), want_v)
+        # the error feedback left behind: within fp32 tolerance of the reference sequence
+        got_new = d_ef[i].cpu().numpy()
+        assert np.abs(got_new - want_new).max() <= TOL * np.abs(ef_acc).max()
+        if not use_dct and bins == 0:
+            # no transform, no quantiser: the sent entries are removed exactly, the rest untouched
+            assert np.array_equal(got_new, want_new)
+        if quant is not None:
+            q, qp = quant[i]
+            wq, wqp = orc.quantize(want_v, bins, 6.0)
+            assert np.array_equal(q.cpu().numpy(), wq)
+
+
+def test_error_feedback_null_round_and_equivalence_with_separate_calls(dev):
+    shape = (192, 128)
+    ef0 = t3(shape, 77, row_scale=True)
+    gr = t3(shape, 78, row_scale=True)
+    # fused step == the reference's call sequence through this module's own API, bitwise
+    d_ef = ef0.clone().to(dev)
+    eb, gb = tc.TensorBatch([d_ef]), tc.TensorBatch([gr.to(dev)])
+    idx12, val, _ = tc.error_feedback_step_batch(eb, gb, 0.9, 32, use_dct=True)
+    tr, comp = tc.ChunkingTransformer(_Stub([d_ef]), 64), tc.TopKCompressor()
+    ref = ef0.clone().to(dev)
+    ref.mul_(0.9)
+    ref.add_(gr.to(dev))
+    i2, v2, xshape, totalk = comp.compress(tr.encode(ref, use_dct=True), 32)
+    ref.sub_(tr.decode(comp.decompress(ref, i2, v2, xshape, totalk), use_dct=True))
+    assert torch.equal(idx12, i2.reshape(-1)) and torch.equal(val.reshape(v2.shape), v2)
+    assert torch.equal(d_ef, ref)
+    # null round: the momentum is cleared, the payload is that of zeros
+    idx12, val, _ = tc.error_feedback_step_batch(eb, gb, 0.9, 32, use_dct=True, null_round=True)
+    assert float(d_ef.abs().max()) == 0.0 and float(val.abs().max()) == 0.0
+    assert np.array_equal(orc.unpack12(idx12.cpu().numpy(), (6, 32))[0], np.arange(32))
+
