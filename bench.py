@@ -51,7 +51,7 @@ def parse():
     ap.add_argument("--workload", default="cfg3_llama1b", help="cfg1_2048x2048 | cfg2_llama150m | cfg3_llama1b | cfg5_72b_block")
     ap.add_argument("--peers", type=int, default=15)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--profile", choices=["encode", "aggregate", "copy"], default=None,
+    ap.add_argument("--profile", choices=["encode", "aggregate", "miner", "copy"], default=None,
                     help="run only that phase's batched launches --steps times (for rocprofv3) and print nothing; "
                          "'copy' runs the library's calibration copy of 1 GiB instead (counter scaling)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline sample")
@@ -153,11 +153,11 @@ def main():
 
     import templar_amd.compress as tc
     import workloads
+    from templar_amd import _lib as _lib_mod
 
     dev = torch.device("cuda:0")
     if args.profile == "copy":
-        from templar_amd import _lib
-
+        _lib = _lib_mod
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB
         dst = torch.empty_like(src)
         lib = _lib.load()
@@ -204,6 +204,36 @@ def main():
 
     if flat_1d is not None:
         tr.shape_dict[flat_1d.shape[0]] = 64
+
+    # ---- miner side (src/tplr/neurons.py:147-171): momentum update + encode, then subtract the
+    # reconstruction, over the whole set in two launches; separate error-feedback tensors
+    def miner_figures(steps, warmup):
+        efs = [torch.zeros_like(g) for g in two_d]
+        eb = tc.TensorBatch(efs)
+        lib = _lib_mod.load()
+        st = torch.cuda.current_stream(dev).cuda_stream
+        k1 = lambda: _lib_mod.check(lib.tplr_ef_encode_topk_pack_batch(  # noqa: E731
+            eb.table.data_ptr(), batch.table.data_ptr(), len(eb), n_chunks, 0.95, k, 1, idx_buf.data_ptr(),
+            val_buf.data_ptr(), st), "ef_encode")
+        k2 = lambda: _lib_mod.check(lib.tplr_ef_subtract_batch(  # noqa: E731
+            idx_buf.data_ptr(), val_buf.data_ptr(), k, eb.table.data_ptr(), len(eb), n_chunks, 1, st), "ef_subtract")
+        both = lambda: (k1(), k2())  # noqa: E731
+        ms_both, _ = event_ms(both, steps, warmup)
+        ms1, _ = event_ms(k1, steps, 1)
+        ms2, _ = event_ms(k2, steps, 1)
+        b1 = n_chunks * (2 * 16384 + 16384 + 11 * k // 2)
+        b2 = n_chunks * (16384 + 11 * k // 2 + 16384)
+        return {
+            "what": "ef = ef*decay + grad, encode+top-k+pack, ef -= decode(payload): two launches over the set",
+            "ms": round(ms_both, 4), "GBps": round((b1 + b2) / (ms_both * 1e-3) / 1e9, 2),
+            "frac_of_hbm_peak": round((b1 + b2) / (ms_both * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "update_encode_ms": round(ms1, 4), "update_encode_bytes": b1,
+            "subtract_decoded_ms": round(ms2, 4), "subtract_decoded_bytes": b2,
+        }
+
+    if args.profile == "miner":
+        miner_figures(args.steps, args.warmup)
+        return
     if args.profile == "encode":
         event_ms(encode2d_only, args.steps, args.warmup)
         return
@@ -214,6 +244,7 @@ def main():
         enc2d_ms, _ = event_ms(encode2d_only, args.steps, 1)      # the fused 2-D kernel alone (dominant)
         enc_pt_ms, _ = event_ms(encode_per_tensor, max(3, args.steps // 2), 1)
     enc2d_bytes = n_chunks * (16384 + 11 * k // 2)
+    miner = miner_figures(max(3, args.steps // 2), 2) if k <= 64 else None
 
     # ---- P peers' flat payloads for the aggregation side (peer p = 0.5 shared + own)
     idxs, vals = [], []
@@ -287,6 +318,8 @@ def main():
             "launches_per_step": 1, "bytes_per_launch": agg_bytes, "ms_per_launch": round(aggk_ms, 4),
         },
     }
+    if miner is not None:
+        result["error_feedback_step"] = miner
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, k, P, args.cpu_seconds)
     print(json.dumps(result))

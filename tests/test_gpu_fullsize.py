@@ -153,3 +153,55 @@ def test_full_set_aggregate_properties(dev):
     # a row may differ only where the k-th and a dropped coefficient (a rounding-level zero) tie
     assert float(same.float().mean()) > 0.999
     assert float((val_r.abs().sum(dim=1) - val_a.abs().sum(dim=1)).abs().max()) <= 1e-4 * float(val_a.abs().sum(dim=1).max())
+
+
+def test_full_set_error_feedback_step(dev):
+    """src/tplr/neurons.py:147-171 over the whole 1B set in two launches.  Properties: the
+    payload is that of the accumulated momentum (ef * decay + grad, bit-exact); what is left
+    behind has (numerically) nothing at the sent coefficients and everything else untouched;
+    energy splits between the payload and the remainder (Parseval)."""
+    grads, k = _set("cfg3_llama1b", dev)
+    efs = [workloads.student_t3(tuple(g.shape), 9000 + j, row_scale=True, device=dev) for j, g in enumerate(grads)]
+    acc = [e * 0.95 + g for e, g in zip(efs, grads)]  # mul then add, as the reference does in place
+    eb, gb = tc.TensorBatch(efs), tc.TensorBatch(grads)
+    n = eb.total_chunks
+    idx12, val, quant = tc.error_feedback_step_batch(eb, gb, 0.95, k, use_dct=True)
+    assert quant is None
+    want_i, want_v = tc.encode_compress_batch(tc.TensorBatch(acc), k, use_dct=True)
+    assert torch.equal(idx12, want_i) and torch.equal(val, want_v)
+    # energy: |acc|^2 = |payload|^2 + |remainder|^2 for an orthonormal transform
+    e_acc = sum(float((a.double() ** 2).sum()) for a in acc)
+    e_rem = sum(float((e.double() ** 2).sum()) for e in efs)
+    e_pay = float((val.double() ** 2).sum())
+    assert abs(e_acc - e_pay - e_rem) <= 1e-5 * e_acc
+    # the remainder's coefficients: ~0 where sent, unchanged elsewhere (checked on the largest tensor)
+    big = max(range(len(efs)), key=lambda i: efs[i].numel())
+
+    class M:
+        def named_parameters(self):
+            from types import SimpleNamespace
+            yield "w", SimpleNamespace(requires_grad=True, shape=tuple(efs[big].shape), dtype=torch.float32, device=dev)
+
+    tr = tc.ChunkingTransformer(M(), 64)
+    c_rem = tr.encode(efs[big], use_dct=True).reshape(-1, 4096)
+    c_acc = tr.encode(acc[big], use_dct=True).reshape(-1, 4096)
+    i_big, _ = eb.payload_slice(big, idx12, val, k)
+    idx = tc.unpack_12bit_indices(i_big, (c_rem.shape[0], k))
+    sent = torch.zeros_like(c_rem, dtype=torch.bool).scatter_(1, idx, True)
+    top = float(c_acc.abs().max())
+    assert float(c_rem[sent].abs().max()) <= TOL * top
+    assert float((c_rem - c_acc)[~sent].abs().max()) <= TOL * top
+    # without the transform the sent entries are removed exactly
+    efs2 = [workloads.student_t3(tuple(g.shape), 9000 + j, row_scale=True, device=dev) for j, g in enumerate(grads[:8])]
+    acc2 = [e * 0.95 + g for e, g in zip(efs2, grads[:8])]
+    eb2 = tc.TensorBatch(efs2)
+    i2, v2, _ = tc.error_feedback_step_batch(eb2, tc.TensorBatch(grads[:8]), 0.95, k, use_dct=False)
+    for j, (e, a) in enumerate(zip(efs2, acc2)):
+        ij, vj = eb2.payload_slice(j, i2, v2, k)
+        y, x = a.shape[0] // 64, a.shape[1] // 64
+        ch = a.reshape(y, 64, x, 64).permute(0, 2, 1, 3).reshape(y * x, 4096)
+        ix = tc.unpack_12bit_indices(ij, (y * x, k))
+        assert torch.equal(ch.gather(1, ix), vj.reshape(y * x, k))
+        want = ch.scatter(1, ix, 0.0).reshape(y, x, 64, 64).permute(0, 2, 1, 3).reshape(a.shape)
+        assert torch.equal(e, want)
+
