@@ -280,6 +280,13 @@ def main():
     aggk_ms, _ = event_ms(aggregate_kernel_only, agg_steps, 1)
     agg_pt_ms, _ = event_ms(aggregate_per_tensor, 3, 1)
     agg_bytes = n_chunks * (P * 11 * k // 2 + 16384)
+    # validator-side checks on the same payloads: pairwise index overlap, repeats, bounds
+    stats = None
+    if P <= 32:
+        st_ms, _ = event_ms(lambda: tc.index_stats_batch(out_batch, idxs, k), agg_steps, 1)
+        st_bytes = n_chunks * P * (k + k // 2)
+        stats = {"what": f"pairwise index overlap + repeats + bounds of {P} peers' packed indices, one launch",
+                 "ms": round(st_ms, 4), "GBps": round(st_bytes / (st_ms * 1e-3) / 1e9, 2), "bytes": st_bytes}
 
     result = {
         "metric": "encode+topk+pack GB/s and 15-peer decode-aggregate ms, 1B grads, 1 GPU",
@@ -320,6 +327,8 @@ def main():
     }
     if miner is not None:
         result["error_feedback_step"] = miner
+    if stats is not None:
+        result["index_stats"] = stats
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, k, P, args.cpu_seconds)
     print(json.dumps(result))

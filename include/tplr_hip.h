@@ -211,6 +211,23 @@ int tplr_ef_encode_topk_pack_batch(const tplr_tensor_desc* d_ef_desc, const tplr
 int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, const tplr_tensor_desc* d_ef_desc,
                            int n_tensors, int64_t total_chunks, int use_dct, void* stream);
 
+/* ---- validator side: checks on the packed index streams ------------------------------
+ * For up to 32 peers whose flat payloads share one row layout (d_desc: n_tensors descriptors, of
+ * which only chunk_begin, x_chunks and y_chunks are read; a parameter of n rows that are not
+ * 64x64 chunks is one descriptor with x_chunks = n, y_chunks = 1), per tensor t:
+ *   d_pair[(t * P + p) * P + q], p < q: entries of peer p that also occur in the same row of
+ *       peer q, summed over the tensor's rows - `(a == b).any(-1).sum(-1)` summed over chunks in
+ *       check_uid_index_overlap (src/tplr/neurons.py:1373-1378); divide by k * rows for its
+ *       `mean_frac`;
+ *   d_dup[t * P + p]: entries of peer p that repeat an earlier entry of their row;
+ *   d_max[t * P + p]: largest index of peer p, for the bounds check of
+ *       Comms.check_compressed_indices (src/tplr/comms.py:2573-2581).
+ * The three arrays are accumulated into with atomics: the caller clears d_pair and d_dup to 0
+ * and d_max to -1.  k even, at most 4096; indices are 12-bit by construction. */
+int tplr_index_stats_batch(const uint8_t* const* h_idx12, int n_peers, int k, const tplr_tensor_desc* d_desc,
+                           int n_tensors, int64_t total_rows, uint64_t* d_pair, uint64_t* d_dup, int32_t* d_max,
+                           void* stream);
+
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes
  * (a multiple of 16, both pointers 16-byte aligned) that moves exactly n_bytes each way.
  * Profilers' HBM traffic counters are scaled by what they report for this kernel. */

@@ -260,3 +260,34 @@ def error_feedback_step(ef, grad, decay: float, topk: int, *, use_dct: bool = Tr
     recon = decode2d(decompress(idx12, sent, xshape, totalk), use_dct=use_dct)
     return ef, idx12, val, ef - recon
 
+
+# ---------------------------------------------------------------- index checks
+def index_overlap(idx_list):
+    """Pairwise overlap of peers' index rows, as check_uid_index_overlap computes it per
+    parameter (src/tplr/neurons.py:1366-1378): idx_list[p] is peer p's (C, k) int64 indices.
+    Returns (inter, frac): inter[i, j] (i < j) = sum over chunks of `(a == b).any(-1).sum(-1)`,
+    frac[i, j] = mean over chunks of inter_c / k (its `mean_frac`)."""
+    P = len(idx_list)
+    rows = [_c(i, np.int64).reshape(-1, np.shape(i)[-1]) for i in idx_list]
+    Cn, k = rows[0].shape
+    inter = np.zeros((P, P), dtype=np.int64)
+    frac = np.zeros((P, P), dtype=np.float64)
+    for i in range(P):
+        for j in range(i + 1, P):
+            a = rows[i][:, :, None]          # (C, k, 1)   :1373
+            b = rows[j][:, None, :]          # (C, 1, k)   :1374
+            per_chunk = (a == b).any(-1).sum(-1)  # :1375
+            inter[i, j] = per_chunk.sum()
+            frac[i, j] = (per_chunk.astype(np.float32) / k).mean()  # :1376
+    return inter, frac
+
+
+def index_bounds(idx, totalk: int):
+    """The bounds check of Comms.check_compressed_indices (src/tplr/comms.py:2573-2581):
+    None if every index is in [0, totalk), else the first offending index."""
+    t = _c(idx, np.int64).reshape(-1)
+    if t.size == 0:
+        raise ValueError("empty index list")
+    bad = t[(t < 0) | (t >= totalk)]
+    return None if bad.size == 0 else int(bad[0])
+

@@ -909,6 +909,60 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
     return idx12, val, quant
 
 
+@torch.no_grad()
+def index_stats_batch(batch: "TensorBatch | Sequence[int]", idxs: Sequence[torch.Tensor], k: int):
+    """Checks on P peers' packed index streams in one launch.
+
+    `batch` is a TensorBatch (rows = its 64x64 chunks), or a list of row counts per parameter
+    for payloads whose rows are not chunks.  Returns (pair, dup, top):
+      pair (T, P, P) int64: pair[t, i, j] for i < j = entries of peer i that also occur in the same
+          row of peer j, summed over parameter t's rows - what check_uid_index_overlap
+          (src/tplr/neurons.py:1373-1378) sums before dividing by k and averaging over rows;
+      dup (T, P) int64: repeated entries inside a row (a top-k selection has none);
+      top (T, P) int32: the largest index, for the bounds check of check_compressed_indices
+          (src/tplr/comms.py:2573-2581)."""
+    import numpy as np
+
+    lib = _lib.load()
+    P = len(idxs)
+    if P > 32:
+        raise NotImplementedError(f"{P} peers: the index statistics kernel takes up to 32")
+    dev = idxs[0].device
+    _need_device(idxs[0], "index_stats_batch")
+    if isinstance(batch, TensorBatch):
+        table, T, total = batch.table, len(batch), batch.total_chunks
+    else:
+        counts = [int(c) for c in batch]
+        desc = np.zeros(len(counts), dtype=np.dtype([("dense", "<u8"), ("ld", "<i8"), ("chunk_begin", "<i8"),
+                                                     ("x_chunks", "<i4"), ("y_chunks", "<i4")]))
+        begin = 0
+        for i, c in enumerate(counts):
+            desc[i] = (0, 0, begin, c, 1)
+            begin += c
+        table, T, total = torch.from_numpy(desc.view(np.uint8).copy()).to(dev), len(counts), begin
+    for i in idxs:
+        if i.dtype != torch.uint8:
+            raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
+        if i.numel() * 2 != total * k * 3:
+            raise RuntimeError(f"{i.numel()} index bytes for {total} rows of k={k}")
+    pair = torch.zeros((T, P, P), dtype=torch.int64, device=dev)
+    dup = torch.zeros((T, P), dtype=torch.int64, device=dev)
+    top = torch.full((T, P), -1, dtype=torch.int32, device=dev)
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+    with torch.cuda.device(dev):
+        st = lib.tplr_index_stats_batch(ip, P, k, _ptr(table), T, total, _ptr(pair), _ptr(dup), _ptr(top), _stream(dev))
+    _lib.check(st, "tplr_index_stats_batch")
+    return pair, dup, top
+
+
+def overlap_fractions(pair: torch.Tensor, rows: Sequence[int], k: int) -> torch.Tensor:
+    """Size-weighted average overlap per peer pair from index_stats_batch's counts: what
+    check_uid_index_overlap accumulates in pair_acc (src/tplr/neurons.py:1376-1385, :1393):
+    sum_t mean_frac_t * (C_t k) / sum_t (C_t k) = sum_t pair[t] / (k sum_t C_t)."""
+    total = float(sum(int(r) for r in rows)) * k
+    return pair.sum(dim=0).double() / total
+
+
 # the names BASELINE.json's north star uses (DeMo-era)
 TransformDCT = ChunkingTransformer
 CompressDCT = TopKCompressor
@@ -916,6 +970,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

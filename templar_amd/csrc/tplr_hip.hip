@@ -941,6 +941,103 @@ __global__ __launch_bounds__(64) void k_ef_subtract_sparse(const uint8_t* __rest
     }
 }
 
+// -----------------------------------------------------------------------------------------
+// Statistics of the packed index streams of up to 32 peers, per tensor:
+//   pair[t][p][q] (p < q) = number of entries of peer p that also occur in the same row of peer q,
+//                           summed over the tensor's rows: the `(a == b).any(-1).sum(-1)` of
+//                           check_uid_index_overlap (src/tplr/neurons.py:1373-1378) before its
+//                           division by k and mean over rows;
+//   dup[t][p]             = entries of peer p that repeat an earlier entry of their own row
+//                           (a top-k selection has none);
+//   mx[t][p]              = largest index of peer p (the bounds check of
+//                           Comms.check_compressed_indices, src/tplr/comms.py:2573-2581).
+// One wave per row at a time: the row's 4096 possible indices each get a 32-bit mask of the peers
+// that sent them (LDS, integer atomics), then every entry looks its mask up and counts the
+// higher-numbered peers in it.  Totals collect in LDS and go out with one 64-bit atomic per
+// non-zero counter when the wave leaves a tensor.
+// -----------------------------------------------------------------------------------------
+constexpr int kStatPeers = 32;
+struct IdxPtrs {
+    const uint8_t* idx[kStatPeers];
+};
+
+__global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int k,
+                                                    const tplr_tensor_desc* __restrict__ table,
+                                                    const tplr_tensor_desc single, int n_tensors, int64_t total,
+                                                    unsigned long long* __restrict__ pair,
+                                                    unsigned long long* __restrict__ dup, int* __restrict__ mx) {
+    __shared__ __align__(16) uint32_t mask[4096];
+    __shared__ uint32_t pair_l[kStatPeers * kStatPeers];
+    __shared__ uint32_t dup_l[kStatPeers];
+    __shared__ int mx_l[kStatPeers];
+    const int lane = threadIdx.x;
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
+    const int64_t idx_stride = k + (k >> 1);
+    Cursor c;
+    cursor_seek(c, table, single, n_tensors, g0);
+    auto clear_totals = [&]() {
+        for (int i = lane; i < kStatPeers * kStatPeers; i += 64) pair_l[i] = 0;
+        if (lane < kStatPeers) dup_l[lane] = 0, mx_l[lane] = -1;
+        wave_lds_fence();
+    };
+    auto flush_totals = [&](int t) {
+        wave_lds_fence();
+        for (int i = lane; i < kStatPeers * kStatPeers; i += 64) {
+            const int p = i / kStatPeers, q = i - p * kStatPeers;
+            if (pair_l[i] && p < P && q < P)
+                atomicAdd(&pair[(static_cast<int64_t>(t) * P + p) * P + q], static_cast<unsigned long long>(pair_l[i]));
+        }
+        if (lane < P) {
+            if (dup_l[lane]) atomicAdd(&dup[static_cast<int64_t>(t) * P + lane], static_cast<unsigned long long>(dup_l[lane]));
+            if (mx_l[lane] >= 0) atomicMax(&mx[static_cast<int64_t>(t) * P + lane], mx_l[lane]);
+        }
+        wave_lds_fence();
+    };
+    clear_totals();
+    int t_cur = c.t;
+    for (int64_t g = g0; g < g1; ++g) {
+        if (c.t != t_cur) {  // wave-uniform
+            flush_totals(t_cur);
+            clear_totals();
+            t_cur = c.t;
+        }
+        const uint4 z = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int q = 0; q < 16; ++q) reinterpret_cast<uint4*>(mask)[q * 64 + lane] = z;
+        wave_lds_fence();
+        for (int p = 0; p < P; ++p) {
+            const gbyte* row = (const gbyte*)ip.idx[p] + g * idx_stride;
+            int top = -1;
+            for (int j = lane; j < k; j += 64) {
+                const uint32_t e = load_idx12(row, j);
+                const uint32_t old = atomicOr(&mask[e], 1u << p);
+                if ((old >> p) & 1u) atomicAdd(&dup_l[p], 1u);
+                top = top > static_cast<int>(e) ? top : static_cast<int>(e);
+            }
+            top = static_cast<int>(wave_max_u32(static_cast<uint32_t>(top + 1))) - 1;
+            if (lane == 0 && top > mx_l[p]) mx_l[p] = top;
+        }
+        wave_lds_fence();
+        for (int p = 0; p + 1 < P; ++p) {
+            const gbyte* row = (const gbyte*)ip.idx[p] + g * idx_stride;
+            for (int j = lane; j < k; j += 64) {
+                const uint32_t e = load_idx12(row, j);
+                uint32_t m = mask[e] >> (p + 1);  // the peers after p that sent e too
+                while (m) {
+                    const int q = p + 1 + __builtin_ctz(m);
+                    atomicAdd(&pair_l[p * kStatPeers + q], 1u);
+                    m &= m - 1;
+                }
+            }
+        }
+        wave_lds_fence();
+        if (g + 1 < g1) cursor_next(c, g + 1);
+    }
+    flush_totals(t_cur);
+}
+
 // generic rows (1-D tensors, un-chunked 2-D rows): exact source-order accumulation
 __global__ __launch_bounds__(64) void k_scatter_rows(const uint8_t* __restrict__ idx12,
                                                      const int64_t* __restrict__ idx64,
@@ -1513,6 +1610,29 @@ int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr
     }
     hipLaunchKernelGGL(k_segment_sumsq, dim3(static_cast<unsigned>(n_tensors) * n_peers * n_slices), dim3(1024), 0,
                        static_cast<hipStream_t>(stream), vp, n_peers, k, n_slices, d_desc, d_sumsq);
+    return launch_status();
+}
+
+int tplr_index_stats_batch(const uint8_t* const* h_idx12, int n_peers, int k, const tplr_tensor_desc* d_desc,
+                           int n_tensors, int64_t total_rows, uint64_t* d_pair, uint64_t* d_dup, int32_t* d_max,
+                           void* stream) {
+    if (!h_idx12 || !d_desc || !d_pair || !d_dup || !d_max || n_peers < 1 || n_tensors < 1 || total_rows < 0 || k < 2 ||
+        (k & 1) || k > 4096)
+        return TPLR_E_BADARG;
+    if (n_peers > kStatPeers) return TPLR_E_TOOMANY;
+    if (total_rows == 0) return 0;
+    IdxPtrs ip;
+    for (int p = 0; p < kStatPeers; ++p) {
+        ip.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
+        if (p < n_peers && !ip.idx[p]) return TPLR_E_BADARG;
+    }
+    static int resident = 0;
+    if (resident == 0) resident = persistent_grid(k_index_stats, int64_t{1} << 40);
+    const int64_t need = ((total_rows + 7) / 8) * 8;
+    tplr_tensor_desc none = {};
+    hipLaunchKernelGGL(k_index_stats, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), ip, n_peers, k, d_desc, none, n_tensors, total_rows,
+                       reinterpret_cast<unsigned long long*>(d_pair), reinterpret_cast<unsigned long long*>(d_dup), d_max);
     return launch_status();
 }
 

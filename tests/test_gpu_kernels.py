@@ -562,3 +562,47 @@ def test_error_feedback_null_round_and_equivalence_with_separate_calls(dev):
     assert float(d_ef.abs().max()) == 0.0 and float(val.abs().max()) == 0.0
     assert np.array_equal(orc.unpack12(idx12.cpu().numpy(), (6, 32))[0], np.arange(32))
 
+
+# ---------------------------------------------------------------- validator side: index checks
+def test_index_stats_match_reference_overlap(dev):
+    rng = np.random.default_rng(21)
+    P, k = 5, 32
+    shapes = [(128, 192), (64, 128)]
+    batch = tc.TensorBatch([torch.zeros(s, device=dev) for s in shapes])
+    n = batch.total_chunks
+    base = np.stack([rng.permutation(4096)[:k] for _ in range(n)])
+    rows = []
+    for p in range(P):
+        own = np.stack([rng.permutation(4096)[:k] for _ in range(n)])
+        keep = rng.random((n, k)) < 0.3 * p / P        # peers share more and more of `base`
+        r = np.where(keep, base, own)
+        # repair accidental repeats inside a row, then plant three real ones for peer 3
+        for c in range(n):
+            u, first = np.unique(r[c], return_index=True)
+            if len(u) < k:
+                spare = np.setdiff1d(np.arange(4096), u)[: k - len(u)]
+                r[c, np.setdiff1d(np.arange(k), first)] = spare
+        rows.append(r.astype(np.int64))
+    rows[3][0, 5] = rows[3][0, 4]
+    rows[3][7, 31] = rows[3][7, 0]
+    rows[3][n - 1, 1] = rows[3][n - 1, 0]
+    idxs = [torch.from_numpy(orc.pack12(r)).to(dev) for r in rows]
+    pair, dup, top = tc.index_stats_batch(batch, idxs, k)
+    assert pair.shape == (2, P, P)
+    for t in range(2):
+        b0, b1 = batch.offsets[t], (batch.offsets[t + 1] if t + 1 < len(shapes) else n)
+        inter, frac = orc.index_overlap([r[b0:b1] for r in rows])
+        assert np.array_equal(np.triu(pair[t].cpu().numpy(), 1), inter)
+        assert np.array_equal(top[t].cpu().numpy(), [r[b0:b1].max() for r in rows])
+    assert dup.sum(dim=0).cpu().tolist() == [0, 0, 0, 3, 0]
+    counts = [(s[0] // 64) * (s[1] // 64) for s in shapes]
+    fr = tc.overlap_fractions(pair, counts, k).cpu().numpy()
+    inter_all, _ = orc.index_overlap(rows)
+    assert np.allclose(np.triu(fr, 1), inter_all / (n * k))
+    # rows that are not chunks: (rows, k) with k = 4, indices below 64; the reference's own known answers
+    a = torch.from_numpy(orc.pack12(np.array([[0, 1, 2, 3]]))).to(dev)
+    b = torch.from_numpy(orc.pack12(np.array([[2, 3, 4, 5]]))).to(dev)
+    pair, dup, top = tc.index_stats_batch([1], [a, b, a], 4)
+    assert pair[0].cpu().tolist() == [[0, 2, 4], [0, 0, 2], [0, 0, 0]] and top[0].cpu().tolist() == [3, 5, 3]
+    assert orc.index_bounds(np.array([0, 1, 2, 3]), 64) is None
+

@@ -301,3 +301,26 @@ def test_golden_fixture_is_reproduced():
     idx, val, _, _ = orc.compress(coef, 32)
     assert np.array_equal(idx, z["idx12"]) and np.array_equal(val, z["val"])
     assert np.array_equal(orc.decode2d(orc.decompress(idx, val, coef.shape, 4096)), z["recon"])
+
+
+# ---------------------------------------------------------------- index checks
+def test_index_overlap_reference_known_answers():
+    # the inline cases of the reference's tests/unit/test_idx_overlap.py:88-140:
+    # identical rows -> 1.0, disjoint -> 0.0, two of four shared -> 0.5
+    same = np.array([[0, 1, 2, 3]])
+    inter, frac = orc.index_overlap([same, same])
+    assert inter[0, 1] == 4 and frac[0, 1] == 1.0
+    inter, frac = orc.index_overlap([np.array([[0, 1, 2, 3]]), np.array([[4, 5, 6, 7]])])
+    assert inter[0, 1] == 0 and frac[0, 1] == 0.0
+    inter, frac = orc.index_overlap([np.array([[0, 1, 2, 3]]), np.array([[2, 3, 4, 5]])])
+    assert inter[0, 1] == 2 and frac[0, 1] == 0.5
+    # against set intersection on random duplicate-free rows, three peers, several chunks
+    rng = np.random.default_rng(5)
+    rows = [np.stack([rng.permutation(256)[:16] for _ in range(7)]) for _ in range(3)]
+    inter, frac = orc.index_overlap(rows)
+    for i in range(3):
+        for j in range(i + 1, 3):
+            want = sum(len(set(rows[i][c]) & set(rows[j][c])) for c in range(7))
+            assert inter[i, j] == want and abs(frac[i, j] - want / (7 * 16)) < 1e-6
+    assert orc.index_bounds(np.array([0, 63]), 64) is None and orc.index_bounds(np.array([1, 64, 70]), 64) == 64
+
