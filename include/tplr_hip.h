@@ -228,6 +228,16 @@ int tplr_index_stats_batch(const uint8_t* const* h_idx12, int n_peers, int k, co
                            int n_tensors, int64_t total_rows, uint64_t* d_pair, uint64_t* d_dup, int32_t* d_max,
                            void* stream);
 
+/* ---- payload staging: de-quantisation of a flat payload --------------------------------
+ * TopKCompressor._dequantize_values (src/tplr/compress.py:637-643) for every parameter of one
+ * peer's flat payload at once (the per-parameter loop of maybe_dequantize_values, :646-696,
+ * src/tplr/neurons.py:325): d_val[i] = d_lookup[t * n_bins + d_codes[i]] + d_shift[t], t the
+ * tensor that row i / k belongs to (d_desc: chunk_begin only).  k a multiple of 4, n_bins <= 256;
+ * codes >= n_bins read the last bin (the reference would raise an index error). */
+int tplr_dequantize_batch(const uint8_t* d_codes, const float* d_lookup, const float* d_shift, int n_bins, int k,
+                          const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_rows, float* d_val,
+                          void* stream);
+
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes
  * (a multiple of 16, both pointers 16-byte aligned) that moves exactly n_bytes each way.
  * Profilers' HBM traffic counters are scaled by what they report for this kernel. */

@@ -910,6 +910,31 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
 
 
 @torch.no_grad()
+def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[QuantParamsT], k: int,
+                     out: torch.Tensor | None = None) -> torch.Tensor:
+    """One peer's flat payload of 8-bit codes -> fp32 values (total_chunks, k), every parameter
+    with its own (shift, lookup): TopKCompressor.maybe_dequantize_values' per-parameter loop
+    (reference :646-696, src/tplr/neurons.py:325) in one launch.  qparams[i] is parameter i's
+    5-tuple as the reference's compress returns it."""
+    lib = _lib.load()
+    dev, n = batch.device, batch.total_chunks
+    if len(qparams) != len(batch):
+        raise IndexError(f"Mismatch in val lengths: dequant({len(qparams)}) vs original({len(batch)})")
+    if codes.dtype != torch.uint8 or codes.numel() != n * k:
+        raise RuntimeError(f"{codes.numel()} codes of {codes.dtype} for {n} chunks of k={k}")
+    n_bins = int(qparams[0][3].numel())
+    lookup = torch.stack([qp[3].to(dev, torch.float32).reshape(n_bins) for qp in qparams]).contiguous()
+    shift = torch.stack([torch.as_tensor(qp[0], dtype=torch.float32, device=dev).reshape(()) for qp in qparams])
+    if out is None:
+        out = torch.empty((n, k), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        st = lib.tplr_dequantize_batch(_ptr(codes.contiguous()), _ptr(lookup), _ptr(shift), n_bins, k, _ptr(batch.table),
+                                       len(batch), n, _ptr(out), _stream(dev))
+    _lib.check(st, "tplr_dequantize_batch")
+    return out
+
+
+@torch.no_grad()
 def index_stats_batch(batch: "TensorBatch | Sequence[int]", idxs: Sequence[torch.Tensor], k: int):
     """Checks on P peers' packed index streams in one launch.
 
@@ -970,6 +995,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

@@ -1038,6 +1038,37 @@ __global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int
     flush_totals(t_cur);
 }
 
+// De-quantise one peer's flat payload of 8-bit codes: value = lookup[t][code] + shift[t], the
+// tensor t found from the row id (TopKCompressor._dequantize_values, src/tplr/compress.py:637-643,
+// for every parameter of the set at once).  Four codes per thread.
+__global__ __launch_bounds__(256) void k_dequantize_batch(const uint8_t* __restrict__ q,
+                                                          const float* __restrict__ lookup,
+                                                          const float* __restrict__ shift, int n_bins, int k,
+                                                          const tplr_tensor_desc* __restrict__ table, int n_tensors,
+                                                          int64_t n4, float* __restrict__ val) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n4; i += stride) {
+        const int64_t row = (i * 4) / k;  // k is a multiple of 4 here: the four codes share a row
+        int lo = 0, hi = n_tensors;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (table[mid].chunk_begin <= row)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        const uchar4 c = reinterpret_cast<const uchar4*>(q)[i];
+        const float* lk = lookup + static_cast<int64_t>(lo) * n_bins;
+        const float sh = shift[lo];
+        float4 o;
+        o.x = lk[c.x < n_bins ? c.x : n_bins - 1] + sh;
+        o.y = lk[c.y < n_bins ? c.y : n_bins - 1] + sh;
+        o.z = lk[c.z < n_bins ? c.z : n_bins - 1] + sh;
+        o.w = lk[c.w < n_bins ? c.w : n_bins - 1] + sh;
+        reinterpret_cast<float4*>(val)[i] = o;
+    }
+}
+
 // generic rows (1-D tensors, un-chunked 2-D rows): exact source-order accumulation
 __global__ __launch_bounds__(64) void k_scatter_rows(const uint8_t* __restrict__ idx12,
                                                      const int64_t* __restrict__ idx64,
@@ -1633,6 +1664,22 @@ int tplr_index_stats_batch(const uint8_t* const* h_idx12, int n_peers, int k, co
     hipLaunchKernelGGL(k_index_stats, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
                        static_cast<hipStream_t>(stream), ip, n_peers, k, d_desc, none, n_tensors, total_rows,
                        reinterpret_cast<unsigned long long*>(d_pair), reinterpret_cast<unsigned long long*>(d_dup), d_max);
+    return launch_status();
+}
+
+int tplr_dequantize_batch(const uint8_t* d_codes, const float* d_lookup, const float* d_shift, int n_bins, int k,
+                          const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_rows, float* d_val,
+                          void* stream) {
+    if (!d_codes || !d_lookup || !d_shift || !d_desc || !d_val || n_bins < 1 || n_bins > 256 || k < 4 || (k & 3) ||
+        n_tensors < 1 || total_rows < 0)
+        return TPLR_E_BADARG;
+    if ((reinterpret_cast<uintptr_t>(d_codes) & 3) || (reinterpret_cast<uintptr_t>(d_val) & 15)) return TPLR_E_BADARG;
+    if (total_rows == 0) return 0;
+    const int64_t n4 = total_rows * k / 4;
+    const int64_t blocks = (n4 + 255) / 256;
+    hipLaunchKernelGGL(k_dequantize_batch, dim3(static_cast<unsigned>(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), d_codes, d_lookup, d_shift, n_bins, k, d_desc, n_tensors, n4,
+                       d_val);
     return launch_status();
 }
 

@@ -606,3 +606,25 @@ def test_index_stats_match_reference_overlap(dev):
     assert pair[0].cpu().tolist() == [[0, 2, 4], [0, 0, 2], [0, 0, 0]] and top[0].cpu().tolist() == [3, 5, 3]
     assert orc.index_bounds(np.array([0, 1, 2, 3]), 64) is None
 
+
+def test_dequantize_batch_matches_per_parameter_reference_path(dev):
+    rng = np.random.default_rng(31)
+    shapes = [(128, 64), (64, 192), (192, 128)]
+    k = 32
+    batch = tc.TensorBatch([torch.zeros(s, device=dev) for s in shapes])
+    for bins in (4, 256):
+        comp = tc.TopKCompressor(use_quantization=True, quantization_bins=bins, quantization_range=6)
+        codes, qps, want = [], [], []
+        for i, s in enumerate(shapes):
+            y, x = s[0] // 64, s[1] // 64
+            v = torch.from_numpy(rng.standard_normal((y, x, k)).astype(np.float32) * (i + 1) + i).to(dev)
+            q, qp = comp._quantize_values(v)
+            codes.append(q.reshape(-1))
+            qps.append(qp)
+            # the reference's arithmetic on the oracle side: lookup[code] + shift
+            want.append(orc.dequantize(q.cpu().numpy(), (float(qp[0]), qp[1], qp[2], qp[3].cpu().numpy())))
+            assert torch.equal(comp._dequantize_values(q, qp).cpu(), torch.from_numpy(want[-1]))
+        got = tc.dequantize_batch(batch, torch.cat(codes), qps, k)
+        assert got.shape == (batch.total_chunks, k)
+        assert np.array_equal(got.cpu().numpy().reshape(-1), np.concatenate([w.reshape(-1) for w in want]))
+
