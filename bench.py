@@ -267,10 +267,15 @@ def main():
     def aggregate_kernel_only():
         tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, scale=scale, use_dct=True)
 
+    # the reference's per-parameter form of the same payloads (lists of P tensors per parameter)
+    per_param = []
+    for i in range(len(out_batch)):
+        sl = [out_batch.payload_slice(i, idxs[p], vals[p], k) for p in range(P)]
+        per_param.append(([a for a, _ in sl], [b for _, b in sl], out_batch.xshape(i)))
+
     def aggregate_per_tensor():
-        for i in range(len(out_batch)):
-            sl = [out_batch.payload_slice(i, idxs[p], vals[p], k) for p in range(P)]
-            tc.batch_decompress_decode([a for a, _ in sl], [b for _, b in sl], out_batch.xshape(i), out=outs[i])
+        for i, (pi, pv, xs) in enumerate(per_param):
+            tc.batch_decompress_decode(pi, pv, xs, out=outs[i])
 
     if args.profile == "aggregate":
         event_ms(aggregate_pass, args.steps, args.warmup)

@@ -167,9 +167,11 @@ int tplr_scatter_rows(const uint8_t* d_idx12, const int64_t* d_idx64, const floa
                       float* d_out, int32_t* d_err, void* stream);
 
 /* ---- peer statistics (src/tplr/compress.py:526-535, :553-556) ---------------------
- * d_sumsq[p] = sum of squares of payload p's n values (h_val: HOST array of n_peers
- * DEVICE pointers). */
-int tplr_peer_sumsq(const float* const* h_val, int n_peers, int64_t n, float* d_sumsq, void* stream);
+ * d_sumsq[p * n_slices + s] = sum of squares of the s-th of n_slices equal runs of payload p's
+ * n values (h_val: HOST array of n_peers DEVICE pointers).  n_slices > 1 lets a few peers with
+ * large payloads use the whole device; the consumer adds the partial sums in order. */
+int tplr_peer_sumsq(const float* const* h_val, int n_peers, int64_t n, int n_slices, float* d_sumsq,
+                    void* stream);
 
 /* d_scale[p] = min(1, med / (norm_p + 1e-8)), med = lower median of the norms
  * (torch.median).  n_partials == 0: d_norm[p] is the norm itself; n_partials >= 1: d_norm holds

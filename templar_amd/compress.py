@@ -413,12 +413,14 @@ def _peer_scales(vals: Sequence[torch.Tensor], block_norms: torch.Tensor | None,
             st = lib.tplr_clip_scales(_ptr(norms), P, 0, _ptr(scale), None, _stream(dev))
         else:
             ptrs = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
-            ss = torch.empty(P, dtype=torch.float32, device=dev)
             n = vals[0].numel()
             if any(v.numel() != n for v in vals):
                 raise ValueError("batch_decompress: all peers must send the same number of values")
-            _lib.check(lib.tplr_peer_sumsq(ptrs, P, n, _ptr(ss), _stream(dev)), "tplr_peer_sumsq")
-            st = lib.tplr_clip_scales(_ptr(ss), P, 1, _ptr(scale), None, _stream(dev))
+            # about 32 K values per block, so that one large tensor still spreads over the device
+            slices = max(1, min(256, n // 32768))
+            ss = torch.empty((P, slices), dtype=torch.float32, device=dev)
+            _lib.check(lib.tplr_peer_sumsq(ptrs, P, n, slices, _ptr(ss), _stream(dev)), "tplr_peer_sumsq")
+            st = lib.tplr_clip_scales(_ptr(ss), P, slices, _ptr(scale), None, _stream(dev))
     _lib.check(st, "tplr_clip_scales")
     return scale
 

@@ -1133,19 +1133,32 @@ struct ValPtrs {
     const float* val[TPLR_MAX_PEERS];
 };
 
-__global__ __launch_bounds__(1024) void k_peer_sumsq(const ValPtrs vp, int64_t n, float* __restrict__ sumsq) {
+// Sum of squares of n values per peer in S slices: block (p, s) reduces the s-th of S equal runs
+// and writes sumsq[p * S + s]; the consumer adds a peer's partial sums in order.  Eight
+// independent accumulators per thread; the reduction order is fixed.
+__global__ __launch_bounds__(1024) void k_peer_sumsq(const ValPtrs vp, int64_t n, int S, float* __restrict__ sumsq) {
     __shared__ float part[16];
-    const int p = blockIdx.x;
+    const int p = blockIdx.x / S, sl = blockIdx.x - p * S;
+    const int64_t i0 = n * sl / S, i1 = n * (sl + 1) / S;
     const float* v = vp.val[p];
-    float s = 0.f;
-    for (int64_t i = threadIdx.x; i < n; i += 1024) s = __builtin_fmaf(v[i], v[i], s);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    int64_t i = i0 + threadIdx.x;
+    for (; i + 7 * 1024 < i1; i += 8 * 1024) {
+        float x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = v[i + u * 1024];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc[u] = __builtin_fmaf(x[u], x[u], acc[u]);
+    }
+    for (; i < i1; i += 1024) acc[0] = __builtin_fmaf(v[i], v[i], acc[0]);
+    float s = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
     s = wave_sum_f32(s);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
     __syncthreads();
     if (threadIdx.x == 0) {
         float t = 0.f;
-        for (int i = 0; i < 16; ++i) t += part[i];
-        sumsq[p] = t;
+        for (int w = 0; w < 16; ++w) t += part[w];
+        sumsq[blockIdx.x] = t;
     }
 }
 
@@ -1601,16 +1614,16 @@ int tplr_scatter_rows(const uint8_t* d_idx12, const int64_t* d_idx64, const floa
     return launch_status();
 }
 
-int tplr_peer_sumsq(const float* const* h_val, int n_peers, int64_t n, float* d_sumsq, void* stream) {
-    if (!h_val || !d_sumsq || n_peers < 1 || n < 0) return TPLR_E_BADARG;
+int tplr_peer_sumsq(const float* const* h_val, int n_peers, int64_t n, int n_slices, float* d_sumsq, void* stream) {
+    if (!h_val || !d_sumsq || n_peers < 1 || n < 0 || n_slices < 1 || n_slices > 4096) return TPLR_E_BADARG;
     if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
     ValPtrs vp;
     for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
         vp.val[p] = p < n_peers ? h_val[p] : nullptr;
         if (p < n_peers && !vp.val[p] && n > 0) return TPLR_E_BADARG;
     }
-    hipLaunchKernelGGL(k_peer_sumsq, dim3(n_peers), dim3(1024), 0, static_cast<hipStream_t>(stream), vp, n,
-                       d_sumsq);
+    hipLaunchKernelGGL(k_peer_sumsq, dim3(static_cast<unsigned>(n_peers) * n_slices), dim3(1024), 0,
+                       static_cast<hipStream_t>(stream), vp, n, n_slices, d_sumsq);
     return launch_status();
 }
 

@@ -396,9 +396,17 @@ def test_clip_scales_and_norms(dev):
     vals = [torch.randn(1000 + 0 * p, device=dev) * (p + 1) for p in range(5)]
     ss = torch.empty(5, device=dev)
     ptrs = (C.c_void_p * 5)(*[v.data_ptr() for v in vals])
-    assert lib.tplr_peer_sumsq(ptrs, 5, 1000, tc._ptr(ss), None) == 0
+    assert lib.tplr_peer_sumsq(ptrs, 5, 1000, 1, tc._ptr(ss), None) == 0
     want = np.array([float((v.double() ** 2).sum()) for v in vals])
     assert np.allclose(ss.cpu().numpy(), want, rtol=1e-5)
+    # in slices (ragged: 1000 values in 7 runs), and the clip factors from the partial sums
+    ss7 = torch.empty((5, 7), device=dev)
+    assert lib.tplr_peer_sumsq(ptrs, 5, 1000, 7, tc._ptr(ss7), None) == 0
+    assert np.allclose(ss7.sum(dim=1).cpu().numpy(), want, rtol=1e-5)
+    sc = torch.empty(5, device=dev)
+    assert lib.tplr_clip_scales(tc._ptr(ss7), 5, 7, tc._ptr(sc), None, None) == 0
+    _, want_sc = orc.clip_scales(np.sqrt(want).astype(np.float32))
+    assert np.allclose(sc.cpu().numpy(), want_sc, rtol=2e-6)
 
 
 def test_bad_arguments_are_rejected(dev):
