@@ -4,8 +4,7 @@
 // in registers (64 floats per lane: lane = row or column, register index = the other
 // coordinate) or in an LDS tile with a row stride of 68 floats, which makes both the
 // row-per-lane 16-byte accesses and the column-per-lane 4-byte accesses bank-conflict
-// free.  The 4 padding floats of every tile row double as 128 eight-byte slots for the
-// top-k candidate list.
+// free.  The decode kernel uses the 4 padding floats of a tile row as per-lane scratch slots.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -95,12 +94,6 @@ __device__ __forceinline__ void tile_rows_to_regs(float (&v)[64], const float* t
         v[4 * c + 2] = t.z;
         v[4 * c + 3] = t.w;
     }
-}
-
-// registers (lane = column, register = row) <-> tile
-__device__ __forceinline__ void regs_to_tile_cols(const float (&v)[64], float* tile, int lane) {
-#pragma unroll
-    for (int r = 0; r < 64; ++r) tile[r * kLd + lane] = v[r];
 }
 
 __device__ __forceinline__ void tile_cols_to_regs(float (&v)[64], const float* tile, int lane) {

@@ -836,9 +836,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         return;
     }
 
-    // The loop is software-pipelined over three chunks.  While chunk g is in registers for the
-    // second pass of its inverse transform (vector ALU only), the tile already receives the
-    // scatter of chunk g + 1, and the payload of chunk g + 2 is on its way from memory.
+    // The other variants (coefficient output, generic peer count or k, per-chunk normalisation):
+    // a plain three-chunk pipeline.  Chunk g leaves the tile for registers, chunk g + 1 is
+    // scattered into the tile, the payload of chunk g + 2 is requested (fast path only).
     Cursor c;
     cursor_seek(c, table, single, n_tensors, g0);
     Out out_cur = out_of(c, g0), out_next = out_cur;
