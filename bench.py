@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the gradient-codec hot path on one MI355X.
 
-Workload (BASELINE.json configs[2] and configs[3]): the LLaMA-style 1B gradient set
+Workload (benchmark configurations 3 and 4): the LLaMA-style 1B gradient set
 (16 layers, hidden 2048, intermediate 8192, vocab 32000; 115 two-dimensional tensors =
 294 144 chunks of 64x64, plus 33 norm vectors), synthetic Student-t(df=3) x 1e-3 gradients
 with log-normal row scales, chunk 64, top-k 32.

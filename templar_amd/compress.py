@@ -990,7 +990,7 @@ def overlap_fractions(pair: torch.Tensor, rows: Sequence[int], k: int) -> torch.
     return pair.sum(dim=0).double() / total
 
 
-# the names BASELINE.json's north star uses (DeMo-era)
+# the DeMo-era names of the two classes
 TransformDCT = ChunkingTransformer
 CompressDCT = TopKCompressor
 

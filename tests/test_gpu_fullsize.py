@@ -1,4 +1,4 @@
-"""Full-size checks on the GPU: the 1B gradient set (294 144 chunks, BASELINE.json configs 3 and 4)
+"""Full-size checks on the GPU: the 1B gradient set (294 144 chunks, benchmark configurations 3 and 4)
 and the 72B block (config 5, k = 64) through the batch entry points of the C ABI.
 
 The CPU oracle cannot cover these sizes in test time, so the checks are properties that do not

@@ -1,4 +1,4 @@
-"""Synthetic gradient sets of BASELINE.json's configs (shared by bench.py and the tests).
+"""Synthetic gradient sets of the five benchmark configurations (shared by bench.py and the tests).
 
 Value law: Student-t(df=3) built as z0 / sqrt((z1^2 + z2^2 + z3^2) / 3) from four
 independent normal draws, times 1e-3; configs 2-5 multiply every row by exp(0.5 n_r),
