@@ -135,8 +135,10 @@ int tplr_encode_topk_pack_batch(const tplr_tensor_desc* d_desc, int n_tensors, i
  * per-chunk L2 norm + 1e-8 (:541-545); accumulate in peer order; divide every touched
  * coefficient by its number of contributions (scatter_reduce "mean",
  * include_self=False, :472-474) unless reduce_mode = TPLR_REDUCE_SUM; then apply the
- * inverse DCT (use_dct != 0, output (R, C) row stride ld_out) or write the dense
- * coefficients as (R/64, C/64, 64, 64) (use_dct == 0, ld_out ignored).
+ * inverse DCT (use_dct != 0, output (R, C) with row stride ld_out >= C); without it
+ * (use_dct == 0) write either the dense coefficient tensor (R/64, C/64, 64, 64) (ld_out == 0:
+ * what batch_decompress returns) or the (R, C) tensor with row stride ld_out >= C (what
+ * decode(use_dct=False) makes of it, a pure re-layout, :281).
  * h_idx12 / h_val are HOST arrays of n_peers DEVICE pointers: payload p holds
  * n_chunks*k*3/2 index bytes and (n_chunks, k) values.  d_sumsq (nullable) receives
  * n_chunks partial sums of squares of the output, one per chunk. */
@@ -147,8 +149,9 @@ int tplr_decode_aggregate(const uint8_t* const* h_idx12, const float* const* h_v
 
 /* The same over a whole gradient set in ONE launch (the per-parameter loop of
  * src/tplr/neurons.py:309-367): every peer's payload is flat over the batch
- * (tplr_tensor_desc), results go to each descriptor's `dense` tensor ((R, C) with stride ld
- * when use_dct != 0, contiguous (R/64, C/64, 64, 64) otherwise); d_scale (nullable) holds
+ * (tplr_tensor_desc), results go to each descriptor's `dense` tensor ((R, C) with row stride
+ * ld; with use_dct == 0 a descriptor with ld == 0 receives the contiguous (R/64, C/64, 64, 64)
+ * coefficient tensor instead); d_scale (nullable) holds
  * n_tensors x n_peers clip factors, d_sumsq (nullable) total_chunks partial sums. */
 int tplr_decode_aggregate_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale,
                                 int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,

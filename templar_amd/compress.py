@@ -427,8 +427,10 @@ def _peer_scales(vals: Sequence[torch.Tensor], block_norms: torch.Tensor | None,
 
 def _aggregate_chunks(idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], scale: torch.Tensor | None,
                       Y: int, X: int, k: int, *, normalise: bool, use_dct: bool, mean: bool = True,
-                      out: torch.Tensor | None = None, sumsq: torch.Tensor | None = None) -> torch.Tensor:
-    """Fused unpack + scatter over peers (+ inverse DCT) on 64x64 chunks."""
+                      out: torch.Tensor | None = None, sumsq: torch.Tensor | None = None,
+                      rows: bool = False) -> torch.Tensor:
+    """Fused unpack + scatter over peers (+ inverse DCT) on 64x64 chunks.  Without the transform
+    the result is the dense coefficient tensor (Y, X, 64, 64), or with `rows` the (R, C) tensor."""
     lib = _lib.load()
     P = len(vals)
     dev = vals[0].device
@@ -443,13 +445,14 @@ def _aggregate_chunks(idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor]
     ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
     vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
     R, Cc = Y * _CH, X * _CH
+    as_rows = use_dct or rows
     if out is None:
-        out = torch.empty((R, Cc) if use_dct else (Y, X, _CH, _CH), dtype=torch.float32, device=dev)
+        out = torch.empty((R, Cc) if as_rows else (Y, X, _CH, _CH), dtype=torch.float32, device=dev)
     if n_chunks:
         with torch.cuda.device(dev):
             st = lib.tplr_decode_aggregate(ip, vp, _ptr(scale), P, k, R, Cc,
                                            _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM, int(normalise), int(use_dct),
-                                           _ptr(out), out.stride(0) if use_dct else 0, _ptr(sumsq), _stream(dev))
+                                           _ptr(out), out.stride(0) if as_rows else 0, _ptr(sumsq), _stream(dev))
         _lib.check(st, "tplr_decode_aggregate")
     return out
 
@@ -500,9 +503,8 @@ class LazyAggregate:
 
     def decode(self, *, use_dct: bool) -> torch.Tensor:
         Y, X = self.shape[0], self.shape[1]
-        if not use_dct:
-            return self.dense().permute(0, 2, 1, 3).reshape(Y * _CH, X * _CH)
-        out = _aggregate_chunks(self.idxs, self.vals, self.scale, Y, X, self.k, normalise=self.normalise, use_dct=True)
+        out = _aggregate_chunks(self.idxs, self.vals, self.scale, Y, X, self.k, normalise=self.normalise,
+                                use_dct=use_dct, rows=True)
         return out if self.dtype == torch.float32 else out.to(self.dtype)
 
 
@@ -739,7 +741,7 @@ def batch_decompress_decode(idxs: Sequence[torch.Tensor], vals: Sequence[torch.T
     if clip_norm and not normalise:
         scale = _peer_scales(vals, block_norms, dev)
     return _aggregate_chunks(idxs, vals, scale, xshape[0], xshape[1], vals[0].shape[-1], normalise=normalise,
-                             use_dct=use_dct, mean=mean, out=out, sumsq=sumsq)
+                             use_dct=use_dct, mean=mean, out=out, sumsq=sumsq, rows=True)
 
 
 # ----------------------------------------------------------------------------------------

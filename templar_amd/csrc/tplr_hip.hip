@@ -652,13 +652,16 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     };
 
     // where a chunk's result goes
+    // Without the transform the result is either the dense coefficient tensor (R/64, C/64, 64, 64)
+    // (row stride 0 in the descriptor) or, with a row stride, the (R, C) tensor itself: decode
+    // without a transform is a pure re-layout (src/tplr/compress.py:281).
     struct Out {
         gfloat* chunk0;
         int64_t ld;
     };
     auto out_of = [&](const Cursor& cu, int64_t g) -> Out {
-        return Out{kUseDct ? cu.base + (cu.y * 64) * cu.ld + static_cast<int64_t>(cu.xc) * 64
-                           : cu.base + (g - cu.begin) * 4096,
+        return Out{(kUseDct || cu.ld > 0) ? cu.base + (cu.y * 64) * cu.ld + static_cast<int64_t>(cu.xc) * 64
+                                          : cu.base + (g - cu.begin) * 4096,
                    cu.ld};
     };
 
@@ -863,6 +866,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             regs_to_tile_rows(v, tile, lane);
             wave_lds_fence();
             tile_cols_to_regs(v, tile, lane);
+        } else if (out_cur.ld > 0) {  // wave-uniform
+            tile_cols_to_regs(v, tile, lane);
         } else {
 #pragma unroll
             for (int q0 = 0; q0 < 16; ++q0) {
@@ -900,7 +905,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         // (the loop-carried destination may have been parked in vector registers: make it scalar
         // again, or every store becomes a loop over distinct descriptors)
         gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0));
-        if (kUseDct) {
+        if (kUseDct || out_cur.ld > 0) {
             store_chunk_rows(v, (void*)dst, uniform64(out_cur.ld), lane);
         } else {
 #pragma unroll
@@ -1573,10 +1578,10 @@ int tplr_decode_aggregate(const uint8_t* const* h_idx12, const float* const* h_v
     if (int s = check_decode(h_idx12, h_val, n_peers, k, reduce_mode)) return s;
     if (!d_out || R < 0 || C < 0) return TPLR_E_BADARG;
     if ((R % 64) || (C % 64)) return TPLR_E_SHAPE;
-    if (use_dct && ld_out < C) return TPLR_E_BADARG;
+    if ((use_dct || ld_out != 0) && ld_out < C) return TPLR_E_BADARG;
     const int64_t n = (R / 64) * (C / 64);
     if (n == 0) return 0;
-    if (C / 64 > 0x7fffffff || R / 64 > 0x7fffffff || (use_dct && !ld_ok(ld_out))) return TPLR_E_TOOMANY;
+    if (C / 64 > 0x7fffffff || R / 64 > 0x7fffffff || (ld_out != 0 && !ld_ok(ld_out))) return TPLR_E_TOOMANY;
     tplr_tensor_desc single;
     single.dense = d_out;
     single.ld = ld_out;

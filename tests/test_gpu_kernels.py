@@ -636,3 +636,38 @@ def test_dequantize_batch_matches_per_parameter_reference_path(dev):
         assert got.shape == (batch.total_chunks, k)
         assert np.array_equal(got.cpu().numpy().reshape(-1), np.concatenate([w.reshape(-1) for w in want]))
 
+
+def test_aggregate_without_transform_writes_the_gradient_layout(dev):
+    # use_dct=False (templar's default hparams): batch_decompress + decode is scatter-mean + re-layout
+    P, k, Y, X = 20, 64, 3, 5
+    idxs, vals = make_peers(P, Y, X, k, 77)
+    norms = np.array([orc.norm2(v) for v in vals], np.float32)
+    dense = orc.batch_decompress(idxs, vals, (Y, X, 64, 64), 4096, block_norms=norms)
+    want = orc.decode2d(dense, use_dct=False)
+    di = [torch.from_numpy(i).to(dev) for i in idxs]
+    dv = [torch.from_numpy(v).to(dev) for v in vals]
+    bn = torch.from_numpy(norms).to(dev)
+    got = tc.batch_decompress_decode(di, dv, (Y, X, 64, 64), block_norms=bn, use_dct=False)
+    assert got.shape == (Y * 64, X * 64)
+    assert np.array_equal(got.cpu().numpy(), want)
+    # through the reference-shaped calls: deferred scatter, then decode
+    comp, tr = tc.TopKCompressor(), tc.ChunkingTransformer(_Stub([torch.empty(Y * 64, X * 64)]), 64)
+    lazy = comp.batch_decompress(torch.empty(1, device=dev), di, dv, (Y, X, 64, 64), 4096, block_norms=bn, defer=True)
+    assert torch.equal(tr.decode(lazy, use_dct=False), got)
+    eager = comp.batch_decompress(torch.empty(1, device=dev), di, dv, (Y, X, 64, 64), 4096, block_norms=bn)
+    assert np.array_equal(eager.cpu().numpy(), dense)
+    assert torch.equal(tr.decode(eager, use_dct=False), got)
+    # into a view with a row stride, and the batch form with row-major descriptors
+    wide = torch.full((Y * 64, X * 64 + 128), -1.0, device=dev)
+    tc.batch_decompress_decode(di, dv, (Y, X, 64, 64), block_norms=bn, use_dct=False, out=wide[:, 64:64 + X * 64])
+    assert torch.equal(wide[:, 64:64 + X * 64], got) and float(wide[:, :64].max()) == -1.0
+    outb = torch.empty(Y * 64, X * 64, device=dev)
+    flat_i = [i.reshape(-1) for i in di]
+    flat_v = [v.reshape(-1, k) for v in dv]
+    scale = tc._peer_scales(dv, bn, dev).reshape(1, P)  # the same clip factors as above
+    tc.batch_decompress_decode_batch(tc.TensorBatch([outb]), flat_i, flat_v, k, scale=scale, use_dct=False)
+    assert torch.equal(outb, got)
+    # its own norms (partial sums added in another order) agree to rounding
+    tc.batch_decompress_decode_batch(tc.TensorBatch([outb]), flat_i, flat_v, k, use_dct=False)
+    assert float((outb - got).abs().max()) <= 1e-6 * float(got.abs().max())
+
