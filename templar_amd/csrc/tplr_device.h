@@ -330,14 +330,18 @@ __device__ __forceinline__ void sort128_desc(uint64_t& e0, uint64_t& e1, int) { 
 // `out_scale` multiplies the gathered values (an exact power of two left over by the caller's
 // transform; the ordering is taken on the unscaled values).
 // `buf` is a kHalfFloats staging buffer, `cand` kCandCap slots; both are free on return.
+// `t_floor` (magnitude bits, wave-uniform, 0 = none) is another lower bound of the k-th largest
+// magnitude that the caller knows, e.g. the same statistic taken over the columns: data whose
+// rows differ in scale put most candidates into a few lanes and pass far too many of them.
 template <bool kTwo>
 __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf, uint64_t* cand, int lane, int k,
-                                                float out_scale) {
+                                                float out_scale, uint32_t t_floor = 0) {
     uint32_t mhi = 0, mlo = 0, cnt = 0, incl = 0, total = 0;
     {
         uint32_t b1, b2;
         lane_stats<kTwo>(w, b1, b2);
-        const uint32_t t0 = stat_threshold<kTwo>(b1, b2, k);
+        const uint32_t t_rows = stat_threshold<kTwo>(b1, b2, k);
+        const uint32_t t0 = t_rows > t_floor ? t_rows : t_floor;
         filter_masks(w, __uint_as_float(t0), mhi, mlo);
         cnt = __popc(mhi) + __popc(mlo);
         incl = wave_incl_scan_u32(cnt);

@@ -431,8 +431,17 @@ __global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_de
             if (g + 1 < g1) cursor_next(cg, g + 1);
         }
         if (g + 1 < g1) cursor_next(c, g + 1);
+        // Untransformed gradients often differ in scale from row to row or column to column;
+        // the select's threshold statistic is then taken in both directions.  (Coefficients of
+        // the transform are mixed across both and one direction is as good as two.)
+        uint32_t t_cols = 0;
+        if (!kUseDct) {
+            uint32_t c1, c2;
+            lane_stats<kTwo>(v, c1, c2);
+            t_cols = stat_threshold<kTwo>(c1, c2, k);
+        }
         chunk_forward<kUseDct>(v, w, buf, lane);
-        const Selected s = select_topk<kTwo>(w, buf, cand, lane, k, kUseDct ? kDctPow2Scale : 1.0f);
+        const Selected s = select_topk<kTwo>(w, buf, cand, lane, k, kUseDct ? kDctPow2Scale : 1.0f, t_cols);
         emit_selected(s, lane, k, g, idx12, val);
     }
 }
