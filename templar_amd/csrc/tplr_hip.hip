@@ -467,16 +467,27 @@ __device__ __forceinline__ uint32_t load_idx12(BytePtr row, int j) {
 typedef uint16_t __attribute__((aligned(1))) unaligned_u16;
 using gu16 = __attribute__((address_space(1))) unaligned_u16;
 
-// Contribution counters, one per coefficient, packed into 32-bit words that LDS atomics update:
-// 4 bits each when at most 15 peers can hit a coefficient (2 KB, so that 8 waves fit the 160 KB
-// of a CU), 8 bits otherwise (4 KB, 7 waves).
+// Contribution counters, one per coefficient, packed into 32-bit words that LDS atomics update,
+// every tile row in words of its own: 4 bits each when at most 15 peers can hit a coefficient
+// (8 words per row, 2 KB), 5 bits up to 31 peers (6 per word, 11 words per row, 2.75 KB) - both
+// leave room for 8 waves in the 160 KB of a CU - and 8 bits beyond (4 KB, 7 waves).
 template <int kBits>
 struct Counters {
     static constexpr int kPerWord = 32 / kBits;
-    static constexpr int kWords = 4096 / kPerWord;
+    static constexpr int kRowWords = (kChunk + kPerWord - 1) / kPerWord;
+    static constexpr int kWords = kChunk * kRowWords;
+    static constexpr int kAlloc = (kWords + 255) / 256 * 256;  // cleared 16 bytes per lane at a time
     static constexpr uint32_t kMask = (1u << kBits) - 1u;
-    __device__ static __forceinline__ uint32_t word(uint32_t e) { return e / kPerWord; }
-    __device__ static __forceinline__ uint32_t shift(uint32_t e) { return (e % kPerWord) * kBits; }
+    // bits 1 .. kBits-1 of every field: set somewhere <=> that counter is at least 2
+    static constexpr uint32_t kMulti = kBits == 4 ? 0xEEEEEEEEu : kBits == 5 ? 0x3DEF7BDEu : 0xFEFEFEFEu;
+    __device__ static __forceinline__ uint32_t word(uint32_t e) {
+        const uint32_t col = e & 63u;
+        return (e >> 6) * kRowWords + (kBits == 5 ? (col * 43u) >> 8 : col / kPerWord);
+    }
+    __device__ static __forceinline__ uint32_t shift(uint32_t e) {
+        const uint32_t col = e & 63u;
+        return (kBits == 5 ? col - ((col * 43u) >> 8) * 6u : col % kPerWord) * kBits;
+    }
 };
 
 // Persistent fused decode.  Per chunk, the peers' entries are accumulated in peer order into an
@@ -499,7 +510,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                                                             float* __restrict__ sumsq) {
     __shared__ __align__(16) float tile[kTileFloats];
     using Cnt = Counters<kCntBits>;
-    __shared__ __align__(16) uint32_t cnt[Cnt::kWords];
+    __shared__ __align__(16) uint32_t cnt[Cnt::kAlloc];
     constexpr bool kFast = kUnits > 0;
     constexpr int kRegs = kFast ? kUnits : 1;
     const int lane = threadIdx.x;
@@ -568,7 +579,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         for (int q = 0; q < 16; ++q) row[q] = z;
         const uint4 zi = make_uint4(0, 0, 0, 0);
 #pragma unroll
-        for (int q = 0; q < Cnt::kWords / 256; ++q) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
+        for (int q = 0; q < Cnt::kAlloc / 256; ++q) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
         wave_lds_fence();
     };
 
@@ -630,18 +641,12 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     auto mean_pass = [&]() {
         wave_lds_fence();
         if (reduce_mode != TPLR_REDUCE_MEAN) return;
-        constexpr int kRowWords = kChunk / Cnt::kPerWord;
-        constexpr uint32_t kMulti = kCntBits == 4 ? 0xEEEEEEEEu : 0xFEFEFEFEu;  // count >= 2
+        constexpr int kRowWords = Cnt::kRowWords;
+        constexpr uint32_t kMulti = Cnt::kMulti;
         const uint32_t* crow = cnt + lane * kRowWords;
         uint32_t todo = 0;  // bit q: word q of the row holds such a counter
 #pragma unroll
-        for (int q4 = 0; q4 < kRowWords / 4; ++q4) {
-            const uint4 t = reinterpret_cast<const uint4*>(crow)[q4];
-            todo |= ((t.x & kMulti) ? 1u : 0u) << (4 * q4);
-            todo |= ((t.y & kMulti) ? 2u : 0u) << (4 * q4);
-            todo |= ((t.z & kMulti) ? 4u : 0u) << (4 * q4);
-            todo |= ((t.w & kMulti) ? 8u : 0u) << (4 * q4);
-        }
+        for (int q = 0; q < kRowWords; ++q) todo |= ((crow[q] & kMulti) ? 1u : 0u) << q;
         uint32_t word = 0, m = 0;
         int q = 0;
         while (todo | m) {
@@ -1551,7 +1556,7 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
         pp.val[p] = p < n_peers ? h_val[p] : nullptr;
         if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
     }
-    // register-resident fast path: k <= 64 and at most 24 peers; 4-bit counters up to 15 peers
+    // register-resident fast path: k <= 64 and at most 24 peers; 4-bit counters up to 15 peers, 5-bit beyond
     const int units = (k > 64 || normalise) ? 0 : n_peers <= 8 ? 8 : n_peers <= 15 ? 16 : n_peers <= 24 ? 24 : 0;
 #define TPLR_DECODE_CASE(U, BITS)                                                                                   \
     case U:                                                                                                         \
@@ -1562,7 +1567,7 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
     switch (units) {
         TPLR_DECODE_CASE(8, 4)
         TPLR_DECODE_CASE(16, 4)
-        TPLR_DECODE_CASE(24, 8)
+        TPLR_DECODE_CASE(24, 5)
         default:
             break;
     }

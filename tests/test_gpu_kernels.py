@@ -327,7 +327,7 @@ def test_aggregate_normalise(dev):
     assert np.array_equal(got.cpu().numpy() != 0, want != 0)
 
 
-@pytest.mark.parametrize("P,k", [(1, 32), (15, 32), (15, 64)])
+@pytest.mark.parametrize("P,k", [(1, 32), (15, 32), (15, 64), (20, 32), (24, 64), (31, 16)])
 def test_aggregate_fused_with_inverse_dct(dev, P, k):
     Y, X = 3, 2
     idxs, vals = make_peers(P, Y, X, k, 9 * P + k)
