@@ -913,6 +913,41 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
     return idx12, val, quant
 
 
+def check_compressed_indices(param_name: str, idxs, totalk: int, allowed_topk: int | None = None,
+                             vals: torch.Tensor | None = None, *, topk_compression: int | None = None) -> None:
+    """Validation of one parameter's packed indices as Comms.check_compressed_indices does it
+    (src/tplr/comms.py:2538-2610), with its error messages: uint8 tensor, values present,
+    non-empty, last dimension == min(allowed top-k, totalk), every index in [0, totalk).
+    `topk_compression` stands in for the reference's `self.hparams.topk_compression` when
+    `allowed_topk` is not given.  Works on host and device tensors; raises ValueError."""
+    if allowed_topk is None:
+        if topk_compression is None:
+            raise TypeError("check_compressed_indices needs allowed_topk or topk_compression")
+        allowed_topk = min(int(topk_compression), totalk)
+    else:
+        allowed_topk = min(allowed_topk, totalk)
+    if not isinstance(idxs, torch.Tensor):
+        raise ValueError(f"[{param_name}] Expected tensor but got {type(idxs)}")
+    if idxs.dtype != torch.uint8:
+        raise ValueError(f"[{param_name}] Expected uint8 for 12-bit packed indices, got {idxs.dtype}")
+    if vals is None:
+        raise ValueError(f"[{param_name}] Values tensor required to validate 12-bit packed indices")
+    if idxs.numel() == 0:
+        raise ValueError(f"[{param_name}] Empty packed indices tensor")
+    try:
+        unpacked = unpack_12bit_indices(idxs, vals.shape)
+        if unpacked.shape[-1] != allowed_topk:
+            raise ValueError(f"[{param_name}] Invalid topk dimension: "
+                             f"shape[-1]={unpacked.shape[-1]} but expected {allowed_topk}")
+        if unpacked.numel() == 0:
+            raise ValueError(f"[{param_name}] empty index list")
+        if unpacked.min().item() < 0 or unpacked.max().item() >= totalk:
+            bad = unpacked[(unpacked < 0) | (unpacked >= totalk)][0].item()
+            raise ValueError(f"[{param_name}] Index {bad} out of bounds (totalk = {totalk})")
+    except Exception as e:  # the reference wraps every failure the same way (:2607-2608)
+        raise ValueError(f"[{param_name}] Failed to unpack 12-bit indices: {e}")
+
+
 @torch.no_grad()
 def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[QuantParamsT], k: int,
                      out: torch.Tensor | None = None) -> torch.Tensor:
@@ -999,6 +1034,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

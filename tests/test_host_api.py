@@ -195,3 +195,43 @@ def test_quantiser_matches_oracle_and_reference_contract():
     assert torch.equal(c.maybe_dequantize_values([q], qp, torch.device("cpu"))[0], deq)  # a bare 5-tuple
     with pytest.raises(IndexError, match="Mismatch in val lengths"):
         c.maybe_dequantize_values([q, q], [qp, None], torch.device("cpu"))
+
+
+# ---------------------------------------------------------------- check_compressed_indices
+def test_check_compressed_indices_reference_cases():
+    """The cases of the reference's tests/test_comms.py:1828-2004 (hparams.topk_compression = 4),
+    on host tensors: same acceptances, same error messages."""
+    chk = lambda name, idxs, totalk, **kw: tc.check_compressed_indices(name, idxs, totalk, topk_compression=4, **kw)  # noqa: E731
+    pk = tc.pack_12bit_indices
+    v = lambda *shape: torch.randn(*shape)  # noqa: E731
+    # valid: flat and multi-dimensional
+    chk("test_param", pk(torch.tensor([1, 5, 9, 3])), 10, vals=v(4))
+    chk("param", pk(torch.tensor([[0, 1, 2, 3], [4, 5, 6, 7]])), 20, vals=v(2, 4))
+    # not packed / wrong dtype
+    for bad in (torch.tensor([0, 1, 2, 3], dtype=torch.long), torch.tensor([0, 1, 2, 3], dtype=torch.int32)):
+        with pytest.raises(ValueError, match="Expected uint8 for 12-bit packed indices"):
+            chk("param", bad, 20, vals=v(4))
+    # wrong top-k dimension, flat and multi-dimensional
+    with pytest.raises(ValueError, match="Invalid topk dimension"):
+        chk("param", pk(torch.tensor([0, 1])), 10, vals=v(2))
+    with pytest.raises(ValueError, match="Invalid topk dimension"):
+        chk("param", pk(torch.tensor([[0, 1, 2, 3, 4, 5], [6, 7, 8, 9, 10, 11]])), 20, vals=v(2, 6))
+    # out of bounds
+    with pytest.raises(ValueError, match="Index 10 out of bounds"):
+        chk("param", pk(torch.tensor([0, 1, 10, 3])), 10, vals=v(4))
+    # allowed_topk override
+    chk("param", pk(torch.tensor([0, 9])), 10, allowed_topk=2, vals=v(2))
+    with pytest.raises(ValueError, match="Invalid topk dimension"):
+        chk("param", pk(torch.tensor([0, 1, 2, 3])), 10, allowed_topk=2, vals=v(4))
+    # totalk below the configured top-k
+    chk("param", pk(torch.tensor([0, 1])), 2, vals=v(2))
+    with pytest.raises(ValueError, match="Invalid topk dimension"):
+        chk("param", pk(torch.tensor([0, 1, 0, 1])), 2, vals=v(4))
+    # the reference's other refusals
+    with pytest.raises(ValueError, match="Values tensor required"):
+        chk("param", pk(torch.tensor([0, 1])), 10)
+    with pytest.raises(ValueError, match="Empty packed indices tensor"):
+        chk("param", torch.empty(0, dtype=torch.uint8), 10, vals=v(0))
+    with pytest.raises(ValueError, match="Expected tensor but got"):
+        chk("param", [0, 1, 2, 3], 10, vals=v(4))
+
