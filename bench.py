@@ -38,8 +38,8 @@ HBM_PEAK_GBPS = 8000.0
 # x 2.000, WRITE_SIZE x 1.000).  The commands and raw figures are in the rocprofv3 summaries kept
 # with the sources.  Only the configuration they were measured on has an entry.
 MEASURED_TRAFFIC = {
-    ("cfg3_llama1b", 15, "encode"): 4_874_555_885,     # 1.001 x algorithmic
-    ("cfg3_llama1b", 15, "aggregate"): 6_068_057_220,  # 1.084 x: streaming loads re-fetch shared index lines
+    ("cfg3_llama1b", 15, "encode"): 4_874_549_190,     # 1.001 x algorithmic
+    ("cfg3_llama1b", 15, "aggregate"): 6_068_511_109,  # 1.084 x: streaming loads re-fetch shared index lines
 }
 
 
@@ -244,7 +244,7 @@ def main():
         enc2d_ms, _ = event_ms(encode2d_only, args.steps, 1)      # the fused 2-D kernel alone (dominant)
         enc_pt_ms, _ = event_ms(encode_per_tensor, max(3, args.steps // 2), 1)
     enc2d_bytes = n_chunks * (16384 + 11 * k // 2)
-    miner = miner_figures(max(3, args.steps // 2), 2) if k <= 64 else None
+    miner = miner_figures(max(3, args.steps // 2), 2) if k <= 64 and args.profile is None else None
 
     # ---- P peers' flat payloads for the aggregation side (peer p = 0.5 shared + own)
     idxs, vals = [], []
