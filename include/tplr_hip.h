@@ -77,6 +77,15 @@ int tplr_unpack12(const uint8_t* d_packed, int64_t n, int64_t* d_idx, void* stre
 int tplr_pack12_host(const int64_t* idx, int64_t n, uint8_t* packed, int64_t* bad);
 int tplr_unpack12_host(const uint8_t* packed, int64_t n, int64_t* idx);
 
+/* Concatenates n_parts HOST buffers (h_src[i], h_bytes[i] bytes) into h_dst with n_threads host
+ * threads (1..64), each copying an equal share of the bytes.  Turns one peer's per-parameter
+ * payload tensors (the lists `state_dict.<name>idxs` / `<name>vals` that
+ * src/tplr/comms.py:1938-1963 builds and neurons/validator.py:94-219 moves tensor by tensor)
+ * into the flat payload the batch entry points read, inside a pinned buffer that then crosses to
+ * the device in one copy.  Blocking; touches no device. */
+int tplr_gather_host(const void* const* h_src, const int64_t* h_bytes, int64_t n_parts, void* h_dst,
+                     int n_threads);
+
 /* ---- chunked 2-D DCT ------------------------------------------------------------
  * Replaces ChunkingTransformer.encode(use_dct=True) for 2-D tensors whose chunk is
  * 64x64 (src/tplr/compress.py:236-246, einsum :203): d_x is (R, C) row-major with

@@ -28,6 +28,7 @@ SIGNATURES = {
     "tplr_unpack12": (_i32, [_vp, _i64, _vp, _vp]),
     "tplr_pack12_host": (_i32, [_vp, _i64, _vp, _vp]),
     "tplr_unpack12_host": (_i32, [_vp, _i64, _vp]),
+    "tplr_gather_host": (_i32, [_vp, _vp, _i64, _vp, _i32]),
     "tplr_dct2d_fwd": (_i32, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "tplr_dct2d_inv": (_i32, [_vp, _i64, _i64, _vp, _i64, _vp]),
     "tplr_dct1d": (_i32, [_vp, _i64, _i32, _vp, _vp]),

@@ -23,6 +23,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+import os
 from typing import Sequence, TypeAlias
 
 import torch
@@ -948,6 +949,15 @@ def check_compressed_indices(param_name: str, idxs, totalk: int, allowed_topk: i
         raise ValueError(f"[{param_name}] Failed to unpack 12-bit indices: {e}")
 
 
+def _qparam_tables(qparams: Sequence[QuantParamsT], dev: torch.device) -> tuple[torch.Tensor, torch.Tensor, int]:
+    """(rows, n_bins) lookups and (rows,) shifts of a list of quant_params 5-tuples on `dev`: stacked
+    where they live, moved once."""
+    n_bins = int(qparams[0][3].numel())
+    lookup = torch.stack([qp[3].reshape(n_bins).float() for qp in qparams])
+    shift = torch.stack([torch.as_tensor(qp[0], dtype=torch.float32, device=lookup.device).reshape(()) for qp in qparams])
+    return lookup.to(dev).contiguous(), shift.to(dev).contiguous(), n_bins
+
+
 @torch.no_grad()
 def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[QuantParamsT], k: int,
                      out: torch.Tensor | None = None) -> torch.Tensor:
@@ -961,9 +971,7 @@ def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[
         raise IndexError(f"Mismatch in val lengths: dequant({len(qparams)}) vs original({len(batch)})")
     if codes.dtype != torch.uint8 or codes.numel() != n * k:
         raise RuntimeError(f"{codes.numel()} codes of {codes.dtype} for {n} chunks of k={k}")
-    n_bins = int(qparams[0][3].numel())
-    lookup = torch.stack([qp[3].to(dev, torch.float32).reshape(n_bins) for qp in qparams]).contiguous()
-    shift = torch.stack([torch.as_tensor(qp[0], dtype=torch.float32, device=dev).reshape(()) for qp in qparams])
+    lookup, shift, n_bins = _qparam_tables(qparams, dev)
     if out is None:
         out = torch.empty((n, k), dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
@@ -971,6 +979,118 @@ def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[
                                        len(batch), n, _ptr(out), _stream(dev))
     _lib.check(st, "tplr_dequantize_batch")
     return out
+
+
+class PayloadStage:
+    """One window's payloads of all peers as flat buffers in the layout the batch kernels read.
+
+    The reference keeps a gathered window as per-parameter Python lists, `state_dict.<name>idxs`,
+    `<name>vals` and `<name>quant_params`, one entry per peer (src/tplr/comms.py:1938-1963), and moves
+    them tensor by tensor (torch.load with map_location :602-606; pinned offload and reload,
+    neurons/validator.py:94-219).  Here peer p's parameters are concatenated in TensorBatch order
+    into one region of a pinned host buffer, the whole window crosses to the device in one copy,
+    and 8-bit codes are expanded on the device by one launch per peer.  Buffers are allocated once
+    (`max_peers` regions) and reused every window; the lists `load` returns are views of them,
+    valid until the next `load`."""
+
+    _ALIGN = 256
+
+    def __init__(self, batch: TensorBatch, k: int, max_peers: int, *, quantized: bool = True):
+        if max_peers < 1 or max_peers > _lib.TPLR_MAX_PEERS:
+            raise ValueError(f"max_peers must be in [1, {_lib.TPLR_MAX_PEERS}]")
+        if k < 2 or k % 2:
+            raise ValueError(f"k must be even and at least 2, got {k}")
+        n = batch.total_chunks
+        self.batch, self.k, self.max_peers, self.quantized = batch, k, max_peers, quantized
+        self.idx_bytes = n * (k // 2) * 3
+        self.val_bytes = n * k * (1 if quantized else 4)
+        up = lambda b: -(-b // self._ALIGN) * self._ALIGN  # noqa: E731
+        self.val_off = up(self.idx_bytes)
+        self.stride = self.val_off + up(self.val_bytes)
+        self.host = torch.empty(max_peers * self.stride, dtype=torch.uint8, pin_memory=True)
+        self.dev = torch.empty(max_peers * self.stride, dtype=torch.uint8, device=batch.device)
+        self.values = torch.empty((max_peers, n, k), dtype=torch.float32, device=batch.device) if quantized else None
+        self._copied: torch.cuda.Event | None = None  # the last host-to-device copy out of `host`
+        self._threads = max(1, min(8, os.cpu_count() or 1))
+
+    def _regions(self, buf: torch.Tensor, p: int) -> tuple[torch.Tensor, torch.Tensor]:
+        b = p * self.stride
+        idx = buf[b:b + self.idx_bytes]
+        val = buf[b + self.val_off:b + self.val_off + self.val_bytes]
+        return idx, (val if self.quantized else val.view(torch.float32))
+
+    @torch.no_grad()
+    def load(self, idxs: Sequence[Sequence[torch.Tensor]], vals: Sequence[Sequence[torch.Tensor]],
+             quant_params: Sequence[Sequence[QuantParamsT]] | None = None):
+        """`idxs[i][p]`, `vals[i][p]`, `quant_params[i][p]`: parameter i (TensorBatch order), peer p, as in
+        the reference's lists.  Host tensors go through the pinned buffer and one copy; device tensors
+        are concatenated on the device.  Returns (idx12, val): lists over peers of the flat packed
+        indices and the fp32 values (total_chunks, k), ready for batch_decompress_decode_batch,
+        peer_clip_scales_batch and index_stats_batch."""
+        T = len(self.batch)
+        if len(idxs) != T or len(vals) != T:
+            raise IndexError(f"{len(idxs)} index lists / {len(vals)} value lists for {T} parameters")
+        P = len(idxs[0])
+        if P < 1 or P > self.max_peers:
+            raise ValueError(f"{P} peers for a stage of {self.max_peers}")
+        want_dtype = torch.uint8 if self.quantized else torch.float32
+        for i in range(T):
+            y, x, _, _ = self.batch.xshape(i)
+            if len(idxs[i]) != P or len(vals[i]) != P:
+                raise IndexError(f"parameter {i}: {len(idxs[i])} index / {len(vals[i])} value entries for {P} peers")
+            for p in range(P):
+                a, v = idxs[i][p], vals[i][p]
+                if a.dtype != torch.uint8:
+                    raise ValueError(f"Expected uint8 for 12-bit packed indices, got {a.dtype}")
+                if v.dtype != want_dtype:
+                    raise ValueError(f"parameter {i}, peer {p}: values are {v.dtype}, the stage holds {want_dtype}")
+                if v.numel() != y * x * self.k or a.numel() * 2 != v.numel() * 3:
+                    raise RuntimeError(f"parameter {i}, peer {p}: {a.numel()} index bytes / {v.numel()} values for "
+                                       f"{y * x} chunks of k={self.k}")
+        on_host = idxs[0][0].device.type == "cpu"
+        if on_host and self._copied is not None:
+            self._copied.synchronize()  # the previous window's copy still reads the pinned buffer
+        if on_host:
+            # per peer: the library's host threads concatenate the parameters' tensors into the
+            # peer's region of the pinned buffer, whose transfer then runs while the next peer is packed
+            lib = _lib.load()
+            with torch.cuda.device(self.dev.device):
+                for p in range(P):
+                    for part, off, nbytes in ((idxs, 0, self.idx_bytes), (vals, self.val_off, self.val_bytes)):
+                        src = [part[i][p] if part[i][p].is_contiguous() else part[i][p].contiguous() for i in range(T)]
+                        ptrs = (C.c_void_p * T)(*[t.data_ptr() for t in src])
+                        sizes = (C.c_int64 * T)(*[t.numel() * t.element_size() for t in src])
+                        _lib.check(lib.tplr_gather_host(ptrs, sizes, T, self.host.data_ptr() + p * self.stride + off,
+                                                        self._threads), "tplr_gather_host")
+                    b = p * self.stride
+                    self.dev[b:b + self.stride].copy_(self.host[b:b + self.stride], non_blocking=True)
+                self._copied = torch.cuda.Event()
+                self._copied.record()
+        else:
+            for p in range(P):
+                ri, rv = self._regions(self.dev, p)
+                torch.cat([idxs[i][p].reshape(-1) for i in range(T)], out=ri)
+                torch.cat([vals[i][p].reshape(-1) for i in range(T)], out=rv)
+        out_i, out_v = [], []
+        for p in range(P):
+            ri, rv = self._regions(self.dev, p)
+            out_i.append(ri)
+            out_v.append(rv.view(-1, self.k))
+        if not self.quantized:
+            return out_i, out_v
+        if quant_params is None or len(quant_params) != T or any(len(q) != P for q in quant_params):
+            raise IndexError("quant_params must hold one entry per parameter and peer")
+        lookup, shift, n_bins = _qparam_tables([quant_params[i][p] for p in range(P) for i in range(T)], self.dev.device)
+        lib = _lib.load()
+        dev, n = self.dev.device, self.batch.total_chunks
+        with torch.cuda.device(dev):
+            for p in range(P):
+                st = lib.tplr_dequantize_batch(_ptr(out_v[p]), _ptr(lookup[p * T:(p + 1) * T]), _ptr(shift[p * T:(p + 1) * T]),
+                                               n_bins, self.k, _ptr(self.batch.table), T, n, _ptr(self.values[p]),
+                                               _stream(dev))
+                _lib.check(st, "tplr_dequantize_batch")
+        self._tables = (lookup, shift)  # alive until the launches above have run
+        return out_i, [self.values[p] for p in range(P)]
 
 
 @torch.no_grad()
@@ -1034,6 +1154,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "PayloadStage", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

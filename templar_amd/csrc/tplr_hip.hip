@@ -3,6 +3,10 @@
 // replaces are documented in include/tplr_hip.h.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <string.h>
+
+#include <thread>
+#include <vector>
 
 #include "../../include/tplr_hip.h"
 #include "tplr_device.h"
@@ -1380,6 +1384,39 @@ int tplr_pack12_host(const int64_t* idx, int64_t n, uint8_t* packed, int64_t* ba
         packed[3 * p + 2] = static_cast<uint8_t>(w >> 16);
     }
     if (bad) *bad = worst > 4095 ? worst : 0;
+    return 0;
+}
+
+int tplr_gather_host(const void* const* h_src, const int64_t* h_bytes, int64_t n_parts, void* h_dst,
+                     int n_threads) {
+    if (n_parts < 0 || n_threads < 1 || n_threads > 64) return TPLR_E_BADARG;
+    if (n_parts == 0) return 0;
+    if (!h_src || !h_bytes || !h_dst) return TPLR_E_BADARG;
+    int64_t total = 0;
+    for (int64_t i = 0; i < n_parts; ++i) {
+        if (h_bytes[i] < 0 || (h_bytes[i] > 0 && !h_src[i])) return TPLR_E_BADARG;
+        total += h_bytes[i];
+    }
+    // every thread copies an equal share of the concatenated bytes, cutting parts where its share ends
+    auto work = [=](int t) {
+        const int64_t lo = total * t / n_threads, hi = total * (t + 1) / n_threads;
+        int64_t at = 0;
+        for (int64_t i = 0; i < n_parts && at < hi; at += h_bytes[i], ++i) {
+            const int64_t b = at > lo ? at : lo, e = at + h_bytes[i] < hi ? at + h_bytes[i] : hi;
+            if (b < e)
+                memcpy(static_cast<char*>(h_dst) + b, static_cast<const char*>(h_src[i]) + (b - at),
+                       static_cast<size_t>(e - b));
+        }
+    };
+    if (n_threads == 1 || total < (1 << 20)) {
+        for (int t = 0; t < n_threads; ++t) work(t);
+        return 0;
+    }
+    std::vector<std::thread> pool;
+    pool.reserve(n_threads - 1);
+    for (int t = 1; t < n_threads; ++t) pool.emplace_back(work, t);
+    work(0);
+    for (auto& th : pool) th.join();
     return 0;
 }
 

@@ -671,3 +671,53 @@ def test_aggregate_without_transform_writes_the_gradient_layout(dev):
     tc.batch_decompress_decode_batch(tc.TensorBatch([outb]), flat_i, flat_v, k, use_dct=False)
     assert float((outb - got).abs().max()) <= 1e-6 * float(got.abs().max())
 
+
+
+# ---------------------------------------------------------------- a gathered window as flat buffers
+@pytest.mark.parametrize("quantized,where", [(True, "cpu"), (False, "cpu"), (True, "cuda")])
+def test_payload_stage_equals_per_parameter_path(dev, quantized, where):
+    # the reference's per-parameter lists (src/tplr/comms.py:1938-1963) of P peers, staged flat and
+    # aggregated in one launch, against the per-parameter calls of src/tplr/neurons.py:309-367
+    shapes = [(128, 192), (64, 64), (256, 128), (64, 320)]
+    k, P = 32, 5
+    comp = tc.TopKCompressor(use_quantization=quantized, quantization_bins=256, quantization_range=6)
+    tr = tc.ChunkingTransformer(_Stub([torch.empty(s) for s in shapes]), 64)
+    idxs, vals, qps = [[] for _ in shapes], [[] for _ in shapes], [[] for _ in shapes]
+    for i, s in enumerate(shapes):
+        for p in range(P):
+            g = t3(s, 4000 + 17 * p + i, row_scale=True).to(dev) * (1 + p)
+            out = comp.compress(tr.encode(g, use_dct=True), k)
+            idxs[i].append(out[0].to(where))
+            vals[i].append(out[1].to(where))
+            if quantized:
+                sh, sc, off, lut, dt = out[4]
+                qps[i].append((sh.to(where), sc, off, lut.to(where), dt))
+    outs = [torch.empty(s, device=dev) for s in shapes]
+    batch = tc.TensorBatch(outs)
+    stage = tc.PayloadStage(batch, k, 8, quantized=quantized)
+    for rep in range(2):  # the second window reuses the buffers
+        fi, fv = stage.load(idxs, vals, qps if quantized else None)
+        assert len(fi) == len(fv) == P and fv[0].shape == (batch.total_chunks, k) and fv[0].dtype == torch.float32
+        scale = tc.peer_clip_scales_batch(batch, fv, k)
+        tc.batch_decompress_decode_batch(batch, fi, fv, k, scale=scale)
+        for i, s in enumerate(shapes):
+            di = [t.to(dev) for t in idxs[i]]
+            dv = [t.to(dev) for t in vals[i]]
+            if quantized:
+                dv = comp.maybe_dequantize_values(dv, [tuple(q) for q in qps[i]], dev)
+            # staged values are the reference's de-quantised values, bit for bit
+            for p in range(P):
+                gi, gv = batch.payload_slice(i, fi[p], fv[p], k)
+                assert torch.equal(gi, di[p]) and torch.equal(gv, dv[p])
+            y, x = batch.xshape(i)[:2]
+            want = tc._aggregate_chunks([a.contiguous() for a in di], [b.contiguous() for b in dv], scale[i].contiguous(),
+                                        y, x, k, normalise=False, use_dct=True)
+            assert torch.equal(outs[i], want)
+            # and the oracle's batch_decompress + decode on the same payloads (its own clip factors)
+            ref = orc.decode2d(orc.batch_decompress([a.cpu().numpy() for a in di], [b.cpu().numpy() for b in dv],
+                                                    batch.xshape(i), 4096), use_dct=True)
+            assert np.abs(outs[i].cpu().numpy() - ref).max() <= 1e-5 * np.abs(ref).max()
+    with pytest.raises(ValueError):
+        tc.PayloadStage(batch, k, 2, quantized=quantized).load(idxs, vals, qps if quantized else None)
+    with pytest.raises(IndexError):
+        stage.load(idxs[:-1], vals[:-1], qps[:-1] if quantized else None)

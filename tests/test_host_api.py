@@ -143,6 +143,26 @@ def test_host_pack_unpack_vectors():
     assert tc.pack_12bit_indices(torch.arange(1000)).numel() == 1500  # 75 % of int16
 
 
+def test_host_gather_concatenates_parts_with_any_thread_count():
+    import ctypes as C
+
+    from templar_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(5)
+    sizes = [0, 1, 7, 4096, 3, 1 << 20, 123457, 0, 999, 2 << 20]
+    parts = [rng.integers(0, 256, n, dtype=np.uint8) for n in sizes]
+    want = np.concatenate(parts)
+    ptrs = (C.c_void_p * len(parts))(*[p.ctypes.data if p.size else None for p in parts])
+    nbytes = (C.c_int64 * len(parts))(*sizes)
+    for threads in (1, 2, 3, 8, 64):
+        dst = np.full(want.size + 16, 0xEE, np.uint8)
+        assert lib.tplr_gather_host(ptrs, nbytes, len(parts), dst.ctypes.data + 8, threads) == 0
+        assert np.array_equal(dst[8:-8], want) and (dst[:8] == 0xEE).all() and (dst[-8:] == 0xEE).all()
+    assert lib.tplr_gather_host(ptrs, nbytes, len(parts), None, 4) == _lib.TPLR_E_BADARG
+    assert lib.tplr_gather_host(ptrs, nbytes, len(parts), 1, 0) == _lib.TPLR_E_BADARG
+    assert lib.tplr_gather_host(None, None, 0, None, 1) == 0
+
+
 def test_pack_unpack_errors():
     with pytest.raises(ValueError, match="Number of indices must be even, got 3"):
         tc.pack_12bit_indices(torch.tensor([1, 2, 3]))
