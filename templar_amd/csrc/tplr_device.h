@@ -175,25 +175,45 @@ __device__ __forceinline__ uint32_t stat_threshold(uint32_t b1, uint32_t b2, int
 __device__ __forceinline__ void filter16(uint32_t& m, float thr, float x0, float x1, float x2, float x3, float x4,
                                          float x5, float x6, float x7, float x8, float x9, float x10, float x11,
                                          float x12, float x13, float x14, float x15) {
-    // m = (m << 16) | predicate bits, first value in the highest bit: compare writes the carry,
-    // add-with-carry of m to itself shifts it in.
-    asm("v_cmp_nlt_f32_e64 vcc, |%[a0]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a1]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a2]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a3]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a4]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a5]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a6]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a7]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a8]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a9]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a10]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a11]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a12]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a13]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a14]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc\n\t"
-        "v_cmp_nlt_f32_e64 vcc, |%[a15]|, %[t]\n\tv_addc_co_u32_e32 %[m], vcc, %[m], %[m], vcc"
-        : [m] "+v"(m)
+    // m = (m << 16) | predicate bits, first value in the highest bit: a compare writes a lane mask,
+    // add-with-carry of m to itself shifts it in.  A vector instruction that reads a scalar register
+    // pair which a vector instruction has just written needs two other instructions in between on
+    // this hardware, and the compiler does not look into inline assembly: the compares run three
+    // ahead of the adds, through three mask registers in turn.
+    uint64_t t0, t1, t2;
+    asm("v_cmp_nlt_f32_e64 %[t0], |%[a0]|, %[t]\n\t"
+        "v_cmp_nlt_f32_e64 %[t1], |%[a1]|, %[t]\n\t"
+        "v_cmp_nlt_f32_e64 %[t2], |%[a2]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t0]\n\t"
+        "v_cmp_nlt_f32_e64 %[t0], |%[a3]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t1]\n\t"
+        "v_cmp_nlt_f32_e64 %[t1], |%[a4]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t2]\n\t"
+        "v_cmp_nlt_f32_e64 %[t2], |%[a5]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t0]\n\t"
+        "v_cmp_nlt_f32_e64 %[t0], |%[a6]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t1]\n\t"
+        "v_cmp_nlt_f32_e64 %[t1], |%[a7]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t2]\n\t"
+        "v_cmp_nlt_f32_e64 %[t2], |%[a8]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t0]\n\t"
+        "v_cmp_nlt_f32_e64 %[t0], |%[a9]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t1]\n\t"
+        "v_cmp_nlt_f32_e64 %[t1], |%[a10]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t2]\n\t"
+        "v_cmp_nlt_f32_e64 %[t2], |%[a11]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t0]\n\t"
+        "v_cmp_nlt_f32_e64 %[t0], |%[a12]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t1]\n\t"
+        "v_cmp_nlt_f32_e64 %[t1], |%[a13]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t2]\n\t"
+        "v_cmp_nlt_f32_e64 %[t2], |%[a14]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t0]\n\t"
+        "v_cmp_nlt_f32_e64 %[t0], |%[a15]|, %[t]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t1]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t2]\n\t"
+        "v_addc_co_u32_e64 %[m], vcc, %[m], %[m], %[t0]"
+        : [m] "+v"(m), [t0] "=&s"(t0), [t1] "=&s"(t1), [t2] "=&s"(t2)
         : [t] "s"(thr), [a0] "v"(x0), [a1] "v"(x1), [a2] "v"(x2), [a3] "v"(x3), [a4] "v"(x4), [a5] "v"(x5),
           [a6] "v"(x6), [a7] "v"(x7), [a8] "v"(x8), [a9] "v"(x9), [a10] "v"(x10), [a11] "v"(x11), [a12] "v"(x12),
           [a13] "v"(x13), [a14] "v"(x14), [a15] "v"(x15)
@@ -287,7 +307,12 @@ constexpr uint64_t keepmax_mask(int k2, int j, int base) {
 // xnor with the lane mask, two selects.
 __device__ __forceinline__ uint64_t cmp_exchange(uint64_t e, uint64_t o, uint64_t keepmax) {
     uint64_t take;
-    asm("v_cmp_gt_u64_e64 %0, %1, %2\n\ts_xnor_b64 %0, %0, %3" : "=&s"(take) : "v"(o), "v"(e), "s"(keepmax) : "scc");
+    // (the s_nop keeps the selects, which read the mask as a vector operand, two instructions away from
+    // the vector compare that first wrote the register pair)
+    asm("v_cmp_gt_u64_e64 %0, %1, %2\n\ts_xnor_b64 %0, %0, %3\n\ts_nop 0"
+        : "=&s"(take)
+        : "v"(o), "v"(e), "s"(keepmax)
+        : "scc");
     uint32_t lo, hi;
     asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(lo) : "v"(static_cast<uint32_t>(e)), "v"(static_cast<uint32_t>(o)), "s"(take));
     asm("v_cndmask_b32_e64 %0, %1, %2, %3"
