@@ -158,3 +158,33 @@ def test_encode_decode_real_tensors(dev):  # :255-275
     want = orc.encode2d(param.cpu().numpy(), 8, 8)
     assert np.abs(encoded_dct.cpu().numpy() - want).max() <= 1e-5 * np.abs(want).max()
     assert torch.allclose(decoded_dct, param, atol=1e-6)
+
+
+# ---------------------------------------------------------------- callers' init-time shape probe
+@pytest.mark.parametrize("use_dct", [False, True])
+def test_init_time_shape_probe(dev, use_dct):
+    # neurons/miner.py:245-254, neurons/validator.py:394-404: encode + compress of an uninitialised
+    # fp16 tensor per parameter, only to record xshape and totalk
+    shapes = [(128, 192), (64,), (2048,), (100, 48), (192, 64)]
+    tr = ChunkingTransformer(_Shapes(shapes, dev), 64)
+    q = TopKCompressor(use_quantization=True, quantization_bins=4, quantization_range=6)
+    want = {(128, 192): ((2, 3, 64, 64), 4096), (64,): ((1, 64), 64), (2048,): ((32, 64), 64),
+            (100, 48): ((2, 1, 50, 48), 2400), (192, 64): ((3, 1, 64, 64), 4096)}
+    for s in shapes:
+        probe = torch.full(s, float("nan"), dtype=torch.float16, device=dev)
+        enc = tr.encode(probe, use_dct=use_dct)
+        idx, val, xshape, totalk, qp = q.compress(enc, 32)
+        assert (tuple(xshape), totalk) == want[s]
+        assert idx.dtype == torch.uint8 and val.dtype == torch.uint8 and len(qp) == 5
+        k = min(32, totalk)
+        assert val.shape == tuple(xshape[:-2 if len(xshape) == 4 else -1]) + (k,)
+        assert idx.numel() * 2 == val.numel() * 3
+
+
+class _Shapes:
+    def __init__(self, shapes, dev):
+        self._p = [torch.nn.Parameter(torch.empty(s, device=dev)) for s in shapes]
+
+    def named_parameters(self):
+        for i, p in enumerate(self._p):
+            yield f"p{i}", p
