@@ -984,6 +984,9 @@ struct IdxPtrs {
     const uint8_t* idx[kStatPeers];
 };
 
+// kPerPass: peers handled by one wave instruction: 2 when k <= 32 (one peer per half of the wave), 1 when
+// k <= 64; 0 = rows of any length, entry by entry.
+template <int kPerPass>
 __global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int k,
                                                     const tplr_tensor_desc* __restrict__ table,
                                                     const tplr_tensor_desc single, int n_tensors, int64_t total,
@@ -1020,6 +1023,88 @@ __global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int
     };
     clear_totals();
     int t_cur = c.t;
+    if constexpr (kPerPass > 0) {
+        // One entry per lane and peer, all peers of a row in registers; the next row's entries are
+        // requested before this row is worked on.  Repeats and maxima are kept per lane and
+        // reach the per-tensor totals when those are flushed.
+        constexpr int kPasses = kStatPeers / kPerPass;
+        const int sub = kPerPass == 2 ? lane >> 5 : 0;
+        const int j = kPerPass == 2 ? (lane & 31) : lane;
+        const bool jon = j < k;
+        const int joff = 3 * (j >> 1) + (j & 1);
+        const uint32_t jshift = (j & 1) * 4;
+        uint32_t cur[kPasses], nxt[kPasses], rep[kPasses];
+        int top[kPasses];
+#pragma unroll
+        for (int i = 0; i < kPasses; ++i) cur[i] = nxt[i] = rep[i] = 0, top[i] = -1;
+        auto request = [&](uint32_t (&e)[kPasses], int64_t g) {
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i) {
+                if (i * kPerPass < P) {  // wave-uniform
+                    const uint8_t* base = ip.idx[i * kPerPass];
+                    if constexpr (kPerPass == 2) base = (sub && i * 2 + 1 < P) ? ip.idx[i * 2 + 1] : base;
+                    const gbyte* row = (const gbyte*)base + g * idx_stride;
+                    if (jon) e[i] = *(const gu16*)(row + joff);
+                }
+            }
+        };
+        auto fold = [&]() {  // per-lane repeats and maxima into the per-tensor totals
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i) {
+                const int p = i * kPerPass + sub;
+                if (i * kPerPass < P) {
+                    if (jon && p < P) {
+                        if (rep[i]) atomicAdd(&dup_l[p], rep[i]);
+                        if (top[i] >= 0) atomicMax(&mx_l[p], top[i]);
+                    }
+                    rep[i] = 0, top[i] = -1;
+                }
+            }
+        };
+        request(nxt, g0);
+        for (int64_t g = g0; g < g1; ++g) {
+            if (c.t != t_cur) {  // wave-uniform
+                fold();
+                flush_totals(t_cur);
+                clear_totals();
+                t_cur = c.t;
+            }
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i) cur[i] = (nxt[i] >> jshift) & 0xfffu;
+            request(nxt, g + 1 < g1 ? g + 1 : g);
+            const uint4 z = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int q = 0; q < 16; ++q) reinterpret_cast<uint4*>(mask)[q * 64 + lane] = z;
+            wave_lds_fence();
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i) {
+                const int p = i * kPerPass + sub;
+                if (i * kPerPass < P && jon && p < P) {
+                    const uint32_t old = atomicOr(&mask[cur[i]], 1u << p);
+                    rep[i] += (old >> p) & 1u;
+                    top[i] = top[i] > static_cast<int>(cur[i]) ? top[i] : static_cast<int>(cur[i]);
+                }
+            }
+            wave_lds_fence();
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i) {
+                const int p = i * kPerPass + sub;
+                if (i * kPerPass < P && jon && p + 1 < P) {
+                    uint32_t m = mask[cur[i]] >> (p + 1);  // the peers after p that sent this entry too
+                    while (m) {
+                        const int q = p + 1 + __builtin_ctz(m);
+                        atomicAdd(&pair_l[p * kStatPeers + q], 1u);
+                        m &= m - 1;
+                    }
+                }
+            }
+            wave_lds_fence();
+            if (g + 1 < g1) cursor_next(c, g + 1);
+        }
+        fold();
+        flush_totals(t_cur);
+        return;
+    }
     for (int64_t g = g0; g < g1; ++g) {
         if (c.t != t_cur) {  // wave-uniform
             flush_totals(t_cur);
@@ -1726,13 +1811,22 @@ int tplr_index_stats_batch(const uint8_t* const* h_idx12, int n_peers, int k, co
         ip.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
         if (p < n_peers && !ip.idx[p]) return TPLR_E_BADARG;
     }
-    static int resident = 0;
-    if (resident == 0) resident = persistent_grid(k_index_stats, int64_t{1} << 40);
     const int64_t need = ((total_rows + 7) / 8) * 8;
     tplr_tensor_desc none = {};
-    hipLaunchKernelGGL(k_index_stats, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
-                       static_cast<hipStream_t>(stream), ip, n_peers, k, d_desc, none, n_tensors, total_rows,
-                       reinterpret_cast<unsigned long long*>(d_pair), reinterpret_cast<unsigned long long*>(d_dup), d_max);
+    auto launch = [&](auto kernel, int& resident) {
+        if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+                           static_cast<hipStream_t>(stream), ip, n_peers, k, d_desc, none, n_tensors, total_rows,
+                           reinterpret_cast<unsigned long long*>(d_pair), reinterpret_cast<unsigned long long*>(d_dup),
+                           d_max);
+    };
+    static int resident[3] = {0, 0, 0};
+    if (k <= 32)
+        launch(k_index_stats<2>, resident[2]);
+    else if (k <= 64)
+        launch(k_index_stats<1>, resident[1]);
+    else
+        launch(k_index_stats<0>, resident[0]);
     return launch_status();
 }
 

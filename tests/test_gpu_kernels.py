@@ -615,6 +615,36 @@ def test_index_stats_match_reference_overlap(dev):
     assert orc.index_bounds(np.array([0, 1, 2, 3]), 64) is None
 
 
+@pytest.mark.parametrize("P,k", [(2, 32), (15, 32), (32, 32), (7, 64), (31, 64), (3, 128), (9, 6)])
+def test_index_stats_every_row_length_and_peer_count(dev, P, k):
+    # k <= 32: two peers per wave instruction; k <= 64: one; longer rows: entry by entry
+    rng = np.random.default_rng(1000 * P + k)
+    counts = [37, 1, 90]
+    n = sum(counts)
+    shared = np.stack([rng.permutation(4096)[:k] for _ in range(n)])
+    rows = []
+    for p in range(P):
+        own = np.stack([rng.permutation(4096)[:k] for _ in range(n)])
+        r = np.where(rng.random((n, k)) < 0.4, shared, own)
+        rows.append(r.astype(np.int64))  # may repeat an index inside a row: counted below
+    rows[P - 1][n - 1, k - 1] = 4095
+    idxs = [torch.from_numpy(orc.pack12(r)).to(dev) for r in rows]
+    pair, dup, top = tc.index_stats_batch(counts, idxs, k)
+    b0 = 0
+    for t, cnt in enumerate(counts):
+        part = [r[b0:b0 + cnt] for r in rows]
+        want_dup = [sum(k - len(np.unique(row)) for row in r) for r in part]
+        assert dup[t].cpu().tolist() == want_dup
+        assert top[t].cpu().tolist() == [int(r.max()) for r in part]
+        # shared entries of peers i < j, row by row, as sets (every repeat of peer i's entry counts once more)
+        got = pair[t].cpu().numpy()
+        for i in range(P):
+            for j in range(i + 1, P):
+                want = sum(int(np.isin(part[i][c], part[j][c]).sum()) for c in range(cnt))
+                assert got[i, j] == want, (t, i, j)
+        b0 += cnt
+
+
 def test_dequantize_batch_matches_per_parameter_reference_path(dev):
     rng = np.random.default_rng(31)
     shapes = [(128, 64), (64, 192), (192, 128)]
