@@ -21,6 +21,7 @@ each and without materialising the dense coefficient tensor.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import math
 import os
@@ -56,12 +57,34 @@ def _stream(dev: torch.device):
     return C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
 
+def _on(dev: torch.device):
+    """Context in which `dev` is the current device (kernel launches go to the current one);
+    free when it already is."""
+    if torch.cuda.current_device() == dev.index:
+        return contextlib.nullcontext()
+    return torch.cuda.device(dev)
+
+
 def _need_device(t: torch.Tensor, what: str) -> None:
     if not t.is_cuda:
         raise RuntimeError(
             f"templar_amd.{what}: tensor is on '{t.device}'; the codec kernels run on a HIP device only "
             "(there is no CPU code path)"
         )
+
+
+def _val_on(v: torch.Tensor, dev: torch.device) -> torch.Tensor:
+    """Values as the kernels read them: fp32, contiguous, on `dev` (no work when they already are)."""
+    if v.device == dev and v.dtype == torch.float32 and v.is_contiguous():
+        return v
+    return _f32c(v.to(dev))
+
+
+def _idx_on(i: torch.Tensor, dev: torch.device) -> torch.Tensor:
+    """A packed index stream as the kernels read it: flat, contiguous, on `dev`."""
+    if i.device == dev and i.dim() == 1 and i.is_contiguous():
+        return i
+    return i.to(dev).reshape(-1).contiguous()
 
 
 def _f32c(t: torch.Tensor) -> torch.Tensor:
@@ -83,7 +106,7 @@ def pack_12bit_indices(indices: torch.Tensor) -> torch.Tensor:
         flat = flat.to(torch.int64)
     flat = flat.contiguous()
     if flat.is_cuda:
-        with torch.cuda.device(flat.device):
+        with _on(flat.device):
             # the reference finds the maximum first (and raises on it) before the parity check
             err = torch.zeros(1, dtype=torch.int32, device=flat.device)
             out = torch.empty((n // 2) * 3, dtype=torch.uint8, device=flat.device)
@@ -127,7 +150,7 @@ def unpack_12bit_indices(packed: torch.Tensor, values_shape: ShapeT) -> torch.Te
     lib = _lib.load()
     out = torch.empty(n, dtype=torch.int64, device=packed.device)
     if packed.is_cuda:
-        with torch.cuda.device(packed.device):
+        with _on(packed.device):
             _lib.check(lib.tplr_unpack12(_ptr(packed), n, _ptr(out), _stream(packed.device)), "tplr_unpack12")
     else:
         _lib.check(lib.tplr_unpack12_host(_ptr(packed), n, _ptr(out)), "tplr_unpack12_host")
@@ -239,7 +262,7 @@ class ChunkingTransformer:
         xin = _f32c(x)
         out = torch.empty((R // h, Cc // w, h, w) if out_chunked else (R, Cc), dtype=torch.float32, device=x.device)
         if out.numel():
-            with torch.cuda.device(x.device):
+            with _on(x.device):
                 st = lib.tplr_dct2d_dense(_ptr(xin), R, Cc, h, w, _ptr(_f32c(bh)), _ptr(_f32c(bw)), int(in_chunked),
                                           int(out_chunked), _ptr(out), _stream(x.device))
             _lib.check(st, "tplr_dct2d_dense")
@@ -280,7 +303,7 @@ class ChunkingTransformer:
                 lib = _lib.load()
                 xin = x if (x.dtype == torch.float32 and x.stride(1) == 1 and x.stride(0) >= Cc) else _f32c(x)
                 out = torch.empty((R // _CH, Cc // _CH, _CH, _CH), dtype=torch.float32, device=x.device)
-                with torch.cuda.device(x.device):
+                with _on(x.device):
                     st = lib.tplr_dct2d_fwd(_ptr(xin), R, Cc, xin.stride(0), _ptr(out), _stream(x.device))
                 _lib.check(st, "tplr_dct2d_fwd")
                 return out if x.dtype == torch.float32 else out.to(x.dtype)
@@ -296,7 +319,7 @@ class ChunkingTransformer:
             lib = _lib.load()
             xin = _f32c(rows)
             out = torch.empty_like(xin)
-            with torch.cuda.device(x.device):
+            with _on(x.device):
                 st = lib.tplr_dct1d(_ptr(xin), xin.shape[0], 0, _ptr(out), _stream(x.device))
             _lib.check(st, "tplr_dct1d")
             return out if x.dtype == torch.float32 else out.to(x.dtype)
@@ -317,7 +340,7 @@ class ChunkingTransformer:
                 lib = _lib.load()
                 xin = _f32c(x)
                 out = torch.empty((Y * h, X * w), dtype=torch.float32, device=x.device)
-                with torch.cuda.device(x.device):
+                with _on(x.device):
                     st = lib.tplr_dct2d_inv(_ptr(xin), Y * h, X * w, _ptr(out), X * w, _stream(x.device))
                 _lib.check(st, "tplr_dct2d_inv")
                 return out if x.dtype == torch.float32 else out.to(x.dtype)
@@ -332,7 +355,7 @@ class ChunkingTransformer:
             lib = _lib.load()
             xin = _f32c(x)
             out = torch.empty_like(xin)
-            with torch.cuda.device(x.device):
+            with _on(x.device):
                 st = lib.tplr_dct1d(_ptr(xin), xin.shape[0], 1, _ptr(out), _stream(x.device))
             _lib.check(st, "tplr_dct1d")
             out = out.reshape(-1)
@@ -380,7 +403,7 @@ def _topk_rows(rows: torch.Tensor, k: int):
     idx = torch.empty(n_rows * (k // 2) * 3, dtype=torch.uint8, device=rows.device)
     val = torch.empty((n_rows, k), dtype=torch.float32, device=rows.device)
     if n_rows:
-        with torch.cuda.device(rows.device):
+        with _on(rows.device):
             st = lib.tplr_topk_pack(_ptr(rows), n_rows, n, k, _ptr(idx), _ptr(val), _stream(rows.device))
         _lib.check(st, "tplr_topk_pack")
     return idx, val
@@ -394,7 +417,7 @@ def _encode_topk(x2d: torch.Tensor, R: int, Cc: int, ld: int, k: int, use_dct: b
     idx = torch.empty(n_chunks * (k // 2) * 3, dtype=torch.uint8, device=x2d.device)
     val = torch.empty((R // _CH, Cc // _CH, k), dtype=torch.float32, device=x2d.device)
     if n_chunks:
-        with torch.cuda.device(x2d.device):
+        with _on(x2d.device):
             st = lib.tplr_encode_topk_pack(_ptr(x2d), R, Cc, ld, k, int(use_dct), _ptr(idx), _ptr(val),
                                            _stream(x2d.device))
         _lib.check(st, "tplr_encode_topk_pack")
@@ -408,7 +431,7 @@ def _peer_scales(vals: Sequence[torch.Tensor], block_norms: torch.Tensor | None,
     if P > _lib.TPLR_MAX_PEERS:
         raise NotImplementedError(f"{P} peers: the HIP aggregate kernel takes up to {_lib.TPLR_MAX_PEERS}")
     scale = torch.empty(P, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         if block_norms is not None:
             norms = block_norms.to(device=dev, dtype=torch.float32).contiguous()
             st = lib.tplr_clip_scales(_ptr(norms), P, 0, _ptr(scale), None, _stream(dev))
@@ -450,7 +473,7 @@ def _aggregate_chunks(idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor]
     if out is None:
         out = torch.empty((R, Cc) if as_rows else (Y, X, _CH, _CH), dtype=torch.float32, device=dev)
     if n_chunks:
-        with torch.cuda.device(dev):
+        with _on(dev):
             st = lib.tplr_decode_aggregate(ip, vp, _ptr(scale), P, k, R, Cc,
                                            _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM, int(normalise), int(use_dct),
                                            _ptr(out), out.stride(0) if as_rows else 0, _ptr(sumsq), _stream(dev))
@@ -476,7 +499,7 @@ def _scatter_rows(idx: torch.Tensor, val: torch.Tensor, n_rows: int, kk: int, ro
         return out
     err = torch.zeros(1, dtype=torch.int32, device=dev)
     packed = idx.dtype == torch.uint8
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.tplr_scatter_rows(_ptr(idx) if packed else None, None if packed else _ptr(idx), _ptr(val), n_rows, kk,
                                    row_len, _lib.REDUCE_MEAN, _ptr(out), _ptr(err), _stream(dev))
     _lib.check(st, "tplr_scatter_rows")
@@ -613,8 +636,8 @@ class TopKCompressor:
                 raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i_data.dtype}")
         _need_device(p, "TopKCompressor.batch_decompress")
         dev = p.device
-        vals = [_f32c(v.to(dev)) for v in val_list]
-        idxs = [i.to(dev).reshape(-1).contiguous() for i in idx_list]
+        vals = [_val_on(v, dev) for v in val_list]
+        idxs = [_idx_on(i, dev) for i in idx_list]
         xshape = tuple(xshape)
         k = vals[0].shape[-1]
         scale = None
@@ -736,8 +759,8 @@ def batch_decompress_decode(idxs: Sequence[torch.Tensor], vals: Sequence[torch.T
             raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
     dev = vals[0].device
     _need_device(vals[0], "batch_decompress_decode")
-    vals = [_f32c(v.to(dev)) for v in vals]
-    idxs = [i.to(dev).reshape(-1).contiguous() for i in idxs]
+    vals = [_val_on(v, dev) for v in vals]
+    idxs = [_idx_on(i, dev) for i in idxs]
     scale = None
     if clip_norm and not normalise:
         scale = _peer_scales(vals, block_norms, dev)
@@ -807,7 +830,7 @@ def encode_compress_batch(batch: TensorBatch, topk: int, *, use_dct: bool = True
         idx12 = torch.empty(n * (k // 2) * 3, dtype=torch.uint8, device=batch.device)
     if val is None:
         val = torch.empty((n, k), dtype=torch.float32, device=batch.device)
-    with torch.cuda.device(batch.device):
+    with _on(batch.device):
         st = lib.tplr_encode_topk_pack_batch(_ptr(batch.table), len(batch), n, k, int(use_dct), _ptr(idx12), _ptr(val),
                                              _stream(batch.device))
     _lib.check(st, "tplr_encode_topk_pack_batch")
@@ -829,7 +852,7 @@ def peer_clip_scales_batch(batch: TensorBatch, vals: Sequence[torch.Tensor], k: 
     ss = torch.empty((len(batch), P, slices), dtype=torch.float32, device=dev)
     scale = torch.empty((len(batch), P), dtype=torch.float32, device=dev)
     vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(lib.tplr_segment_sumsq(vp, P, k, _ptr(batch.table), len(batch), slices, _ptr(ss), _stream(dev)),
                    "tplr_segment_sumsq")
         _lib.check(lib.tplr_clip_scales_batch(_ptr(ss), len(batch), P, slices, _ptr(scale), None, _stream(dev)),
@@ -857,7 +880,7 @@ def batch_decompress_decode_batch(out: TensorBatch, idxs: Sequence[torch.Tensor]
         scale = peer_clip_scales_batch(out, vals, k)
     ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
     vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
-    with torch.cuda.device(out.device):
+    with _on(out.device):
         st = lib.tplr_decode_aggregate_batch(ip, vp, _ptr(scale), P, k, _ptr(out.table), len(out), n,
                                              _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM, int(normalise), int(use_dct),
                                              _ptr(sumsq), _stream(out.device))
@@ -888,7 +911,7 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
     dev, n = ef.device, ef.total_chunks
     idx12 = torch.empty(n * (k // 2) * 3, dtype=torch.uint8, device=dev)
     val = torch.empty((n, k), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         if null_round:
             for t in ef.tensors:
                 t.zero_()
@@ -907,7 +930,7 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
             q, qp = compressor._quantize_values(val[b:b + y * x].reshape(y, x, k))
             quant.append((q, qp))
             sent[b:b + y * x] = compressor._dequantize_values(q, qp).reshape(y * x, k)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.tplr_ef_subtract_batch(_ptr(idx12), _ptr(sent), k, _ptr(ef.table), len(ef), n, int(use_dct),
                                         _stream(dev))
     _lib.check(st, "tplr_ef_subtract_batch")
@@ -974,7 +997,7 @@ def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[
     lookup, shift, n_bins = _qparam_tables(qparams, dev)
     if out is None:
         out = torch.empty((n, k), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.tplr_dequantize_batch(_ptr(codes.contiguous()), _ptr(lookup), _ptr(shift), n_bins, k, _ptr(batch.table),
                                        len(batch), n, _ptr(out), _stream(dev))
     _lib.check(st, "tplr_dequantize_batch")
@@ -1054,7 +1077,7 @@ class PayloadStage:
             # per peer: the library's host threads concatenate the parameters' tensors into the
             # peer's region of the pinned buffer, whose transfer then runs while the next peer is packed
             lib = _lib.load()
-            with torch.cuda.device(self.dev.device):
+            with _on(self.dev.device):
                 for p in range(P):
                     for part, off, nbytes in ((idxs, 0, self.idx_bytes), (vals, self.val_off, self.val_bytes)):
                         src = [part[i][p] if part[i][p].is_contiguous() else part[i][p].contiguous() for i in range(T)]
@@ -1083,7 +1106,7 @@ class PayloadStage:
         lookup, shift, n_bins = _qparam_tables([quant_params[i][p] for p in range(P) for i in range(T)], self.dev.device)
         lib = _lib.load()
         dev, n = self.dev.device, self.batch.total_chunks
-        with torch.cuda.device(dev):
+        with _on(dev):
             for p in range(P):
                 st = lib.tplr_dequantize_batch(_ptr(out_v[p]), _ptr(lookup[p * T:(p + 1) * T]), _ptr(shift[p * T:(p + 1) * T]),
                                                n_bins, self.k, _ptr(self.batch.table), T, n, _ptr(self.values[p]),
@@ -1133,7 +1156,7 @@ def index_stats_batch(batch: "TensorBatch | Sequence[int]", idxs: Sequence[torch
     dup = torch.zeros((T, P), dtype=torch.int64, device=dev)
     top = torch.full((T, P), -1, dtype=torch.int32, device=dev)
     ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.tplr_index_stats_batch(ip, P, k, _ptr(table), T, total, _ptr(pair), _ptr(dup), _ptr(top), _stream(dev))
     _lib.check(st, "tplr_index_stats_batch")
     return pair, dup, top
