@@ -225,6 +225,11 @@ def main():
         ms_both, _ = event_ms(both, steps, warmup)
         ms1, _ = event_ms(k1, steps, 1)
         ms2, _ = event_ms(k2, steps, 1)
+        # the same step through the Python entry point with templar's 4-bin quantiser on
+        # (hparams.json:59-60): + one quantise and one de-quantise launch over the payload
+        q4 = tc.TopKCompressor(use_quantization=True, quantization_bins=4, quantization_range=6)
+        _, ms_q = event_ms(lambda: tc.error_feedback_step_batch(eb, batch, 0.95, k, use_dct=True, compressor=q4),
+                           max(3, steps // 4), 1)
         b1 = n_chunks * (2 * 16384 + 16384 + 11 * k // 2)
         b2 = n_chunks * (16384 + 11 * k // 2 + 16384)
         return {
@@ -233,6 +238,7 @@ def main():
             "frac_of_hbm_peak": round((b1 + b2) / (ms_both * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
             "update_encode_ms": round(ms1, 4), "update_encode_bytes": b1,
             "subtract_decoded_ms": round(ms2, 4), "subtract_decoded_bytes": b2,
+            "with_4bin_quantiser_wall_ms": round(ms_q, 4),
         }
 
     if args.profile == "miner":

@@ -363,6 +363,26 @@ class ChunkingTransformer:
         return self.einsum_2d_t(x, self._basis32(self.b_dict, n1, x.device)).reshape(-1)
 
 
+_FLAT_DESC: dict = {}
+
+
+def _flat_desc(rows: int, dev: torch.device) -> torch.Tensor:
+    """Device descriptor of one un-chunked tensor of `rows` payload rows (what the flat-payload
+    kernels take for a single parameter); a few hundred distinct sizes per model, kept."""
+    import numpy as np
+
+    key = (dev, rows)
+    t = _FLAT_DESC.get(key)
+    if t is None:
+        if len(_FLAT_DESC) >= 4096:
+            _FLAT_DESC.clear()
+        desc = np.zeros(1, dtype=np.dtype([("dense", "<u8"), ("ld", "<i8"), ("chunk_begin", "<i8"), ("x_chunks", "<i4"),
+                                           ("y_chunks", "<i4")]))
+        desc[0] = (0, 0, 0, rows, 1)
+        t = _FLAT_DESC[key] = torch.from_numpy(desc.view(np.uint8).copy()).to(dev)
+    return t
+
+
 # ----------------------------------------------------------------------------------------
 # kernels behind TopKCompressor
 # ----------------------------------------------------------------------------------------
@@ -671,6 +691,22 @@ class TopKCompressor:
     @torch.no_grad()
     def _quantize_values(self, val: torch.Tensor) -> tuple[torch.Tensor, QuantParamsT]:
         half = self.n_bins // 2
+        n = val.numel()
+        if val.is_cuda and val.dtype == torch.float32 and n >= 4 and n % 4 == 0 and self.n_bins <= 256:
+            # one launch (sums in double) instead of a dozen reductions and scatters; the scale is the
+            # only value that travels to the host, as in the reference (float(scale), :620)
+            lib = _lib.load()
+            dev = val.device
+            v = val.contiguous()
+            q = torch.empty(val.shape, dtype=torch.uint8, device=dev)
+            stats = torch.empty(2, dtype=torch.float32, device=dev)
+            lookup = torch.empty(self.n_bins, dtype=torch.float32, device=dev)
+            with _on(dev):
+                st = lib.tplr_quantize_batch(_ptr(v), 4, _ptr(_flat_desc(n // 4, dev)), 1, self.n_bins,
+                                             C.c_float(self.range_in_sigmas), _ptr(q), _ptr(stats[0:1]), _ptr(stats[1:2]),
+                                             _ptr(lookup), _stream(dev))
+            _lib.check(st, "tplr_quantize_batch")
+            return q, (stats[0], float(stats[1]), half, lookup, val.dtype)
         shift = val.mean()
         centred = val - shift
         scale = self.range_in_sigmas * (centred.norm() / math.sqrt(centred.numel() - 1)) / self.n_bins
@@ -923,13 +959,19 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
     _lib.check(st, "tplr_ef_encode_topk_pack_batch")
     quant, sent = None, val
     if compressor is not None and compressor.use_quantization:
-        quant, sent = [], torch.empty_like(val)
+        codes, shift, scale, lookup = quantize_batch(ef, val, k, compressor.n_bins, compressor.range_in_sigmas)
+        sent = torch.empty_like(val)
+        with _on(dev):
+            st = lib.tplr_dequantize_batch(_ptr(codes), _ptr(lookup), _ptr(shift), compressor.n_bins, k, _ptr(ef.table),
+                                           len(ef), n, _ptr(sent), _stream(dev))
+        _lib.check(st, "tplr_dequantize_batch")
+        scales = scale.tolist()  # the reference's quant_params carry the scale as a Python float (:620)
+        quant = []
         for i in range(len(ef)):
             y, x, _, _ = ef.xshape(i)
             b = ef.offsets[i]
-            q, qp = compressor._quantize_values(val[b:b + y * x].reshape(y, x, k))
-            quant.append((q, qp))
-            sent[b:b + y * x] = compressor._dequantize_values(q, qp).reshape(y * x, k)
+            quant.append((codes[b:b + y * x].reshape(y, x, k),
+                          (shift[i], scales[i], compressor.n_bins // 2, lookup[i], torch.float32)))
     with _on(dev):
         st = lib.tplr_ef_subtract_batch(_ptr(idx12), _ptr(sent), k, _ptr(ef.table), len(ef), n, int(use_dct),
                                         _stream(dev))
@@ -979,6 +1021,26 @@ def _qparam_tables(qparams: Sequence[QuantParamsT], dev: torch.device) -> tuple[
     lookup = torch.stack([qp[3].reshape(n_bins).float() for qp in qparams])
     shift = torch.stack([torch.as_tensor(qp[0], dtype=torch.float32, device=lookup.device).reshape(()) for qp in qparams])
     return lookup.to(dev).contiguous(), shift.to(dev).contiguous(), n_bins
+
+
+@torch.no_grad()
+def quantize_batch(batch: TensorBatch, val: torch.Tensor, k: int, n_bins: int = 256, range_in_sigmas: float = 6.0):
+    """TopKCompressor._quantize_values (reference :582-621) for every parameter of a flat payload
+    in one launch: codes (total_chunks, k) uint8, and per parameter shift (T,), scale (T,) and
+    lookup (T, n_bins), all on the device.  Sums are carried in double and rounded once."""
+    lib = _lib.load()
+    dev, n, T = batch.device, batch.total_chunks, len(batch)
+    if val.dtype != torch.float32 or val.numel() != n * k or not val.is_contiguous():
+        raise RuntimeError(f"{val.numel()} values of {val.dtype} for {n} chunks of k={k}")
+    codes = torch.empty((n, k), dtype=torch.uint8, device=dev)
+    shift = torch.empty(T, dtype=torch.float32, device=dev)
+    scale = torch.empty(T, dtype=torch.float32, device=dev)
+    lookup = torch.empty((T, n_bins), dtype=torch.float32, device=dev)
+    with _on(dev):
+        st = lib.tplr_quantize_batch(_ptr(val), k, _ptr(batch.table), T, n_bins, C.c_float(range_in_sigmas), _ptr(codes),
+                                     _ptr(shift), _ptr(scale), _ptr(lookup), _stream(dev))
+    _lib.check(st, "tplr_quantize_batch")
+    return codes, shift, scale, lookup
 
 
 @torch.no_grad()
@@ -1177,6 +1239,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "PayloadStage", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

@@ -1149,6 +1149,109 @@ __global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int
 // De-quantise one peer's flat payload of 8-bit codes: value = lookup[t][code] + shift[t], the
 // tensor t found from the row id (TopKCompressor._dequantize_values, src/tplr/compress.py:637-643,
 // for every parameter of the set at once).  Four codes per thread.
+// The statistical quantiser over each tensor's sent values (src/tplr/compress.py:582-621): one
+// workgroup per tensor makes the three passes of the reference - mean, norm of the centred values,
+// codes with per-bin means - over that tensor's part of the flat payload.  Sums are carried in
+// double and rounded once, where the reference's fp32 reductions round on the way.
+__device__ __forceinline__ double block_sum_f64(double x, double* part, int tid) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off);
+    __syncthreads();  // `part` may still be read from the previous call
+    if ((tid & 63) == 0) part[tid >> 6] = x;
+    __syncthreads();
+    double s = 0.0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) s += part[w];
+    return s;
+}
+
+__global__ __launch_bounds__(1024) void k_quantize_batch(const float* __restrict__ val, int k,
+                                                          const tplr_tensor_desc* __restrict__ table, int n_bins,
+                                                          float range_in_sigmas, uint8_t* __restrict__ codes,
+                                                          float* __restrict__ shift_out, float* __restrict__ scale_out,
+                                                          float* __restrict__ lookup) {
+    __shared__ double part[16];
+    __shared__ double bin_sum[256];
+    __shared__ unsigned int bin_cnt[256];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const tplr_tensor_desc d = table[t];
+    const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks * k;  // k is a multiple of 4
+    const float* v = val + d.chunk_begin * k;
+    uint8_t* q = codes + d.chunk_begin * k;
+    const int64_t n4 = n >> 2;
+    double acc = 0.0;
+    for (int64_t i = tid; i < n4; i += 1024) {
+        const float4 x = reinterpret_cast<const float4*>(v)[i];
+        acc += (static_cast<double>(x.x) + x.y) + (static_cast<double>(x.z) + x.w);
+    }
+    const float shift = static_cast<float>(block_sum_f64(acc, part, tid) / static_cast<double>(n));  // :594
+    acc = 0.0;
+    for (int64_t i = tid; i < n4; i += 1024) {
+        const float4 x = reinterpret_cast<const float4*>(v)[i];
+        const float a = x.x - shift, b = x.y - shift, c = x.z - shift, e = x.w - shift;  // :595
+        acc += (static_cast<double>(a) * a + static_cast<double>(b) * b) +
+               (static_cast<double>(c) * c + static_cast<double>(e) * e);
+    }
+    const double ss = block_sum_f64(acc, part, tid);
+    const float sd = static_cast<float>(sqrt(ss) / sqrt(static_cast<double>(n - 1)));  // :597
+    float scale = range_in_sigmas * sd / static_cast<float>(n_bins);                    // :598
+    if (scale == 0.f || scale != scale || __builtin_isinf(scale)) scale = 1.0f;         // :599-600
+    const float offset = static_cast<float>(n_bins / 2), top = static_cast<float>(n_bins - 1);
+    auto code = [&](float x, float& c) {
+        c = x - shift;
+        float r = __builtin_rintf(c / scale + offset);  // :604-605, ties to even as torch.round
+        r = r < 0.f ? 0.f : r;
+        r = r > top ? top : r;                          // :606
+        return static_cast<uint32_t>(r);
+    };
+    if (n_bins <= 8) {
+        // a handful of bins (templar runs four): per-thread sums, no contended atomics
+        double s8[8], c8[8];
+#pragma unroll
+        for (int b = 0; b < 8; ++b) s8[b] = c8[b] = 0.0;
+        auto tally = [&](uint32_t qq, float c) {
+#pragma unroll
+            for (int b = 0; b < 8; ++b) {
+                s8[b] += qq == static_cast<uint32_t>(b) ? static_cast<double>(c) : 0.0;  // :614-617
+                c8[b] += qq == static_cast<uint32_t>(b) ? 1.0 : 0.0;
+            }
+        };
+        for (int64_t i = tid; i < n4; i += 1024) {
+            const float4 x = reinterpret_cast<const float4*>(v)[i];
+            float c0, c1, c2, c3;
+            const uint32_t q0 = code(x.x, c0), q1 = code(x.y, c1), q2 = code(x.z, c2), q3 = code(x.w, c3);
+            reinterpret_cast<uchar4*>(q)[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
+                                                          static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
+            tally(q0, c0), tally(q1, c1), tally(q2, c2), tally(q3, c3);
+        }
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const double sum = block_sum_f64(s8[b], part, tid), cnt = block_sum_f64(c8[b], part, tid);
+            if (tid == 0 && b < n_bins)
+                lookup[static_cast<int64_t>(t) * n_bins + b] = cnt > 0.0 ? static_cast<float>(sum / cnt) : 0.f;  // :619
+        }
+    } else {
+        if (tid < 256) bin_sum[tid] = 0.0, bin_cnt[tid] = 0u;
+        __syncthreads();
+        for (int64_t i = tid; i < n4; i += 1024) {
+            const float4 x = reinterpret_cast<const float4*>(v)[i];
+            float c0, c1, c2, c3;
+            const uint32_t q0 = code(x.x, c0), q1 = code(x.y, c1), q2 = code(x.z, c2), q3 = code(x.w, c3);
+            reinterpret_cast<uchar4*>(q)[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
+                                                          static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
+            atomicAdd(&bin_sum[q0], static_cast<double>(c0)), atomicAdd(&bin_cnt[q0], 1u);  // :614-617
+            atomicAdd(&bin_sum[q1], static_cast<double>(c1)), atomicAdd(&bin_cnt[q1], 1u);
+            atomicAdd(&bin_sum[q2], static_cast<double>(c2)), atomicAdd(&bin_cnt[q2], 1u);
+            atomicAdd(&bin_sum[q3], static_cast<double>(c3)), atomicAdd(&bin_cnt[q3], 1u);
+        }
+        __syncthreads();
+        if (tid < n_bins)
+            lookup[static_cast<int64_t>(t) * n_bins + tid] =
+                bin_cnt[tid] ? static_cast<float>(bin_sum[tid] / static_cast<double>(bin_cnt[tid])) : 0.f;  // :619
+    }
+    if (tid == 0) shift_out[t] = shift, scale_out[t] = scale;
+}
+
 __global__ __launch_bounds__(256) void k_dequantize_batch(const uint8_t* __restrict__ q,
                                                           const float* __restrict__ lookup,
                                                           const float* __restrict__ shift, int n_bins, int k,
@@ -1827,6 +1930,19 @@ int tplr_index_stats_batch(const uint8_t* const* h_idx12, int n_peers, int k, co
         launch(k_index_stats<1>, resident[1]);
     else
         launch(k_index_stats<0>, resident[0]);
+    return launch_status();
+}
+
+int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
+                        float range_in_sigmas, uint8_t* d_codes, float* d_shift, float* d_scale, float* d_lookup,
+                        void* stream) {
+    if (!d_val || !d_desc || !d_codes || !d_shift || !d_scale || !d_lookup || n_tensors < 1 || k < 4 || (k & 3) ||
+        n_bins < 1 || n_bins > 256)
+        return TPLR_E_BADARG;
+    if ((reinterpret_cast<uintptr_t>(d_val) & 15) || (reinterpret_cast<uintptr_t>(d_codes) & 3)) return TPLR_E_BADARG;
+    hipLaunchKernelGGL(k_quantize_batch, dim3(static_cast<unsigned>(n_tensors)), dim3(1024), 0,
+                       static_cast<hipStream_t>(stream), d_val, k, d_desc, n_bins, range_in_sigmas, d_codes, d_shift,
+                       d_scale, d_lookup);
     return launch_status();
 }
 

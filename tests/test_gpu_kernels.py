@@ -645,6 +645,71 @@ def test_index_stats_every_row_length_and_peer_count(dev, P, k):
         b0 += cnt
 
 
+@pytest.mark.parametrize("bins", [4, 256, 7])
+def test_quantize_batch_matches_oracle_per_parameter(dev, bins):
+    # one launch over a flat payload against the oracle's quantiser (reference :582-621) run per parameter;
+    # both carry their sums in double, so shift, scale, codes and bin means agree to the last bit
+    rng = np.random.default_rng(77 + bins)
+    shapes = [(128, 64), (64, 192), (1024, 512), (64, 64), (192, 128)]
+    k = 32
+    batch = tc.TensorBatch([torch.zeros(s, device=dev) for s in shapes])
+    parts = []
+    for i, s in enumerate(shapes):
+        rows = (s[0] // 64) * (s[1] // 64)
+        v = rng.standard_t(3, size=(rows, k)).astype(np.float32) * np.float32(10.0 ** (i - 3)) + np.float32(0.01 * i)
+        parts.append(v)
+    parts[3][:] = np.float32(0.25)  # a constant parameter: the scale falls back to 1
+    val = torch.from_numpy(np.concatenate(parts)).to(dev)
+    codes, shift, scale, lookup = tc.quantize_batch(batch, val, k, bins, 6.0)
+    assert codes.shape == (batch.total_chunks, k) and codes.dtype == torch.uint8 and lookup.shape == (len(shapes), bins)
+    b0 = 0
+    for i, v in enumerate(parts):
+        q, (sh, sc, half, lut) = orc.quantize(v, bins, 6.0)
+        assert half == bins // 2
+        assert float(shift[i]) == sh and float(scale[i]) == sc, (i, float(shift[i]), sh, float(scale[i]), sc)
+        got_q = codes[b0:b0 + v.shape[0]].cpu().numpy()
+        assert np.array_equal(got_q, q), (i, int((got_q != q).sum()))
+        assert np.allclose(lookup[i].cpu().numpy(), lut, rtol=1e-6, atol=0)
+        b0 += v.shape[0]
+    assert float(scale[3]) == 1.0
+    # what the receiving side rebuilds from it: lookup[code] + shift, per parameter
+    back = tc.dequantize_batch(batch, codes.reshape(-1), [(shift[i], float(scale[i]), bins // 2, lookup[i], torch.float32)
+                                                          for i in range(len(shapes))], k)
+    b0 = 0
+    for i, v in enumerate(parts):
+        q, qp = orc.quantize(v, bins, 6.0)
+        want = orc.dequantize(q, qp)
+        got = back[b0:b0 + v.shape[0]].cpu().numpy()
+        assert np.abs(got - want).max() <= 1e-6 * max(np.abs(want).max(), 1e-30)
+        b0 += v.shape[0]
+
+
+@pytest.mark.parametrize("bins", [4, 256])
+def test_compressor_quantiser_on_the_device_matches_oracle(dev, bins):
+    # TopKCompressor._quantize_values on device tensors (one launch) against the oracle, then through
+    # compress -> decompress as the callers use it (src/tplr/neurons.py:157-166)
+    comp = tc.TopKCompressor(use_quantization=True, quantization_bins=bins, quantization_range=6)
+    rng = np.random.default_rng(5 + bins)
+    for shape in [(2, 3, 32), (7, 64), (1, 4), (33, 1, 12)]:
+        v = (rng.standard_normal(shape) * 0.02 + 0.003).astype(np.float32)
+        q, (shift, scale, half, lut, dt) = comp._quantize_values(torch.from_numpy(v).to(dev))
+        wq, (wshift, wscale, whalf, wlut) = orc.quantize(v, bins, 6.0)
+        assert q.shape == v.shape and q.dtype == torch.uint8 and isinstance(scale, float) and dt == torch.float32
+        assert float(shift) == wshift and scale == wscale and half == whalf
+        assert np.array_equal(q.cpu().numpy(), wq) and np.allclose(lut.cpu().numpy(), wlut, rtol=1e-6, atol=0)
+        back = comp._dequantize_values(q, (shift, scale, half, lut, dt))
+        assert np.array_equal(back.cpu().numpy(), orc.dequantize(wq, (wshift, wscale, whalf, lut.cpu().numpy())))
+    x = t3((128, 192), 404, row_scale=True).to(dev)
+    enc = tc.ChunkingTransformer(_Stub([torch.empty(128, 192)]), 64).encode(x, use_dct=True)
+    idx, qv, xshape, totalk, qp = comp.compress(enc, 32)
+    dense = comp.decompress(x, idx, qv, xshape, totalk, qp)
+    i2, v2, _, _ = tc.TopKCompressor().compress(enc, 32)
+    wq, wqp = orc.quantize(v2.cpu().numpy(), bins, 6.0)
+    want = orc.decompress(i2.cpu().numpy(), orc.dequantize(wq, wqp), xshape, totalk)
+    assert torch.equal(i2, idx) and np.array_equal(qv.cpu().numpy(), wq)
+    assert np.abs(dense.cpu().numpy() - want).max() <= 1e-6 * np.abs(want).max()
+
+
 def test_dequantize_batch_matches_per_parameter_reference_path(dev):
     rng = np.random.default_rng(31)
     shapes = [(128, 64), (64, 192), (192, 128)]
