@@ -169,6 +169,21 @@ __device__ __forceinline__ uint32_t stat_threshold(uint32_t b1, uint32_t b2, int
     return t;
 }
 
+// The larger of the two thresholds that two sets of lane statistics give (rows and columns of an
+// untransformed chunk), in one search: a candidate passes when either set has k entries at or
+// above it.
+template <bool kTwo>
+__device__ __forceinline__ uint32_t stat_threshold_either(uint32_t b1, uint32_t b2, uint32_t c1, uint32_t c2, int k) {
+    uint32_t t = 0;
+    for (int bit = 30; bit >= 0; --bit) {
+        const uint32_t c = t | (1u << bit);
+        int nb = __popcll(__ballot(b1 >= c)), nc = __popcll(__ballot(c1 >= c));
+        if (kTwo) nb += __popcll(__ballot(b2 >= c)), nc += __popcll(__ballot(c2 >= c));
+        if (nb >= k || nc >= k) t = c;
+    }
+    return t;
+}
+
 // 64-bit per-lane mask (hi: d = 0..31 at bits 31..0, lo: d = 32..63) of the values that are
 // not below the float threshold.  A superset is fine here, so NaN and any denormal-flush
 // behaviour of the compare only add candidates.
@@ -355,18 +370,17 @@ __device__ __forceinline__ void sort128_desc(uint64_t& e0, uint64_t& e1, int) { 
 // `out_scale` multiplies the gathered values (an exact power of two left over by the caller's
 // transform; the ordering is taken on the unscaled values).
 // `buf` is a kHalfFloats staging buffer, `cand` kCandCap slots; both are free on return.
-// `t_floor` (magnitude bits, wave-uniform, 0 = none) is another lower bound of the k-th largest
-// magnitude that the caller knows, e.g. the same statistic taken over the columns: data whose
-// rows differ in scale put most candidates into a few lanes and pass far too many of them.
-template <bool kTwo>
+// kOther: `o1`, `o2` are a second set of lane statistics of the same chunk, e.g. taken over the
+// columns: data whose rows differ in scale put most candidates into a few lanes and one direction
+// alone passes far too many of them; the threshold is then the larger of the two directions'.
+template <bool kTwo, bool kOther = false>
 __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf, uint64_t* cand, int lane, int k,
-                                                float out_scale, uint32_t t_floor = 0) {
+                                                float out_scale, uint32_t o1 = 0, uint32_t o2 = 0) {
     uint32_t mhi = 0, mlo = 0, cnt = 0, incl = 0, total = 0;
     {
         uint32_t b1, b2;
         lane_stats<kTwo>(w, b1, b2);
-        const uint32_t t_rows = stat_threshold<kTwo>(b1, b2, k);
-        const uint32_t t0 = t_rows > t_floor ? t_rows : t_floor;
+        const uint32_t t0 = kOther ? stat_threshold_either<kTwo>(b1, b2, o1, o2, k) : stat_threshold<kTwo>(b1, b2, k);
         filter_masks(w, __uint_as_float(t0), mhi, mlo);
         cnt = __popc(mhi) + __popc(mlo);
         incl = wave_incl_scan_u32(cnt);

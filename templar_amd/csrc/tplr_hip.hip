@@ -438,14 +438,11 @@ __global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_de
         // Untransformed gradients often differ in scale from row to row or column to column;
         // the select's threshold statistic is then taken in both directions.  (Coefficients of
         // the transform are mixed across both and one direction is as good as two.)
-        uint32_t t_cols = 0;
-        if (!kUseDct) {
-            uint32_t c1, c2;
-            lane_stats<kTwo>(v, c1, c2);
-            t_cols = stat_threshold<kTwo>(c1, c2, k);
-        }
+        uint32_t c1 = 0, c2 = 0;
+        if (!kUseDct) lane_stats<kTwo>(v, c1, c2);
         chunk_forward<kUseDct>(v, w, buf, lane);
-        const Selected s = select_topk<kTwo>(w, buf, cand, lane, k, kUseDct ? kDctPow2Scale : 1.0f, t_cols);
+        const Selected s =
+            select_topk<kTwo, !kUseDct>(w, buf, cand, lane, k, kUseDct ? kDctPow2Scale : 1.0f, c1, c2);
         emit_selected(s, lane, k, g, idx12, val);
     }
 }
