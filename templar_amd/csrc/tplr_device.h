@@ -301,9 +301,30 @@ __device__ __forceinline__ void keep_first(uint32_t& hi, uint32_t& lo, int keep)
     lo = l;
 }
 
-__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t x, int j) {
-    const uint32_t lo = __shfl_xor(static_cast<uint32_t>(x), j);
-    const uint32_t hi = __shfl_xor(static_cast<uint32_t>(x >> 32), j);
+// x of lane ^ J.  Distances below 16 stay inside a row of 16 lanes and are data-parallel moves
+// (no trip through the LDS crossbar, whose queue the sort would otherwise fill); 16 and 32 cross rows.
+template <int J>
+__device__ __forceinline__ uint32_t lane_xor_u32(uint32_t x) {
+    const int v = static_cast<int>(x);
+    if constexpr (J == 1) {
+        return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false));  // quad_perm:[1,0,3,2]
+    } else if constexpr (J == 2) {
+        return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false));  // quad_perm:[2,3,0,1]
+    } else if constexpr (J == 4) {
+        // lanes 0-3 and 8-11 of a row take lane + 4, lanes 4-7 and 12-15 take lane - 4
+        const int t = __builtin_amdgcn_update_dpp(v, v, 0x104, 0xf, 0x5, false);                 // row_shl:4
+        return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(t, v, 0x114, 0xf, 0xa, false));  // row_shr:4
+    } else if constexpr (J == 8) {
+        return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(v, v, 0x128, 0xf, 0xf, false));  // row_ror:8
+    } else {
+        return static_cast<uint32_t>(__shfl_xor(v, J));
+    }
+}
+
+template <int J>
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t x) {
+    const uint32_t lo = lane_xor_u32<J>(static_cast<uint32_t>(x));
+    const uint32_t hi = lane_xor_u32<J>(static_cast<uint32_t>(x >> 32));
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
@@ -330,7 +351,9 @@ __device__ __forceinline__ uint64_t cmp_exchange(uint64_t e, uint64_t o, uint64_
         : "scc");
     uint32_t lo, hi;
     asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(lo) : "v"(static_cast<uint32_t>(e)), "v"(static_cast<uint32_t>(o)), "s"(take));
-    asm("v_cndmask_b32_e64 %0, %1, %2, %3"
+    // (the next stage may read the result with a data-parallel move, which must stay two instructions
+    // behind the vector write of its source; the compiler does not see the write inside the assembly)
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3\n\ts_nop 1"
         : "=v"(hi)
         : "v"(static_cast<uint32_t>(e >> 32)), "v"(static_cast<uint32_t>(o >> 32)), "s"(take));
     return (static_cast<uint64_t>(hi) << 32) | lo;
@@ -339,7 +362,7 @@ __device__ __forceinline__ uint64_t cmp_exchange(uint64_t e, uint64_t o, uint64_
 // bitonic sort, descending, of 64 (one per lane) or 128 (two per lane) keys
 template <int K2, int J>
 __device__ __forceinline__ void sort64_step(uint64_t& e) {
-    e = cmp_exchange(e, shfl_xor_u64(e, J), keepmax_mask(K2, J, 0));
+    e = cmp_exchange(e, shfl_xor_u64<J>(e), keepmax_mask(K2, J, 0));
     if constexpr (J > 1)
         sort64_step<K2, J / 2>(e);
     else if constexpr (K2 < 64)
@@ -356,8 +379,8 @@ __device__ __forceinline__ void sort128_step(uint64_t& e0, uint64_t& e1) {
         e0 = a;
         e1 = b;
     } else {
-        e0 = cmp_exchange(e0, shfl_xor_u64(e0, J), keepmax_mask(K2, J, 0));
-        e1 = cmp_exchange(e1, shfl_xor_u64(e1, J), keepmax_mask(K2, J, 64));
+        e0 = cmp_exchange(e0, shfl_xor_u64<J>(e0), keepmax_mask(K2, J, 0));
+        e1 = cmp_exchange(e1, shfl_xor_u64<J>(e1), keepmax_mask(K2, J, 64));
     }
     if constexpr (J > 1)
         sort128_step<K2, J / 2>(e0, e1);
