@@ -957,7 +957,7 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
             st = lib.tplr_ef_encode_topk_pack_batch(_ptr(ef.table), _ptr(grad.table), len(ef), n, C.c_float(decay), k,
                                                     int(use_dct), _ptr(idx12), _ptr(val), _stream(dev))
     _lib.check(st, "tplr_ef_encode_topk_pack_batch")
-    quant, sent = None, val
+    quant, sent, codes = None, val, None
     if compressor is not None and compressor.use_quantization:
         codes, shift, scale, lookup = quantize_batch(ef, val, k, compressor.n_bins, compressor.range_in_sigmas)
         sent = torch.empty_like(val)
@@ -965,17 +965,27 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
             st = lib.tplr_dequantize_batch(_ptr(codes), _ptr(lookup), _ptr(shift), compressor.n_bins, k, _ptr(ef.table),
                                            len(ef), n, _ptr(sent), _stream(dev))
         _lib.check(st, "tplr_dequantize_batch")
-        scales = scale.tolist()  # the reference's quant_params carry the scale as a Python float (:620)
-        quant = []
-        for i in range(len(ef)):
-            y, x, _, _ = ef.xshape(i)
-            b = ef.offsets[i]
-            quant.append((codes[b:b + y * x].reshape(y, x, k),
-                          (shift[i], scales[i], compressor.n_bins // 2, lookup[i], torch.float32)))
+        # the reference's quant_params carry the scale as a Python float (:620): the copy to the host
+        # is queued here and read after the subtraction has been launched
+        with _on(dev):
+            scale_host = torch.empty(len(ef), dtype=torch.float32, pin_memory=True)
+            scale_host.copy_(scale, non_blocking=True)
+            copied = torch.cuda.Event()
+            copied.record()
     with _on(dev):
         st = lib.tplr_ef_subtract_batch(_ptr(idx12), _ptr(sent), k, _ptr(ef.table), len(ef), n, int(use_dct),
                                         _stream(dev))
     _lib.check(st, "tplr_ef_subtract_batch")
+    if codes is not None:
+        # the per-parameter form of the reference's compress output
+        parts = []
+        for i in range(len(ef)):
+            y, x, _, _ = ef.xshape(i)
+            b = ef.offsets[i]
+            parts.append((codes[b:b + y * x].view(y, x, k), shift[i], lookup[i]))
+        copied.synchronize()
+        half = compressor.n_bins // 2
+        quant = [(q, (sh, sc, half, lut, torch.float32)) for (q, sh, lut), sc in zip(parts, scale_host.tolist())]
     return idx12, val, quant
 
 

@@ -1176,19 +1176,31 @@ __global__ __launch_bounds__(1024) void k_quantize_batch(const float* __restrict
     const float* v = val + d.chunk_begin * k;
     uint8_t* q = codes + d.chunk_begin * k;
     const int64_t n4 = n >> 2;
+    // every pass walks the tensor four float4 per thread at a time, so that four loads are in flight
+    const float4* v4 = reinterpret_cast<const float4*>(v);
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto walk = [&](auto&& body) {
+        for (int64_t i = tid; i < n4; i += 4096) {
+            const bool h1 = i + 1024 < n4, h2 = i + 2048 < n4, h3 = i + 3072 < n4;
+            const float4 x0 = v4[i];
+            const float4 x1 = h1 ? v4[i + 1024] : zero4;
+            const float4 x2 = h2 ? v4[i + 2048] : zero4;
+            const float4 x3 = h3 ? v4[i + 3072] : zero4;
+            body(i, x0);
+            if (h1) body(i + 1024, x1);
+            if (h2) body(i + 2048, x2);
+            if (h3) body(i + 3072, x3);
+        }
+    };
     double acc = 0.0;
-    for (int64_t i = tid; i < n4; i += 1024) {
-        const float4 x = reinterpret_cast<const float4*>(v)[i];
-        acc += (static_cast<double>(x.x) + x.y) + (static_cast<double>(x.z) + x.w);
-    }
+    walk([&](int64_t, const float4& x) { acc += (static_cast<double>(x.x) + x.y) + (static_cast<double>(x.z) + x.w); });
     const float shift = static_cast<float>(block_sum_f64(acc, part, tid) / static_cast<double>(n));  // :594
     acc = 0.0;
-    for (int64_t i = tid; i < n4; i += 1024) {
-        const float4 x = reinterpret_cast<const float4*>(v)[i];
+    walk([&](int64_t, const float4& x) {
         const float a = x.x - shift, b = x.y - shift, c = x.z - shift, e = x.w - shift;  // :595
         acc += (static_cast<double>(a) * a + static_cast<double>(b) * b) +
                (static_cast<double>(c) * c + static_cast<double>(e) * e);
-    }
+    });
     const double ss = block_sum_f64(acc, part, tid);
     const float sd = static_cast<float>(sqrt(ss) / sqrt(static_cast<double>(n - 1)));  // :597
     float scale = range_in_sigmas * sd / static_cast<float>(n_bins);                    // :598
@@ -1201,6 +1213,7 @@ __global__ __launch_bounds__(1024) void k_quantize_batch(const float* __restrict
         r = r > top ? top : r;                          // :606
         return static_cast<uint32_t>(r);
     };
+    uchar4* q4 = reinterpret_cast<uchar4*>(q);
     if (n_bins <= 8) {
         // a handful of bins (templar runs four): per-thread sums, no contended atomics
         double s8[8], c8[8];
@@ -1213,14 +1226,13 @@ __global__ __launch_bounds__(1024) void k_quantize_batch(const float* __restrict
                 c8[b] += qq == static_cast<uint32_t>(b) ? 1.0 : 0.0;
             }
         };
-        for (int64_t i = tid; i < n4; i += 1024) {
-            const float4 x = reinterpret_cast<const float4*>(v)[i];
+        walk([&](int64_t i, const float4& x) {
             float c0, c1, c2, c3;
             const uint32_t q0 = code(x.x, c0), q1 = code(x.y, c1), q2 = code(x.z, c2), q3 = code(x.w, c3);
-            reinterpret_cast<uchar4*>(q)[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
-                                                          static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
+            q4[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
+                                static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
             tally(q0, c0), tally(q1, c1), tally(q2, c2), tally(q3, c3);
-        }
+        });
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
             const double sum = block_sum_f64(s8[b], part, tid), cnt = block_sum_f64(c8[b], part, tid);
@@ -1230,17 +1242,16 @@ __global__ __launch_bounds__(1024) void k_quantize_batch(const float* __restrict
     } else {
         if (tid < 256) bin_sum[tid] = 0.0, bin_cnt[tid] = 0u;
         __syncthreads();
-        for (int64_t i = tid; i < n4; i += 1024) {
-            const float4 x = reinterpret_cast<const float4*>(v)[i];
+        walk([&](int64_t i, const float4& x) {
             float c0, c1, c2, c3;
             const uint32_t q0 = code(x.x, c0), q1 = code(x.y, c1), q2 = code(x.z, c2), q3 = code(x.w, c3);
-            reinterpret_cast<uchar4*>(q)[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
-                                                          static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
+            q4[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
+                                static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
             atomicAdd(&bin_sum[q0], static_cast<double>(c0)), atomicAdd(&bin_cnt[q0], 1u);  // :614-617
             atomicAdd(&bin_sum[q1], static_cast<double>(c1)), atomicAdd(&bin_cnt[q1], 1u);
             atomicAdd(&bin_sum[q2], static_cast<double>(c2)), atomicAdd(&bin_cnt[q2], 1u);
             atomicAdd(&bin_sum[q3], static_cast<double>(c3)), atomicAdd(&bin_cnt[q3], 1u);
-        }
+        });
         __syncthreads();
         if (tid < n_bins)
             lookup[static_cast<int64_t>(t) * n_bins + tid] =
