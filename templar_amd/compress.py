@@ -1028,8 +1028,16 @@ def _qparam_tables(qparams: Sequence[QuantParamsT], dev: torch.device) -> tuple[
     """(rows, n_bins) lookups and (rows,) shifts of a list of quant_params 5-tuples on `dev`: stacked
     where they live, moved once."""
     n_bins = int(qparams[0][3].numel())
-    lookup = torch.stack([qp[3].reshape(n_bins).float() for qp in qparams])
-    shift = torch.stack([torch.as_tensor(qp[0], dtype=torch.float32, device=lookup.device).reshape(()) for qp in qparams])
+    try:  # the usual case: every lookup a flat fp32 tensor, every shift a 0-dim fp32 tensor, one device
+        lookup = torch.stack([qp[3] for qp in qparams])
+        shift = torch.stack([qp[0] for qp in qparams])
+        if lookup.dtype != torch.float32 or shift.dtype != torch.float32 or lookup.shape != (len(qparams), n_bins) \
+                or shift.shape != (len(qparams),):
+            raise TypeError
+    except (TypeError, RuntimeError):
+        lookup = torch.stack([qp[3].reshape(n_bins).float() for qp in qparams])
+        shift = torch.stack([torch.as_tensor(qp[0], dtype=torch.float32, device=lookup.device).reshape(())
+                             for qp in qparams])
     return lookup.to(dev).contiguous(), shift.to(dev).contiguous(), n_bins
 
 
@@ -1090,7 +1098,8 @@ class PayloadStage:
 
     _ALIGN = 256
 
-    def __init__(self, batch: TensorBatch, k: int, max_peers: int, *, quantized: bool = True):
+    def __init__(self, batch: TensorBatch, k: int, max_peers: int, *, quantized: bool = True,
+                 host_threads: int | None = None):
         if max_peers < 1 or max_peers > _lib.TPLR_MAX_PEERS:
             raise ValueError(f"max_peers must be in [1, {_lib.TPLR_MAX_PEERS}]")
         if k < 2 or k % 2:
@@ -1106,7 +1115,9 @@ class PayloadStage:
         self.dev = torch.empty(max_peers * self.stride, dtype=torch.uint8, device=batch.device)
         self.values = torch.empty((max_peers, n, k), dtype=torch.float32, device=batch.device) if quantized else None
         self._copied: torch.cuda.Event | None = None  # the last host-to-device copy out of `host`
-        self._threads = max(1, min(8, os.cpu_count() or 1))
+        self._val_sizes = [batch.xshape(i)[0] * batch.xshape(i)[1] * k for i in range(len(batch))]
+        self._idx_sizes = [v // 2 * 3 for v in self._val_sizes]
+        self._threads = max(1, min(64, host_threads if host_threads else min(8, os.cpu_count() or 1)))
 
     def _regions(self, buf: torch.Tensor, p: int) -> tuple[torch.Tensor, torch.Tensor]:
         b = p * self.stride
@@ -1129,19 +1140,23 @@ class PayloadStage:
         if P < 1 or P > self.max_peers:
             raise ValueError(f"{P} peers for a stage of {self.max_peers}")
         want_dtype = torch.uint8 if self.quantized else torch.float32
-        for i in range(T):
-            y, x, _, _ = self.batch.xshape(i)
-            if len(idxs[i]) != P or len(vals[i]) != P:
-                raise IndexError(f"parameter {i}: {len(idxs[i])} index / {len(vals[i])} value entries for {P} peers")
-            for p in range(P):
-                a, v = idxs[i][p], vals[i][p]
+        for p in range(P):  # sizes and types of all tensors of a peer, compared as lists
+            try:
+                pi, pv = [row[p] for row in idxs], [row[p] for row in vals]
+            except IndexError:
+                raise IndexError(f"every parameter needs {P} index and value entries") from None
+            if [a.numel() for a in pi] != self._idx_sizes or [v.numel() for v in pv] != self._val_sizes:
+                bad = next(i for i in range(T) if pi[i].numel() != self._idx_sizes[i] or pv[i].numel() != self._val_sizes[i])
+                raise RuntimeError(f"parameter {bad}, peer {p}: {pi[bad].numel()} index bytes / {pv[bad].numel()} values for "
+                                   f"{self._val_sizes[bad] // self.k} chunks of k={self.k}")
+            for a in pi:
                 if a.dtype != torch.uint8:
                     raise ValueError(f"Expected uint8 for 12-bit packed indices, got {a.dtype}")
+            for v in pv:
                 if v.dtype != want_dtype:
-                    raise ValueError(f"parameter {i}, peer {p}: values are {v.dtype}, the stage holds {want_dtype}")
-                if v.numel() != y * x * self.k or a.numel() * 2 != v.numel() * 3:
-                    raise RuntimeError(f"parameter {i}, peer {p}: {a.numel()} index bytes / {v.numel()} values for "
-                                       f"{y * x} chunks of k={self.k}")
+                    raise ValueError(f"peer {p}: values are {v.dtype}, the stage holds {want_dtype}")
+        if any(len(row) != P for row in idxs) or any(len(row) != P for row in vals):
+            raise IndexError(f"every parameter needs {P} index and value entries")
         on_host = idxs[0][0].device.type == "cpu"
         if on_host and self._copied is not None:
             self._copied.synchronize()  # the previous window's copy still reads the pinned buffer
