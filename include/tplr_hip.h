@@ -252,6 +252,14 @@ int tplr_dequantize_batch(const uint8_t* d_codes, const float* d_lookup, const f
                           const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_rows, float* d_val,
                           void* stream);
 
+/* The same arithmetic for ONE parameter's codes from n_peers peers, every peer with its own
+ * lookup (d_lookup: n_peers x n_bins) and shift (d_shift: n_peers): the loop of
+ * maybe_dequantize_values (src/tplr/compress.py:668-690) as it is called per parameter in
+ * src/tplr/neurons.py:325, in one launch.  h_codes / h_out: host arrays of n_peers device pointers
+ * (n codes in, n floats out, each; codes 4-byte and outputs 16-byte aligned).  n a multiple of 4. */
+int tplr_dequantize_peers(const uint8_t* const* h_codes, int n_peers, int64_t n, const float* d_lookup,
+                          const float* d_shift, int n_bins, float* const* h_out, void* stream);
+
 /* TopKCompressor._quantize_values (src/tplr/compress.py:582-621) for every parameter of a flat
  * payload in one launch (the reference runs it per parameter inside compress, :419-421): per
  * tensor t, shift = mean of its values, scale = range_in_sigmas * std / n_bins (1 when that is 0,

@@ -730,6 +730,38 @@ class TopKCompressor:
             lookup = lookup.to(val.device)
         return (lookup[val.long()] + shift).to(orig_dtype)
 
+    def _dequantize_peers(self, vals, qparams, device) -> list[torch.Tensor] | None:
+        """All peers' codes of one parameter in one launch, when they are plain: uint8 on one HIP device,
+        equal sizes (a multiple of 4), fp32 targets, a 5-tuple for every peer.  None otherwise."""
+        P = len(vals)
+        dev = torch.device(device)
+        if dev.type != "cuda" or P == 0 or P > _lib.TPLR_MAX_PEERS or len(qparams) < P:
+            return None
+        if dev.index is None:
+            dev = torch.device("cuda", torch.cuda.current_device())
+        n = vals[0].numel()
+        if n == 0 or n % 4:
+            return None
+        vals = [v if v.device == dev else v.to(dev, non_blocking=True) for v in vals]
+        for v, qp in zip(vals, qparams):
+            if qp is None or len(qp) != 5 or qp[4] != torch.float32 or not isinstance(qp[3], torch.Tensor) \
+                    or v.numel() != n or v.device != dev or not v.is_contiguous():
+                return None
+        try:
+            lookup, shift, n_bins = _qparam_tables(qparams[:P], dev)
+        except (RuntimeError, TypeError):
+            return None
+        if n_bins > 256:
+            return None
+        lib = _lib.load()
+        outs = [torch.empty(v.shape, dtype=torch.float32, device=dev) for v in vals]
+        cp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
+        op = (C.c_void_p * P)(*[o.data_ptr() for o in outs])
+        with _on(dev):
+            st = lib.tplr_dequantize_peers(cp, P, n, _ptr(lookup), _ptr(shift), n_bins, op, _stream(dev))
+        _lib.check(st, "tplr_dequantize_peers")
+        return outs
+
     def maybe_dequantize_values(self, vals: list[torch.Tensor], qparams: list[QuantParamsT],
                                 device: torch.device) -> list[torch.Tensor]:
         """Dequantise a list of per-peer values when all of them are uint8 (reference :646-696)."""
@@ -742,6 +774,9 @@ class TopKCompressor:
             qparams = [qparams]  # a single 5-tuple
         if not isinstance(qparams, list):
             qparams = [qparams]
+        fast = self._dequantize_peers(vals, qparams, device)
+        if fast is not None:
+            return fast
         out: list[torch.Tensor] = []
         for i, v in enumerate(vals):
             v = v.to(device)

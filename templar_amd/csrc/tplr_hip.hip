@@ -1941,6 +1941,54 @@ int tplr_index_stats_batch(const uint8_t* const* h_idx12, int n_peers, int k, co
     return launch_status();
 }
 
+struct DeqPtrs {
+    const uint8_t* codes[TPLR_MAX_PEERS];
+    float* out[TPLR_MAX_PEERS];
+};
+
+// One parameter's codes of P peers, each with its own lookup and shift: block row p serves peer p.
+__global__ __launch_bounds__(256) void k_dequantize_peers(const DeqPtrs pp, int64_t n4,
+                                                          const float* __restrict__ lookup,
+                                                          const float* __restrict__ shift, int n_bins) {
+    const int p = blockIdx.y;
+    const uchar4* q = reinterpret_cast<const uchar4*>(pp.codes[p]);
+    float4* o = reinterpret_cast<float4*>(pp.out[p]);
+    const float* lk = lookup + static_cast<int64_t>(p) * n_bins;
+    const float sh = shift[p];
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n4; i += stride) {
+        const uchar4 c = q[i];
+        float4 r;
+        r.x = lk[c.x < n_bins ? c.x : n_bins - 1] + sh;
+        r.y = lk[c.y < n_bins ? c.y : n_bins - 1] + sh;
+        r.z = lk[c.z < n_bins ? c.z : n_bins - 1] + sh;
+        r.w = lk[c.w < n_bins ? c.w : n_bins - 1] + sh;
+        o[i] = r;
+    }
+}
+
+int tplr_dequantize_peers(const uint8_t* const* h_codes, int n_peers, int64_t n, const float* d_lookup,
+                          const float* d_shift, int n_bins, float* const* h_out, void* stream) {
+    if (!h_codes || !h_out || !d_lookup || !d_shift || n_peers < 1 || n < 0 || (n & 3) || n_bins < 1 || n_bins > 256)
+        return TPLR_E_BADARG;
+    if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
+    if (n == 0) return 0;
+    DeqPtrs pp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        pp.codes[p] = p < n_peers ? h_codes[p] : nullptr;
+        pp.out[p] = p < n_peers ? h_out[p] : nullptr;
+        if (p < n_peers && (!pp.codes[p] || !pp.out[p] || (reinterpret_cast<uintptr_t>(pp.codes[p]) & 3) ||
+                            (reinterpret_cast<uintptr_t>(pp.out[p]) & 15)))
+            return TPLR_E_BADARG;
+    }
+    const int64_t n4 = n >> 2;
+    int64_t bx = (n4 + 255) / 256;
+    bx = bx > 2048 ? 2048 : bx;
+    hipLaunchKernelGGL(k_dequantize_peers, dim3(static_cast<unsigned>(bx), static_cast<unsigned>(n_peers)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), pp, n4, d_lookup, d_shift, n_bins);
+    return launch_status();
+}
+
 int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
                         float range_in_sigmas, uint8_t* d_codes, float* d_shift, float* d_scale, float* d_lookup,
                         void* stream) {

@@ -710,6 +710,35 @@ def test_compressor_quantiser_on_the_device_matches_oracle(dev, bins):
     assert np.abs(dense.cpu().numpy() - want).max() <= 1e-6 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("bins", [4, 256])
+def test_maybe_dequantize_values_one_launch_for_all_peers(dev, bins):
+    # src/tplr/neurons.py:325: one parameter's uint8 values of P peers with their quant_params
+    comp = tc.TopKCompressor(use_quantization=True, quantization_bins=bins, quantization_range=6)
+    rng = np.random.default_rng(9 + bins)
+    P, shape = 7, (3, 5, 32)
+    host, codes, qps = [], [], []
+    for p in range(P):
+        v = (rng.standard_normal(shape) * (p + 1) * 1e-3 + 1e-4 * p).astype(np.float32)
+        q, qp = orc.quantize(v, bins, 6.0)
+        host.append((q, qp))
+        codes.append(torch.from_numpy(q).to(dev))
+        qps.append((torch.tensor(qp[0], device=dev), qp[1], qp[2], torch.from_numpy(qp[3]).to(dev), torch.float32))
+    out = comp.maybe_dequantize_values(codes, qps, dev)
+    assert len(out) == P
+    for p in range(P):
+        assert out[p].dtype == torch.float32 and out[p].shape == shape
+        assert np.array_equal(out[p].cpu().numpy(), orc.dequantize(*host[p]))
+        assert torch.equal(out[p], comp._dequantize_values(codes[p], qps[p]))
+    # payloads still on the host, and shapes the one-launch form does not take: same results
+    out_h = comp.maybe_dequantize_values([c.cpu() for c in codes], [(a.cpu(), b, c, d.cpu(), e) for a, b, c, d, e in qps], dev)
+    assert all(torch.equal(a, b) and a.device == out[0].device for a, b in zip(out_h, out))
+    odd = [c.reshape(-1)[:30] for c in codes]  # 30 codes: not a multiple of 4
+    out_o = comp.maybe_dequantize_values(odd, qps, dev)
+    assert all(torch.equal(a, b.reshape(-1)[:30]) for a, b in zip(out_o, out))
+    with pytest.raises(IndexError):
+        comp.maybe_dequantize_values(codes, qps[:-1] + [None], dev)
+
+
 def test_dequantize_batch_matches_per_parameter_reference_path(dev):
     rng = np.random.default_rng(31)
     shapes = [(128, 64), (64, 192), (192, 128)]
