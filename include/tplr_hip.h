@@ -261,15 +261,17 @@ int tplr_dequantize_peers(const uint8_t* const* h_codes, int n_peers, int64_t n,
                           const float* d_shift, int n_bins, float* const* h_out, void* stream);
 
 /* TopKCompressor._quantize_values (src/tplr/compress.py:582-621) for every parameter of a flat
- * payload in one launch (the reference runs it per parameter inside compress, :419-421): per
- * tensor t, shift = mean of its values, scale = range_in_sigmas * std / n_bins (1 when that is 0,
- * NaN or infinite), d_codes[i] = clamp(round_half_even((v - shift) / scale + n_bins / 2), 0,
- * n_bins - 1), d_lookup[t * n_bins + b] = mean of the centred values coded b (0 for an unused
- * bin).  Sums are carried in double.  d_shift, d_scale: n_tensors floats.  k a multiple of 4,
- * n_bins <= 256, d_val 16-byte aligned; d_desc as above (chunk_begin and chunk counts). */
+ * payload (the reference runs it per parameter inside compress, :419-421): per tensor t,
+ * shift = mean of its values, scale = range_in_sigmas * std / n_bins (1 when that is 0, NaN or
+ * infinite), d_codes[i] = clamp(round_half_even((v - shift) / scale + n_bins / 2), 0, n_bins - 1),
+ * d_lookup[t * n_bins + b] = mean of the centred values coded b (0 for an unused bin).  Four
+ * launches; every tensor is cut into n_slices (1..1024) runs of rows whose partial sums (double)
+ * pass through d_work: n_tensors * n_slices * (2 + 2 * n_bins) doubles, contents irrelevant on
+ * entry.  d_shift, d_scale: n_tensors floats.  k a multiple of 4, n_bins <= 256, d_val 16-byte
+ * aligned; d_desc as above (chunk_begin and chunk counts). */
 int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
-                        float range_in_sigmas, uint8_t* d_codes, float* d_shift, float* d_scale, float* d_lookup,
-                        void* stream);
+                        float range_in_sigmas, int n_slices, double* d_work, uint8_t* d_codes, float* d_shift,
+                        float* d_scale, float* d_lookup, void* stream);
 
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes
  * (a multiple of 16, both pointers 16-byte aligned) that moves exactly n_bytes each way.

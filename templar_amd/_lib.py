@@ -48,7 +48,7 @@ SIGNATURES = {
     "tplr_ef_subtract_batch": (_i32, [_vp, _vp, _i32, _vp, _i32, _i64, _i32, _vp]),
     "tplr_dequantize_batch": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp]),
     "tplr_dequantize_peers": (_i32, [_vp, _i32, _i64, _vp, _vp, _i32, _vp, _vp]),
-    "tplr_quantize_batch": (_i32, [_vp, _i32, _vp, _i32, _i32, C.c_float, _vp, _vp, _vp, _vp, _vp]),
+    "tplr_quantize_batch": (_i32, [_vp, _i32, _vp, _i32, _i32, C.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
     "tplr_index_stats_batch": (_i32, [_vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp, _vp, _vp]),
 }
 

@@ -701,10 +701,12 @@ class TopKCompressor:
             q = torch.empty(val.shape, dtype=torch.uint8, device=dev)
             stats = torch.empty(2, dtype=torch.float32, device=dev)
             lookup = torch.empty(self.n_bins, dtype=torch.float32, device=dev)
+            slices = max(1, min(256, n // 16384))
+            work = torch.empty(slices * (2 + 2 * self.n_bins), dtype=torch.float64, device=dev)
             with _on(dev):
                 st = lib.tplr_quantize_batch(_ptr(v), 4, _ptr(_flat_desc(n // 4, dev)), 1, self.n_bins,
-                                             C.c_float(self.range_in_sigmas), _ptr(q), _ptr(stats[0:1]), _ptr(stats[1:2]),
-                                             _ptr(lookup), _stream(dev))
+                                             C.c_float(self.range_in_sigmas), slices, _ptr(work), _ptr(q),
+                                             _ptr(stats[0:1]), _ptr(stats[1:2]), _ptr(lookup), _stream(dev))
             _lib.check(st, "tplr_quantize_batch")
             return q, (stats[0], float(stats[1]), half, lookup, val.dtype)
         shift = val.mean()
@@ -1089,9 +1091,11 @@ def quantize_batch(batch: TensorBatch, val: torch.Tensor, k: int, n_bins: int = 
     shift = torch.empty(T, dtype=torch.float32, device=dev)
     scale = torch.empty(T, dtype=torch.float32, device=dev)
     lookup = torch.empty((T, n_bins), dtype=torch.float32, device=dev)
+    slices = max(1, min(64, 2048 // T))  # enough workgroups to fill the device
+    work = torch.empty(T * slices * (2 + 2 * n_bins), dtype=torch.float64, device=dev)
     with _on(dev):
-        st = lib.tplr_quantize_batch(_ptr(val), k, _ptr(batch.table), T, n_bins, C.c_float(range_in_sigmas), _ptr(codes),
-                                     _ptr(shift), _ptr(scale), _ptr(lookup), _stream(dev))
+        st = lib.tplr_quantize_batch(_ptr(val), k, _ptr(batch.table), T, n_bins, C.c_float(range_in_sigmas), slices,
+                                     _ptr(work), _ptr(codes), _ptr(shift), _ptr(scale), _ptr(lookup), _stream(dev))
     _lib.check(st, "tplr_quantize_batch")
     return codes, shift, scale, lookup
 

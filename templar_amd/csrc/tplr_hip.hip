@@ -1146,65 +1146,107 @@ __global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int
 // De-quantise one peer's flat payload of 8-bit codes: value = lookup[t][code] + shift[t], the
 // tensor t found from the row id (TopKCompressor._dequantize_values, src/tplr/compress.py:637-643,
 // for every parameter of the set at once).  Four codes per thread.
-// The statistical quantiser over each tensor's sent values (src/tplr/compress.py:582-621): one
-// workgroup per tensor makes the three passes of the reference - mean, norm of the centred values,
-// codes with per-bin means - over that tensor's part of the flat payload.  Sums are carried in
-// double and rounded once, where the reference's fp32 reductions round on the way.
-__device__ __forceinline__ double block_sum_f64(double x, double* part, int tid) {
+// The statistical quantiser over each tensor's sent values (src/tplr/compress.py:582-621): the
+// reference's three passes - mean, norm of the centred values, codes with per-bin means - as three
+// launches over slices of every tensor plus one that finishes the tables.  Partial sums are carried
+// in double, kept per (tensor, slice) in a caller-provided workspace and added in slice order by
+// whoever needs the total, so every workgroup of a tensor derives the same shift and scale.
+// Workspace layout (doubles): sum[T][S], sumsq[T][S], then bins[T][S][2 * n_bins] (sums, counts).
+struct QuantSlice {
+    const float4* v;
+    uchar4* q;
+    int64_t n4;  // float4 groups in this slice
+    int64_t n;   // values in the whole tensor
+    int t, s;
+};
+
+__device__ __forceinline__ QuantSlice quant_slice(const float* val, uint8_t* codes, const tplr_tensor_desc* table,
+                                                   int k, int S) {
+    QuantSlice qs;
+    qs.t = blockIdx.x / S;
+    qs.s = blockIdx.x - qs.t * S;
+    const tplr_tensor_desc d = table[qs.t];
+    const int64_t rows = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
+    const int64_t r0 = rows * qs.s / S, r1 = rows * (qs.s + 1) / S;
+    qs.v = reinterpret_cast<const float4*>(val + (d.chunk_begin + r0) * k);
+    qs.q = codes ? reinterpret_cast<uchar4*>(codes + (d.chunk_begin + r0) * k) : nullptr;
+    qs.n4 = (r1 - r0) * k >> 2;  // k is a multiple of 4
+    qs.n = rows * k;
+    return qs;
+}
+
+__device__ __forceinline__ double block256_sum_f64(double x, double* part, int tid) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off);
     __syncthreads();  // `part` may still be read from the previous call
     if ((tid & 63) == 0) part[tid >> 6] = x;
     __syncthreads();
+    return (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+__device__ __forceinline__ double slices_total(const double* w, int S) {
     double s = 0.0;
-#pragma unroll
-    for (int w = 0; w < 16; ++w) s += part[w];
+    for (int i = 0; i < S; ++i) s += w[i];
     return s;
 }
 
-__global__ __launch_bounds__(1024) void k_quantize_batch(const float* __restrict__ val, int k,
-                                                          const tplr_tensor_desc* __restrict__ table, int n_bins,
-                                                          float range_in_sigmas, uint8_t* __restrict__ codes,
-                                                          float* __restrict__ shift_out, float* __restrict__ scale_out,
-                                                          float* __restrict__ lookup) {
-    __shared__ double part[16];
-    __shared__ double bin_sum[256];
-    __shared__ unsigned int bin_cnt[256];
-    const int t = blockIdx.x, tid = threadIdx.x;
-    const tplr_tensor_desc d = table[t];
-    const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks * k;  // k is a multiple of 4
-    const float* v = val + d.chunk_begin * k;
-    uint8_t* q = codes + d.chunk_begin * k;
-    const int64_t n4 = n >> 2;
-    // every pass walks the tensor four float4 per thread at a time, so that four loads are in flight
-    const float4* v4 = reinterpret_cast<const float4*>(v);
-    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    auto walk = [&](auto&& body) {
-        for (int64_t i = tid; i < n4; i += 4096) {
-            const bool h1 = i + 1024 < n4, h2 = i + 2048 < n4, h3 = i + 3072 < n4;
-            const float4 x0 = v4[i];
-            const float4 x1 = h1 ? v4[i + 1024] : zero4;
-            const float4 x2 = h2 ? v4[i + 2048] : zero4;
-            const float4 x3 = h3 ? v4[i + 3072] : zero4;
-            body(i, x0);
-            if (h1) body(i + 1024, x1);
-            if (h2) body(i + 2048, x2);
-            if (h3) body(i + 3072, x3);
-        }
-    };
+__device__ __forceinline__ float quant_shift(const double* work, int t, int S, int64_t n) {
+    return static_cast<float>(slices_total(work + static_cast<int64_t>(t) * S, S) / static_cast<double>(n));  // :594
+}
+
+__device__ __forceinline__ float quant_scale(const double* work, int T, int t, int S, int64_t n, int n_bins,
+                                             float range_in_sigmas) {
+    const double ss = slices_total(work + (static_cast<int64_t>(T) + t) * S, S);
+    const float sd = static_cast<float>(sqrt(ss) / sqrt(static_cast<double>(n - 1)));  // :597
+    const float scale = range_in_sigmas * sd / static_cast<float>(n_bins);              // :598
+    return (scale == 0.f || scale != scale || __builtin_isinf(scale)) ? 1.0f : scale;   // :599-600
+}
+
+__global__ __launch_bounds__(256) void k_quant_sum(const float* __restrict__ val, int k,
+                                                   const tplr_tensor_desc* __restrict__ table, int S,
+                                                   double* __restrict__ work) {
+    __shared__ double part[4];
+    const int tid = threadIdx.x;
+    const QuantSlice qs = quant_slice(val, nullptr, table, k, S);
     double acc = 0.0;
-    walk([&](int64_t, const float4& x) { acc += (static_cast<double>(x.x) + x.y) + (static_cast<double>(x.z) + x.w); });
-    const float shift = static_cast<float>(block_sum_f64(acc, part, tid) / static_cast<double>(n));  // :594
-    acc = 0.0;
-    walk([&](int64_t, const float4& x) {
+    for (int64_t i = tid; i < qs.n4; i += 256) {
+        const float4 x = qs.v[i];
+        acc += (static_cast<double>(x.x) + x.y) + (static_cast<double>(x.z) + x.w);
+    }
+    acc = block256_sum_f64(acc, part, tid);
+    if (tid == 0) work[blockIdx.x] = acc;
+}
+
+__global__ __launch_bounds__(256) void k_quant_sumsq(const float* __restrict__ val, int k,
+                                                     const tplr_tensor_desc* __restrict__ table, int T, int S,
+                                                     double* __restrict__ work) {
+    __shared__ double part[4];
+    const int tid = threadIdx.x;
+    const QuantSlice qs = quant_slice(val, nullptr, table, k, S);
+    const float shift = quant_shift(work, qs.t, S, qs.n);
+    double acc = 0.0;
+    for (int64_t i = tid; i < qs.n4; i += 256) {
+        const float4 x = qs.v[i];
         const float a = x.x - shift, b = x.y - shift, c = x.z - shift, e = x.w - shift;  // :595
         acc += (static_cast<double>(a) * a + static_cast<double>(b) * b) +
                (static_cast<double>(c) * c + static_cast<double>(e) * e);
-    });
-    const double ss = block_sum_f64(acc, part, tid);
-    const float sd = static_cast<float>(sqrt(ss) / sqrt(static_cast<double>(n - 1)));  // :597
-    float scale = range_in_sigmas * sd / static_cast<float>(n_bins);                    // :598
-    if (scale == 0.f || scale != scale || __builtin_isinf(scale)) scale = 1.0f;         // :599-600
+    }
+    acc = block256_sum_f64(acc, part, tid);
+    if (tid == 0) work[static_cast<int64_t>(T) * S + blockIdx.x] = acc;
+}
+
+__global__ __launch_bounds__(256) void k_quant_codes(const float* __restrict__ val, int k,
+                                                     const tplr_tensor_desc* __restrict__ table, int T, int S, int n_bins,
+                                                     float range_in_sigmas, uint8_t* __restrict__ codes,
+                                                     double* __restrict__ work) {
+    __shared__ double part[4];
+    __shared__ double bin_sum[256];
+    __shared__ unsigned int bin_cnt[256];
+    const int tid = threadIdx.x;
+    const QuantSlice qs = quant_slice(val, codes, table, k, S);
+    const float shift = quant_shift(work, qs.t, S, qs.n);
+    const float scale = quant_scale(work, T, qs.t, S, qs.n, n_bins, range_in_sigmas);
+    double* out = work + 2 * static_cast<int64_t>(T) * S + static_cast<int64_t>(blockIdx.x) * 2 * n_bins;
     const float offset = static_cast<float>(n_bins / 2), top = static_cast<float>(n_bins - 1);
     auto code = [&](float x, float& c) {
         c = x - shift;
@@ -1213,7 +1255,6 @@ __global__ __launch_bounds__(1024) void k_quantize_batch(const float* __restrict
         r = r > top ? top : r;                          // :606
         return static_cast<uint32_t>(r);
     };
-    uchar4* q4 = reinterpret_cast<uchar4*>(q);
     if (n_bins <= 8) {
         // a handful of bins (templar runs four): per-thread sums, no contended atomics
         double s8[8], c8[8];
@@ -1226,38 +1267,55 @@ __global__ __launch_bounds__(1024) void k_quantize_batch(const float* __restrict
                 c8[b] += qq == static_cast<uint32_t>(b) ? 1.0 : 0.0;
             }
         };
-        walk([&](int64_t i, const float4& x) {
+        for (int64_t i = tid; i < qs.n4; i += 256) {
+            const float4 x = qs.v[i];
             float c0, c1, c2, c3;
             const uint32_t q0 = code(x.x, c0), q1 = code(x.y, c1), q2 = code(x.z, c2), q3 = code(x.w, c3);
-            q4[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
-                                static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
+            qs.q[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
+                                  static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
             tally(q0, c0), tally(q1, c1), tally(q2, c2), tally(q3, c3);
-        });
+        }
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            const double sum = block_sum_f64(s8[b], part, tid), cnt = block_sum_f64(c8[b], part, tid);
-            if (tid == 0 && b < n_bins)
-                lookup[static_cast<int64_t>(t) * n_bins + b] = cnt > 0.0 ? static_cast<float>(sum / cnt) : 0.f;  // :619
+            const double sum = block256_sum_f64(s8[b], part, tid), cnt = block256_sum_f64(c8[b], part, tid);
+            if (tid == 0 && b < n_bins) out[b] = sum, out[n_bins + b] = cnt;
         }
     } else {
-        if (tid < 256) bin_sum[tid] = 0.0, bin_cnt[tid] = 0u;
+        bin_sum[tid] = 0.0, bin_cnt[tid] = 0u;
         __syncthreads();
-        walk([&](int64_t i, const float4& x) {
+        for (int64_t i = tid; i < qs.n4; i += 256) {
+            const float4 x = qs.v[i];
             float c0, c1, c2, c3;
             const uint32_t q0 = code(x.x, c0), q1 = code(x.y, c1), q2 = code(x.z, c2), q3 = code(x.w, c3);
-            q4[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
-                                static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
+            qs.q[i] = make_uchar4(static_cast<unsigned char>(q0), static_cast<unsigned char>(q1),
+                                  static_cast<unsigned char>(q2), static_cast<unsigned char>(q3));
             atomicAdd(&bin_sum[q0], static_cast<double>(c0)), atomicAdd(&bin_cnt[q0], 1u);  // :614-617
             atomicAdd(&bin_sum[q1], static_cast<double>(c1)), atomicAdd(&bin_cnt[q1], 1u);
             atomicAdd(&bin_sum[q2], static_cast<double>(c2)), atomicAdd(&bin_cnt[q2], 1u);
             atomicAdd(&bin_sum[q3], static_cast<double>(c3)), atomicAdd(&bin_cnt[q3], 1u);
-        });
+        }
         __syncthreads();
-        if (tid < n_bins)
-            lookup[static_cast<int64_t>(t) * n_bins + tid] =
-                bin_cnt[tid] ? static_cast<float>(bin_sum[tid] / static_cast<double>(bin_cnt[tid])) : 0.f;  // :619
+        if (tid < n_bins) out[tid] = bin_sum[tid], out[n_bins + tid] = static_cast<double>(bin_cnt[tid]);
     }
-    if (tid == 0) shift_out[t] = shift, scale_out[t] = scale;
+}
+
+__global__ __launch_bounds__(256) void k_quant_tables(const tplr_tensor_desc* __restrict__ table, int k, int T, int S,
+                                                      int n_bins, float range_in_sigmas,
+                                                      const double* __restrict__ work, float* __restrict__ shift_out,
+                                                      float* __restrict__ scale_out, float* __restrict__ lookup) {
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const tplr_tensor_desc d = table[t];
+    const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks * k;
+    if (tid < n_bins) {
+        const double* bins = work + 2 * static_cast<int64_t>(T) * S + static_cast<int64_t>(t) * S * 2 * n_bins;
+        double sum = 0.0, cnt = 0.0;
+        for (int s = 0; s < S; ++s) sum += bins[s * 2 * n_bins + tid], cnt += bins[s * 2 * n_bins + n_bins + tid];
+        lookup[static_cast<int64_t>(t) * n_bins + tid] = cnt > 0.0 ? static_cast<float>(sum / cnt) : 0.f;  // :619
+    }
+    if (tid == 0) {
+        shift_out[t] = quant_shift(work, t, S, n);
+        scale_out[t] = quant_scale(work, T, t, S, n, n_bins, range_in_sigmas);
+    }
 }
 
 __global__ __launch_bounds__(256) void k_dequantize_batch(const uint8_t* __restrict__ q,
@@ -1990,15 +2048,21 @@ int tplr_dequantize_peers(const uint8_t* const* h_codes, int n_peers, int64_t n,
 }
 
 int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
-                        float range_in_sigmas, uint8_t* d_codes, float* d_shift, float* d_scale, float* d_lookup,
-                        void* stream) {
-    if (!d_val || !d_desc || !d_codes || !d_shift || !d_scale || !d_lookup || n_tensors < 1 || k < 4 || (k & 3) ||
-        n_bins < 1 || n_bins > 256)
+                        float range_in_sigmas, int n_slices, double* d_work, uint8_t* d_codes, float* d_shift,
+                        float* d_scale, float* d_lookup, void* stream) {
+    if (!d_val || !d_desc || !d_work || !d_codes || !d_shift || !d_scale || !d_lookup || n_tensors < 1 || k < 4 ||
+        (k & 3) || n_bins < 1 || n_bins > 256 || n_slices < 1 || n_slices > 1024)
         return TPLR_E_BADARG;
     if ((reinterpret_cast<uintptr_t>(d_val) & 15) || (reinterpret_cast<uintptr_t>(d_codes) & 3)) return TPLR_E_BADARG;
-    hipLaunchKernelGGL(k_quantize_batch, dim3(static_cast<unsigned>(n_tensors)), dim3(1024), 0,
-                       static_cast<hipStream_t>(stream), d_val, k, d_desc, n_bins, range_in_sigmas, d_codes, d_shift,
-                       d_scale, d_lookup);
+    if (static_cast<int64_t>(n_tensors) * n_slices > 0x7fffffff) return TPLR_E_TOOMANY;
+    const dim3 grid(static_cast<unsigned>(n_tensors) * n_slices), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(k_quant_sum, grid, block, 0, st, d_val, k, d_desc, n_slices, d_work);
+    hipLaunchKernelGGL(k_quant_sumsq, grid, block, 0, st, d_val, k, d_desc, n_tensors, n_slices, d_work);
+    hipLaunchKernelGGL(k_quant_codes, grid, block, 0, st, d_val, k, d_desc, n_tensors, n_slices, n_bins, range_in_sigmas,
+                       d_codes, d_work);
+    hipLaunchKernelGGL(k_quant_tables, dim3(static_cast<unsigned>(n_tensors)), block, 0, st, d_desc, k, n_tensors,
+                       n_slices, n_bins, range_in_sigmas, d_work, d_shift, d_scale, d_lookup);
     return launch_status();
 }
 
