@@ -190,6 +190,31 @@ def test_topk_skewed_chunks(dev):
     check_topk(rows.reshape(16, 4096), 64, dev)
 
 
+@pytest.mark.parametrize("kind", ["normal", "few_levels", "heavy_tails_row_scaled", "sparse"])
+def test_select_is_bit_exact_on_other_value_laws(dev, kind):
+    # untransformed encode = select straight from the tensor: canonical order against the oracle for
+    # every k the sort network serves (one key per lane, two keys per lane) and for tie-heavy inputs
+    rng = np.random.default_rng(sum(map(ord, kind)))
+    Y, X = 3, 5
+    shape = (Y * 64, X * 64)
+    if kind == "normal":
+        x = rng.standard_normal(shape)
+    elif kind == "few_levels":
+        x = rng.integers(-3, 4, shape)  # seven distinct values: ties everywhere
+    elif kind == "heavy_tails_row_scaled":
+        x = rng.standard_t(2, shape) * np.exp(rng.standard_normal((shape[0], 1)))
+    else:
+        x = np.where(rng.random(shape) < 0.01, rng.standard_normal(shape), 0.0)
+    x = x.astype(np.float32)
+    chunks = x.reshape(Y, 64, X, 64).transpose(0, 2, 1, 3).reshape(Y * X, 4096)
+    xt = torch.from_numpy(x).to(dev)
+    for k in (2, 8, 32, 64, 128):
+        idx, val, _, _ = tc.encode_compress(xt, k, use_dct=False)
+        want_i, want_v = orc.topk_rows(chunks, k)
+        assert np.array_equal(tc.unpack_12bit_indices(idx, val.shape).cpu().numpy().reshape(-1, k), want_i), (kind, k)
+        assert np.array_equal(val.cpu().numpy().reshape(-1, k), want_v), (kind, k)
+
+
 def test_topk_special_values(dev):
     rows = np.zeros((6, 4096), np.float32)
     rows[1, [5, 900, 17]] = [2.0, -2.0, 2.0]
