@@ -2053,7 +2053,9 @@ int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_des
     if (!d_val || !d_desc || !d_work || !d_codes || !d_shift || !d_scale || !d_lookup || n_tensors < 1 || k < 4 ||
         (k & 3) || n_bins < 1 || n_bins > 256 || n_slices < 1 || n_slices > 1024)
         return TPLR_E_BADARG;
-    if ((reinterpret_cast<uintptr_t>(d_val) & 15) || (reinterpret_cast<uintptr_t>(d_codes) & 3)) return TPLR_E_BADARG;
+    if ((reinterpret_cast<uintptr_t>(d_val) & 15) || (reinterpret_cast<uintptr_t>(d_codes) & 3) ||
+        (reinterpret_cast<uintptr_t>(d_work) & 7))
+        return TPLR_E_BADARG;
     if (static_cast<int64_t>(n_tensors) * n_slices > 0x7fffffff) return TPLR_E_TOOMANY;
     const dim3 grid(static_cast<unsigned>(n_tensors) * n_slices), block(256);
     hipStream_t st = static_cast<hipStream_t>(stream);

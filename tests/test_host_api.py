@@ -6,6 +6,8 @@ import json
 import os
 import re
 
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -161,6 +163,45 @@ def test_host_gather_concatenates_parts_with_any_thread_count():
     assert lib.tplr_gather_host(ptrs, nbytes, len(parts), None, 4) == _lib.TPLR_E_BADARG
     assert lib.tplr_gather_host(ptrs, nbytes, len(parts), 1, 0) == _lib.TPLR_E_BADARG
     assert lib.tplr_gather_host(None, None, 0, None, 1) == 0
+
+
+def test_entry_points_reject_bad_arguments_before_any_launch():
+    # argument checks run on the host and return before a kernel is launched: no device needed.
+    # (1 stands for "some non-null pointer": a rejected call never dereferences it.)
+    from templar_amd import _lib
+    lib = _lib.load()
+    E = _lib
+    p = 1 << 12
+    assert lib.tplr_version() > 0
+    assert lib.tplr_pack12(None, 2, p, None, None) == E.TPLR_E_BADARG
+    assert lib.tplr_pack12(p, 3, p, None, None) == E.TPLR_E_ODD
+    assert lib.tplr_pack12(p, -2, p, None, None) == E.TPLR_E_BADARG
+    assert lib.tplr_pack12(None, 0, None, None, None) == 0
+    assert lib.tplr_unpack12(None, 2, p, None) == E.TPLR_E_BADARG
+    assert lib.tplr_unpack12(p, 5, p, None) == E.TPLR_E_ODD
+    assert lib.tplr_dct2d_fwd(None, 64, 64, 64, p, None) == E.TPLR_E_BADARG
+    assert lib.tplr_dct2d_fwd(p, 64, 96 + 1, 128, p, None) == E.TPLR_E_SHAPE
+    assert lib.tplr_dct2d_inv(p, 63, 64, p, 64, None) == E.TPLR_E_SHAPE
+    assert lib.tplr_topk_pack(p, 1, 4096, 33, p, p, None) == E.TPLR_E_BADARG      # odd k
+    assert lib.tplr_topk_pack(p, 1, 5000, 32, p, p, None) == E.TPLR_E_TOOMANY     # row too long
+    assert lib.tplr_encode_topk_pack(p, 64, 64, 32, 32, 1, p, p, None) == E.TPLR_E_BADARG  # stride below the width
+    assert lib.tplr_encode_topk_pack(p, 64, 64, 64, 130, 1, p, p, None) == E.TPLR_E_BADARG  # k above 128
+    assert lib.tplr_encode_topk_pack_batch(None, 1, 1, 32, 1, p, p, None) == E.TPLR_E_BADARG
+    ptrs = (C.c_void_p * 2)(p, p)
+    assert lib.tplr_decode_aggregate(ptrs, ptrs, None, 2, 31, 64, 64, 0, 0, 1, p, 64, None, None) == E.TPLR_E_BADARG
+    assert lib.tplr_decode_aggregate(ptrs, ptrs, None, 2, 32, 64, 65, 0, 0, 1, p, 65, None, None) == E.TPLR_E_SHAPE
+    many = (C.c_void_p * 129)(*([p] * 129))
+    assert lib.tplr_decode_aggregate(many, many, None, 129, 32, 64, 64, 0, 0, 1, p, 64, None, None) == E.TPLR_E_TOOMANY
+    assert lib.tplr_index_stats_batch(many, 33, 32, p, 1, 1, p, p, p, None) == E.TPLR_E_TOOMANY
+    assert lib.tplr_index_stats_batch(ptrs, 2, 33, p, 1, 1, p, p, p, None) == E.TPLR_E_BADARG
+    assert lib.tplr_dequantize_batch(p, p, p, 300, 32, p, 1, 1, p, None) == E.TPLR_E_BADARG   # more than 256 bins
+    assert lib.tplr_dequantize_peers(ptrs, 2, 6, p, p, 4, ptrs, None) == E.TPLR_E_BADARG       # n not a multiple of 4
+    assert lib.tplr_quantize_batch(p, 32, p, 1, 4, C.c_float(6.0), 0, p, p, p, p, p, None) == E.TPLR_E_BADARG  # no slices
+    assert lib.tplr_quantize_batch(p + 4, 32, p, 1, 4, C.c_float(6.0), 1, p, p, p, p, p, None) == E.TPLR_E_BADARG
+    assert lib.tplr_segment_sumsq(ptrs, 2, 32, p, 1, 0, p, None) == E.TPLR_E_BADARG
+    assert lib.tplr_clip_scales(None, 2, 0, p, None, None) == E.TPLR_E_BADARG
+    for code in (0, E.TPLR_E_BADARG, E.TPLR_E_ODD, E.TPLR_E_SHAPE, E.TPLR_E_TOOMANY, 1):
+        assert len(lib.tplr_status_string(code)) > 0
 
 
 def test_pack_unpack_errors():
