@@ -1,4 +1,5 @@
-"""The reference's op sequence on torch CPU tensors.  Test infrastructure only.
+"""The reference's op sequence on torch tensors (CPU for the checks and the host baseline; it
+follows its inputs' device, so the benchmark can also time it on the GPU).  Test infrastructure only.
 
 This restates src/tplr/compress.py (tplr 2.1.28) as plain functions that issue the same
 torch primitives in the same order - strided view + 3-operand einsum, abs/topk(sorted=False)/
@@ -81,7 +82,7 @@ def pack12(indices: torch.Tensor) -> torch.Tensor:
     if flat.numel() % 2:
         raise ValueError(f"Number of indices must be even, got {flat.numel()}")
     flat = flat.to(torch.int32)
-    out = torch.zeros(flat.numel() // 2 * 3, dtype=torch.uint8)
+    out = torch.zeros(flat.numel() // 2 * 3, dtype=torch.uint8, device=indices.device)
     if flat.numel():
         a, b = flat.reshape(-1, 2).unbind(1)
         out[0::3] = (a & 0xFF).to(torch.uint8)
@@ -93,10 +94,10 @@ def pack12(indices: torch.Tensor) -> torch.Tensor:
 def unpack12(packed: torch.Tensor, shape) -> torch.Tensor:
     n = int(torch.prod(torch.tensor(shape)).item())
     if n == 0:
-        return torch.zeros(shape, dtype=torch.int64)
+        return torch.zeros(shape, dtype=torch.int64, device=packed.device)
     if n % 2:
         raise ValueError(f"Number of indices must be even, got {n}")
-    out = torch.zeros(n, dtype=torch.int64)
+    out = torch.zeros(n, dtype=torch.int64, device=packed.device)
     b0, b1, b2 = (packed[i::3].to(torch.int64) for i in range(3))
     out[0::2] = b0 | ((b1 & 0x0F) << 8)
     out[1::2] = ((b1 >> 4) & 0x0F) | (b2 << 4)
@@ -121,7 +122,7 @@ def compress(x: torch.Tensor, topk: int):
 
 
 def decompress(idx: torch.Tensor, val: torch.Tensor, xshape, totalk: int, dtype=torch.float32):
-    x = torch.zeros(xshape, dtype=dtype)
+    x = torch.zeros(xshape, dtype=dtype, device=val.device)
     if len(xshape) > 2:
         x = x.reshape(xshape[0], xshape[1], -1)
     if idx.dtype == torch.uint8:
