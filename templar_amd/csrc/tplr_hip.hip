@@ -981,9 +981,27 @@ struct IdxPtrs {
     const uint8_t* idx[kStatPeers];
 };
 
+// body(Index<0>{}) ... body(Index<N - 1>{}): a loop whose counter is a constant in the body, so that
+// arrays indexed by it stay in registers whatever the optimiser thinks of unrolling
+template <int I>
+struct Index {
+    static constexpr int value = I;
+};
+template <int N, typename Body>
+__device__ __forceinline__ void static_for(Body&& body) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(body);
+        body(Index<N - 1>{});
+    }
+}
+
 // kPerPass: peers handled by one wave instruction: 2 when k <= 32 (one peer per half of the wave), 1 when
-// k <= 64; 0 = rows of any length, entry by entry.
-template <int kPerPass>
+// k <= 64; 0 = rows of any length, entry by entry.  kPasses: wave instructions per row that the
+// register arrays are sized for (kPerPass * kPasses peers at most).  kPlanes > 0: shared entries are
+// counted in registers - every lane keeps, per pass, one counter per later peer as kPlanes bit planes
+// (bit j of plane b = bit b of the count for peer p + 1 + j), incremented with a ripple of ANDs and
+// XORs and summed over the lanes every 2^kPlanes - 1 rows; 0 = counted with LDS atomics.
+template <int kPerPass, int kPasses = 1, int kPlanes = 0>
 __global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int k,
                                                     const tplr_tensor_desc* __restrict__ table,
                                                     const tplr_tensor_desc single, int n_tensors, int64_t total,
@@ -1024,16 +1042,21 @@ __global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int
         // One entry per lane and peer, all peers of a row in registers; the next row's entries are
         // requested before this row is worked on.  Repeats and maxima are kept per lane and
         // reach the per-tensor totals when those are flushed.
-        constexpr int kPasses = kStatPeers / kPerPass;
         const int sub = kPerPass == 2 ? lane >> 5 : 0;
         const int j = kPerPass == 2 ? (lane & 31) : lane;
         const bool jon = j < k;
         const int joff = 3 * (j >> 1) + (j & 1);
         const uint32_t jshift = (j & 1) * 4;
-        uint32_t cur[kPasses], nxt[kPasses], rep[kPasses];
+        uint32_t cur[kPasses], nxt[kPasses];
         int top[kPasses];
+        uint32_t planes[kPlanes ? kPasses : 1][kPlanes ? kPlanes : 1];
 #pragma unroll
-        for (int i = 0; i < kPasses; ++i) cur[i] = nxt[i] = rep[i] = 0, top[i] = -1;
+        for (int i = 0; i < kPasses; ++i) cur[i] = nxt[i] = 0, top[i] = -1;
+#pragma unroll
+        for (int i = 0; i < (kPlanes ? kPasses : 1); ++i)
+#pragma unroll
+            for (int b = 0; b < (kPlanes ? kPlanes : 1); ++b) planes[i][b] = 0;
+        int pending = 0;  // rows counted in the planes since they were last summed
         auto request = [&](uint32_t (&e)[kPasses], int64_t g) {
 #pragma unroll
             for (int i = 0; i < kPasses; ++i) {
@@ -1045,16 +1068,47 @@ __global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int
                 }
             }
         };
-        auto fold = [&]() {  // per-lane repeats and maxima into the per-tensor totals
+        // bit planes -> pair counters: for every pass and later peer, the lanes' counts are summed plane
+        // by plane with ballots (the two halves of the wave are two peers when kPerPass == 2)
+        auto sum_planes = [&]() __attribute__((always_inline)) {
+            if constexpr (kPlanes > 0) {
+                static_for<kPasses>([&](auto pass) __attribute__((always_inline)) {
+                    constexpr int i = decltype(pass)::value;
+                    const int p0 = i * kPerPass;
+                    if (p0 + 1 < P) {  // wave-uniform
+                        const int later = P - 1 - p0;
+                        for (int jb = 0; jb < later; ++jb) {
+                            uint32_t lo = 0, hi = 0;
+#pragma unroll
+                            for (int b = 0; b < kPlanes; ++b) {
+                                const uint64_t hit = __ballot(((planes[i][b] >> jb) & 1u) != 0u);
+                                if constexpr (kPerPass == 2) {
+                                    lo += static_cast<uint32_t>(__popc(static_cast<uint32_t>(hit))) << b;
+                                    hi += static_cast<uint32_t>(__popc(static_cast<uint32_t>(hit >> 32))) << b;
+                                } else {
+                                    lo += static_cast<uint32_t>(__popcll(hit)) << b;
+                                }
+                            }
+                            if (lane == 0) {
+                                pair_l[p0 * kStatPeers + p0 + 1 + jb] += lo;
+                                if (kPerPass == 2 && p0 + 2 + jb < P) pair_l[(p0 + 1) * kStatPeers + p0 + 2 + jb] += hi;
+                            }
+                        }
+#pragma unroll
+                        for (int b = 0; b < kPlanes; ++b) planes[i][b] = 0;
+                    }
+                });
+            }
+            pending = 0;
+        };
+        auto fold = [&]() __attribute__((always_inline)) {  // per-lane counts and maxima into the per-tensor totals
+            sum_planes();
 #pragma unroll
             for (int i = 0; i < kPasses; ++i) {
                 const int p = i * kPerPass + sub;
                 if (i * kPerPass < P) {
-                    if (jon && p < P) {
-                        if (rep[i]) atomicAdd(&dup_l[p], rep[i]);
-                        if (top[i] >= 0) atomicMax(&mx_l[p], top[i]);
-                    }
-                    rep[i] = 0, top[i] = -1;
+                    if (jon && p < P && top[i] >= 0) atomicMax(&mx_l[p], top[i]);
+                    top[i] = -1;
                 }
             }
         };
@@ -1078,24 +1132,37 @@ __global__ __launch_bounds__(64) void k_index_stats(const IdxPtrs ip, int P, int
                 const int p = i * kPerPass + sub;
                 if (i * kPerPass < P && jon && p < P) {
                     const uint32_t old = atomicOr(&mask[cur[i]], 1u << p);
-                    rep[i] += (old >> p) & 1u;
+                    if ((old >> p) & 1u) atomicAdd(&dup_l[p], 1u);  // a repeat inside the row: rare
                     top[i] = top[i] > static_cast<int>(cur[i]) ? top[i] : static_cast<int>(cur[i]);
                 }
             }
             wave_lds_fence();
-#pragma unroll
-            for (int i = 0; i < kPasses; ++i) {
+            static_for<kPasses>([&](auto pass) __attribute__((always_inline)) {
+                constexpr int i = decltype(pass)::value;
                 const int p = i * kPerPass + sub;
-                if (i * kPerPass < P && jon && p + 1 < P) {
-                    uint32_t m = mask[cur[i]] >> (p + 1);  // the peers after p that sent this entry too
-                    while (m) {
-                        const int q = p + 1 + __builtin_ctz(m);
-                        atomicAdd(&pair_l[p * kStatPeers + q], 1u);
-                        m &= m - 1;
+                if (i * kPerPass + 1 < P) {  // wave-uniform: a later peer exists
+                    // the peers after p that sent this lane's entry too, bit 0 = peer p + 1
+                    const uint32_t m = (jon && p + 1 < P) ? mask[cur[i]] >> ((p + 1) & 31) : 0u;
+                    if constexpr (kPlanes > 0) {
+                        uint32_t carry = m;
+#pragma unroll
+                        for (int b = 0; b < kPlanes; ++b) {
+                            const uint32_t t = planes[i][b] & carry;
+                            planes[i][b] ^= carry;
+                            carry = t;
+                        }
+                    } else {
+                        uint32_t w = m;
+                        while (w) {
+                            const int q = p + 1 + __builtin_ctz(w);
+                            atomicAdd(&pair_l[p * kStatPeers + q], 1u);
+                            w &= w - 1;
+                        }
                     }
                 }
-            }
+            });
             wave_lds_fence();
+            if (kPlanes > 0 && ++pending == (1 << kPlanes) - 1) sum_planes();
             if (g + 1 < g1) cursor_next(c, g + 1);
         }
         fold();
@@ -1989,13 +2056,19 @@ int tplr_index_stats_batch(const uint8_t* const* h_idx12, int n_peers, int k, co
                            reinterpret_cast<unsigned long long*>(d_pair), reinterpret_cast<unsigned long long*>(d_dup),
                            d_max);
     };
-    static int resident[3] = {0, 0, 0};
-    if (k <= 32)
-        launch(k_index_stats<2>, resident[2]);
+    static int resident[6] = {0, 0, 0, 0, 0, 0};
+    if (k <= 32 && n_peers <= 16)
+        launch(k_index_stats<2, 8, 8>, resident[0]);
+    else if (k <= 32)
+        launch(k_index_stats<2, 16, 8>, resident[1]);
+    else if (k <= 64 && n_peers <= 16)
+        launch(k_index_stats<1, 16, 8>, resident[2]);
+    else if (k <= 64 && n_peers <= 24)
+        launch(k_index_stats<1, 24, 6>, resident[3]);
     else if (k <= 64)
-        launch(k_index_stats<1>, resident[1]);
+        launch(k_index_stats<1, 32, 0>, resident[4]);
     else
-        launch(k_index_stats<0>, resident[0]);
+        launch(k_index_stats<0>, resident[5]);
     return launch_status();
 }
 
