@@ -205,3 +205,48 @@ def test_full_set_error_feedback_step(dev):
         want = ch.scatter(1, ix, 0.0).reshape(y, x, 64, 64).permute(0, 2, 1, 3).reshape(a.shape)
         assert torch.equal(e, want)
 
+
+
+@pytest.mark.parametrize("P,k", [(20, 64), (15, 32), (12, 64)])
+def test_full_size_index_statistics_against_bitmaps(dev, P, k):
+    # the 1B set's 294 144 rows: every wave walks 144 rows, so the per-lane bit-plane counters are
+    # summed in mid-run and at tensor boundaries.  Reference: one 4096-bit membership map per peer
+    # and row built with torch.scatter_, shared entries = map_j gathered at peer i's indices.
+    shapes = [s for s in workloads.CONFIGS["cfg3_llama1b"]["shapes"] if len(s) == 2]
+    counts = [(a // 64) * (b // 64) for a, b in shapes]
+    n = sum(counts)
+    g = torch.Generator(device=dev)
+    g.manual_seed(100 * P + k)
+    base = torch.rand((n, 4096), device=dev, generator=g).topk(k, dim=-1).indices
+    rows, packed = [], []
+    for p in range(P):
+        own = torch.rand((n, 4096), device=dev, generator=g).topk(k, dim=-1).indices
+        # a varying share of `base`, column by column; entries repeated inside a row are allowed here
+        # (both counts treat them alike: every copy in peer i counts, the other peer's set does not grow)
+        keep = torch.rand((n, k), device=dev, generator=g) < (0.1 + 0.04 * p)
+        r = torch.where(keep, base, own)
+        rows.append(r)
+        packed.append(tc.pack_12bit_indices(r.contiguous()))
+        del own, keep
+    pair, dup, top = tc.index_stats_batch(counts, packed, k)
+    bounds = np.cumsum([0] + counts)
+    seg = torch.zeros(n, dtype=torch.int64, device=dev)
+    for t in range(len(counts)):
+        seg[bounds[t]:bounds[t + 1]] = t
+    maps = []
+    for p in range(P):
+        m = torch.zeros((n, 4096), dtype=torch.bool, device=dev)
+        m.scatter_(1, rows[p], True)
+        maps.append(m)
+    want = torch.zeros((len(counts), P, P), dtype=torch.int64, device=dev)
+    for i in range(P):
+        for j in range(i + 1, P):
+            per_row = maps[j].gather(1, rows[i]).sum(dim=1)
+            want[:, i, j].index_add_(0, seg, per_row)
+    assert torch.equal(torch.triu(pair, 1), want)
+    for p in range(P):
+        distinct = maps[p].sum(dim=1)
+        want_dup = torch.zeros(len(counts), dtype=torch.int64, device=dev).index_add_(0, seg, k - distinct)
+        assert torch.equal(dup[:, p], want_dup)
+        want_top = torch.stack([rows[p][bounds[t]:bounds[t + 1]].max() for t in range(len(counts))])
+        assert torch.equal(top[:, p].long(), want_top)
