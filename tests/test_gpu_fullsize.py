@@ -250,3 +250,52 @@ def test_full_size_index_statistics_against_bitmaps(dev, P, k):
         assert torch.equal(dup[:, p], want_dup)
         want_top = torch.stack([rows[p][bounds[t]:bounds[t + 1]].max() for t in range(len(counts))])
         assert torch.equal(top[:, p].long(), want_top)
+
+
+@pytest.mark.parametrize("use_dct", [False, True])
+def test_full_set_aggregate_against_torch_scatter_reduce(dev, use_dct):
+    # the 1B set, 15 peers, every chunk: torch's own scatter_reduce_(mean, include_self=False) on the
+    # concatenated payloads (the reference's op sequence, src/tplr/compress.py:559-580, run on the GPU),
+    # then its einsum decode, against the one-launch aggregate
+    from oracle import torch_cpu_path as tcp
+
+    P, k = 15, 32
+    shapes = [s for s in workloads.CONFIGS["cfg3_llama1b"]["shapes"] if len(s) == 2]
+    counts = [(a // 64) * (b // 64) for a, b in shapes]
+    n = sum(counts)
+    g = torch.Generator(device=dev)
+    g.manual_seed(4242)
+    base = torch.rand((n, 4096), device=dev, generator=g).topk(k, dim=-1).indices
+    rows, packed, vals = [], [], []
+    for p in range(P):
+        own = torch.rand((n, 4096), device=dev, generator=g).topk(k, dim=-1).indices
+        r = own.clone()
+        r[:, : 4 + p] = base[:, : 4 + p]  # the peers agree on a growing part of every row ...
+        clash = (r[:, 4 + p:, None] == base[:, None, : 4 + p]).any(-1)  # ... and must not repeat it in the rest
+        keep_rows = ~clash.any(dim=1)  # rows whose own part repeats a shared index fall back to `own`
+        r = torch.where(keep_rows[:, None], r, own)
+        rows.append(r)
+        packed.append(tc.pack_12bit_indices(r.contiguous()))
+        vals.append(torch.randn((n, k), device=dev, generator=g) * (1 + p))
+        del own, clash
+    scale = torch.rand((len(shapes), P), device=dev, generator=g) * 0.5 + 0.5
+    outs = [torch.full(s, float("nan"), device=dev) for s in shapes]
+    tc.batch_decompress_decode_batch(tc.TensorBatch(outs), packed, vals, k, scale=scale, use_dct=use_dct)
+    _, b = tcp.basis(64)
+    b = b.to(dev)
+    begin = 0
+    worst = 0.0
+    for t, (shape, cnt) in enumerate(zip(shapes, counts)):
+        sl = slice(begin, begin + cnt)
+        idx = torch.cat([r[sl] for r in rows], dim=1)
+        val = torch.cat([vals[p][sl] * scale[t, p] for p in range(P)], dim=1)
+        dense = torch.zeros((cnt, 4096), device=dev).scatter_reduce_(1, idx, val, reduce="mean", include_self=False)
+        Y, X = shape[0] // 64, shape[1] // 64
+        want = tcp.decode(dense.reshape(Y, X, 64, 64), b, b, use_dct=use_dct)
+        err = (outs[t] - want).abs().max().item() / want.abs().max().item()
+        worst = max(worst, err)
+        assert err <= (TOL if use_dct else 2e-6), (t, shape, err)
+        if not use_dct:
+            assert torch.equal(outs[t] != 0, want != 0)
+        begin += cnt
+    assert worst > 0.0 or not use_dct
