@@ -299,3 +299,37 @@ def test_full_set_aggregate_against_torch_scatter_reduce(dev, use_dct):
             assert torch.equal(outs[t] != 0, want != 0)
         begin += cnt
     assert worst > 0.0 or not use_dct
+
+
+def test_full_set_transform_and_selection_against_torch(dev):
+    # every tensor of the 1B set: the chunked transform against torch's einsum with the reference's
+    # FFT-built basis (the reference's op sequence on the GPU), and the fused kernel's payload against
+    # torch.topk on this library's own coefficients - magnitudes bit for bit, values gathered at the
+    # selected indices bit for bit
+    from oracle import torch_cpu_path as tcp
+
+    grads, k = _set("cfg3_llama1b", dev)
+    batch = tc.TensorBatch(grads)
+    idx12, val = tc.encode_compress_batch(batch, k, use_dct=True)
+    f, _ = tcp.basis(64)
+    f = f.to(dev)
+    worst = 0.0
+    for i, x in enumerate(grads):
+        class M:
+            def named_parameters(self):
+                from types import SimpleNamespace
+                yield "w", SimpleNamespace(requires_grad=True, shape=tuple(x.shape), dtype=torch.float32, device=dev)
+
+        coef = tc.ChunkingTransformer(M(), 64).encode(x, use_dct=True)
+        ref = tcp.encode(x, 64, 64, f, f)
+        err = (coef - ref).abs().max().item() / ref.abs().max().item()
+        worst = max(worst, err)
+        assert err <= TOL, (i, tuple(x.shape), err)
+        rows = coef.reshape(-1, 4096)
+        pi, pv = batch.payload_slice(i, idx12, val, k)
+        pv = pv.reshape(-1, k)
+        sel = tc.unpack_12bit_indices(pi, pv.shape)
+        assert torch.equal(rows.gather(1, sel), pv)
+        top = torch.topk(rows.abs(), k, dim=1, largest=True, sorted=True).values
+        assert torch.equal(top, pv.abs())
+    assert worst > 0.0
