@@ -214,13 +214,18 @@ def main():
     val_buf = torch.empty((n_chunks, k), dtype=torch.float32, device=dev)
     # the norm vectors (64-element chunks) as one flat tensor: one transform + one select launch
     flat_1d = torch.cat(one_d) if one_d else None
+    if flat_1d is not None:  # the norm vectors live back to back, as views of one flat buffer
+        one_d = list(flat_1d.split([g.numel() for g in one_d]))
+    rows_1d = tc.RowBatch(one_d) if one_d and all(g.numel() % 64 == 0 for g in one_d) else None
 
     def encode2d_only():
         tc.encode_compress_batch(batch, k, use_dct=True, idx12=idx_buf, val=val_buf)
 
     def encode_pass():
         encode2d_only()
-        if flat_1d is not None:
+        if rows_1d is not None:
+            tc.encode_compress_rows_batch(rows_1d, k, use_dct=True)
+        elif flat_1d is not None:
             comp.compress(tr.encode(flat_1d, use_dct=True), k)
 
     def encode_per_tensor():
@@ -283,7 +288,7 @@ def main():
     miner = miner_figures(max(3, args.steps // 2), 2) if k <= 64 and args.profile is None else None
 
     # ---- P peers' flat payloads for the aggregation side (peer p = 0.5 shared + own)
-    idxs, vals = [], []
+    idxs, vals, idxs_1d, vals_1d = [], [], [], []
     for p in range(P):
         own = [workloads.student_t3(tuple(g.shape), 1000 * (p + 1) + j, row_scale=True, device=dev).add_(g, alpha=0.5)
                for j, g in enumerate(two_d)]
@@ -292,11 +297,23 @@ def main():
         idxs.append(i12)
         vals.append(v)
         del own
+        if rows_1d is not None:  # the norm vectors' payloads, same recipe
+            own = [workloads.student_t3(tuple(g.shape), 2000 * (p + 1) + j, row_scale=False, device=dev).add_(g, alpha=0.5)
+                   for j, g in enumerate(one_d)]
+            i12, v = tc.encode_compress_rows_batch(tc.RowBatch(own), k, use_dct=True)
+            idxs_1d.append(i12)
+            vals_1d.append(v)
     outs = two_d  # the gradients are not needed any more: decode into their storage
     out_batch = batch
 
-    def aggregate_pass():
+    def aggregate_2d_pass():
         tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, clip_norm=True, use_dct=True)
+
+    def aggregate_pass():
+        aggregate_2d_pass()
+        if rows_1d is not None:
+            tc.batch_decompress_decode_rows_batch(rows_1d, idxs_1d, vals_1d, min(k, 64), clip_norm=True, use_dct=True,
+                                                  validate=False)
 
     scale = tc.peer_clip_scales_batch(out_batch, vals, k)
 
@@ -322,10 +339,12 @@ def main():
         return
     agg_steps = max(3, args.steps // 2)
     agg_ms, agg_wall = event_ms(aggregate_pass, agg_steps, 2)
+    agg2d_ms, _ = event_ms(aggregate_2d_pass, agg_steps, 1)
     aggk_ms, _ = event_ms(aggregate_kernel_only, agg_steps, 1)
     agg_pt_ms, _ = event_ms(aggregate_per_tensor, 3, 1)
     agg_rc_ms, _ = event_ms(aggregate_reference_calls, 3, 1)
-    agg_bytes = n_chunks * (P * 11 * k // 2 + 16384)
+    agg_bytes = n_chunks * (P * 11 * k // 2 + 16384)           # the fused kernel's launch
+    agg_pass_bytes = workloads.aggregate_bytes(shapes, k, P)  # the whole set, norm vectors included
     # validator-side checks on the same payloads: pairwise index overlap, repeats, bounds
     stats = None
     if P <= 32:
@@ -369,8 +388,9 @@ def main():
                    "chunk": 64, "topk": k, "peers": P, "use_dct": True},
         "encode_wall_ms": round(enc_wall, 4),
         "aggregate_ms": round(agg_ms, 4),
-        "aggregate_GBps": round(agg_bytes / (agg_ms * 1e-3) / 1e9, 2),
+        "aggregate_GBps": round(agg_pass_bytes / (agg_ms * 1e-3) / 1e9, 2),
         "aggregate_wall_ms": round(agg_wall, 4),
+        "aggregate_2d_ms": round(agg2d_ms, 4),
         "per_tensor_launches": {"encode_ms": round(enc_pt_ms, 4), "aggregate_ms": round(agg_pt_ms, 4),
                                 "note": "same work as one fused launch per tensor through the reference-shaped API",
                                 "reference_calls_encode_ms": round(enc_rc_ms, 4),

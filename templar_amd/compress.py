@@ -501,7 +501,8 @@ def _aggregate_chunks(idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor]
     return out
 
 
-def _scatter_rows(idx: torch.Tensor, val: torch.Tensor, n_rows: int, kk: int, row_len: int) -> torch.Tensor:
+def _scatter_rows(idx: torch.Tensor, val: torch.Tensor, n_rows: int, kk: int, row_len: int, *,
+                  validate: bool = True) -> torch.Tensor:
     """Generic rows: idx is packed uint8 or int64, val is (rows_sent, kk) with rows_sent <= n_rows
     (torch's scatter lets the index cover fewer rows than the target; the rest stay zero)."""
     if row_len > _lib.TPLR_MAX_ROW:
@@ -523,7 +524,7 @@ def _scatter_rows(idx: torch.Tensor, val: torch.Tensor, n_rows: int, kk: int, ro
         st = lib.tplr_scatter_rows(_ptr(idx) if packed else None, None if packed else _ptr(idx), _ptr(val), n_rows, kk,
                                    row_len, _lib.REDUCE_MEAN, _ptr(out), _ptr(err), _stream(dev))
     _lib.check(st, "tplr_scatter_rows")
-    bad = int(err.item())  # the reference's scatter raises on an out-of-range index as well
+    bad = int(err.item()) if validate else 0  # the reference's scatter raises on an out-of-range index as well
     if bad:
         raise RuntimeError(f"index {bad} is out of bounds for dimension -1 with size {row_len}")
     return out
@@ -1026,6 +1027,114 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
     return idx12, val, quant
 
 
+# ---- the 1-D parameters of a model (norm vectors): rows of 64, a handful of launches for all of them ----
+class RowBatch:
+    """A set of 1-D fp32 device tensors whose lengths are multiples of 64, addressed as one list of
+    rows of 64 elements, tensor by tensor (ChunkingTransformer's 1-D layout, reference :244-251 with
+    a chunk of 64).  The flat payload of the set is indexed by the global row id, like a
+    TensorBatch's by the chunk id: indices of row g at byte g*3k/2, values at float g*k."""
+
+    def __init__(self, tensors: Sequence[torch.Tensor]):
+        if not tensors:
+            raise ValueError("RowBatch needs at least one tensor")
+        dev = tensors[0].device
+        self.offsets: list[int] = []
+        begin = 0
+        for i, t in enumerate(tensors):
+            _need_device(t, "RowBatch")
+            if t.device != dev or t.dtype != torch.float32 or t.dim() != 1 or t.numel() % _CH or not t.is_contiguous():
+                raise ValueError(f"tensor {i}: need fp32, 1-D, contiguous, length divisible by {_CH}, one device")
+            self.offsets.append(begin)
+            begin += t.numel() // _CH
+        self.tensors = list(tensors)
+        self.rows = [t.numel() // _CH for t in tensors]
+        self.total_rows = begin
+        self.device = dev
+        # tensors that lie back to back in one allocation (views of a flat parameter buffer) are
+        # read and written in place, without a gathering copy
+        self.flat = None
+        first = tensors[0]
+        if all(t.untyped_storage().data_ptr() == first.untyped_storage().data_ptr() for t in tensors) and \
+                all(b.data_ptr() == a.data_ptr() + a.numel() * 4 for a, b in zip(tensors, tensors[1:])):
+            self.flat = torch.as_strided(first, (begin * _CH,), (1,))
+        # row -> tensor id, for per-tensor factors applied to flat payloads
+        self.segment = torch.repeat_interleave(torch.arange(len(tensors), device=dev),
+                                               torch.tensor(self.rows, device=dev))
+        # the descriptor table the flat-payload kernels walk: a tensor's rows in place of its chunks
+        import numpy as np
+
+        desc = np.zeros(len(tensors), dtype=np.dtype([("dense", "<u8"), ("ld", "<i8"), ("chunk_begin", "<i8"),
+                                                      ("x_chunks", "<i4"), ("y_chunks", "<i4")]))
+        for i, (b, n) in enumerate(zip(self.offsets, self.rows)):
+            desc[i] = (0, 0, b, n, 1)
+        self.table = torch.from_numpy(desc.view(np.uint8).copy()).to(dev)
+
+    def __len__(self) -> int:
+        return len(self.tensors)
+
+    def payload_slice(self, i: int, idx12: torch.Tensor, val: torch.Tensor, k: int):
+        """Tensor i's part of a flat payload, in the reference's per-parameter form (xshape (rows, 64))."""
+        b, n = self.offsets[i], self.rows[i]
+        return idx12[b * (k // 2) * 3:(b + n) * (k // 2) * 3], val[b:b + n]
+
+
+@torch.no_grad()
+def encode_compress_rows_batch(batch: RowBatch, topk: int, *, use_dct: bool = True):
+    """encode + compress of every 1-D tensor of the set (src/tplr/neurons.py:155-159 per parameter) in
+    three launches: concatenate, 64-point transform of every row, top-k per row.  Returns the flat
+    payload (idx12 uint8, val (total_rows, k)); totalk is 64 for every row."""
+    lib = _lib.load()
+    k = _clamp_k(_CH, topk)
+    dev = batch.device
+    rows = (batch.flat if batch.flat is not None else torch.cat(batch.tensors)).reshape(-1, _CH)
+    if use_dct:
+        coef = torch.empty_like(rows)
+        with _on(dev):
+            st = lib.tplr_dct1d(_ptr(rows), rows.shape[0], 0, _ptr(coef), _stream(dev))
+        _lib.check(st, "tplr_dct1d")
+        rows = coef
+    return _topk_rows(rows, k)
+
+
+@torch.no_grad()
+def batch_decompress_decode_rows_batch(out: RowBatch, idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], k: int,
+                                       *, clip_norm: bool = True, use_dct: bool = True, validate: bool = True) -> None:
+    """batch_decompress + decode (src/tplr/neurons.py:341-367) of every 1-D parameter at once: peer p's
+    flat payload is (idxs[p], vals[p]).  Per parameter and peer the values are clipped to the median
+    norm over the peers (reference :526-556), every row takes the mean over the peers that sent each
+    element (:574-580), the rows go back through the 64-point transform and into the tensors of `out`.
+    The payloads are a few hundred KB: a fixed, small number of launches whatever the number of
+    parameters.  `validate` (default) raises on an index of 64 or more, as torch's scatter does, which
+    costs a synchronisation; without it such entries are dropped."""
+    lib = _lib.load()
+    P, R, T, dev = len(vals), out.total_rows, len(out), out.device
+    for i, v in zip(idxs, vals):
+        if i.dtype != torch.uint8:
+            raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
+        if v.dtype != torch.float32 or v.numel() != R * k or i.numel() * 2 != R * k * 3:
+            raise RuntimeError(f"flat payload mismatch: {i.numel()} index bytes / {v.numel()} values for {R} rows, k={k}")
+    v = torch.stack([x.reshape(R, k) for x in vals])                                  # (P, R, k)
+    if clip_norm:
+        clip = peer_clip_scales_batch(out, [v[p] for p in range(P)], k)               # (T, P), two launches
+        v = v * clip.t()[:, out.segment].unsqueeze(-1)
+    idx = unpack_12bit_indices(torch.cat([i.reshape(-1) for i in idxs]), (P, R, k))   # one launch for all peers
+    cat_i = idx.permute(1, 0, 2).reshape(R, P * k).contiguous()                       # peer order inside a row
+    cat_v = v.permute(1, 0, 2).reshape(R, P * k).contiguous()
+    rows = _scatter_rows(cat_i, cat_v, R, P * k, _CH, validate=validate)
+    if use_dct:
+        dec = out.flat.view(R, _CH) if out.flat is not None else torch.empty_like(rows)
+        with _on(dev):
+            st = lib.tplr_dct1d(_ptr(rows), R, 1, _ptr(dec), _stream(dev))
+        _lib.check(st, "tplr_dct1d")
+        if out.flat is not None:
+            return
+        rows = dec
+    if out.flat is not None:
+        out.flat.copy_(rows.reshape(-1))
+    else:
+        torch._foreach_copy_(out.tensors, list(rows.reshape(-1).split([t.numel() for t in out.tensors])))
+
+
 def check_compressed_indices(param_name: str, idxs, totalk: int, allowed_topk: int | None = None,
                              vals: torch.Tensor | None = None, *, topk_compression: int | None = None) -> None:
     """Validation of one parameter's packed indices as Comms.check_compressed_indices does it
@@ -1303,6 +1412,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

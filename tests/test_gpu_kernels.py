@@ -870,3 +870,53 @@ def test_payload_stage_equals_per_parameter_path(dev, quantized, where):
         tc.PayloadStage(batch, k, 2, quantized=quantized).load(idxs, vals, qps if quantized else None)
     with pytest.raises(IndexError):
         stage.load(idxs[:-1], vals[:-1], qps[:-1] if quantized else None)
+
+
+# ---------------------------------------------------------------- the 1-D parameters as one set
+@pytest.mark.parametrize("use_dct", [True, False])
+def test_row_batch_matches_per_parameter_calls_and_oracle(dev, use_dct):
+    lengths = [64, 2048, 128, 768]
+    P, k = 5, 32
+    comp = tc.TopKCompressor()
+    tr = tc.ChunkingTransformer(_Stub([torch.empty(n) for n in lengths]), 64)
+    grads = [t3((n,), 70 + i).to(dev) * (i + 1) for i, n in enumerate(lengths)]
+    rb = tc.RowBatch(grads)
+    assert rb.total_rows == sum(n // 64 for n in lengths)
+    idx12, val = tc.encode_compress_rows_batch(rb, k, use_dct=use_dct)
+    for i, g in enumerate(grads):
+        wi, wv, xshape, totalk = comp.compress(tr.encode(g, use_dct=use_dct), k)
+        gi, gv = rb.payload_slice(i, idx12, val, k)
+        assert torch.equal(gi, wi) and torch.equal(gv, wv) and totalk == 64 and tuple(xshape) == (lengths[i] // 64, 64)
+    # P peers' flat payloads -> every parameter
+    pay = []
+    for p in range(P):
+        pg = [0.5 * g + t3(tuple(g.shape), 500 + 10 * p + i).to(dev) * (1 + p) for i, g in enumerate(grads)]
+        pay.append(tc.encode_compress_rows_batch(tc.RowBatch(pg), k, use_dct=use_dct))
+    idxs, vals = [a for a, _ in pay], [b for _, b in pay]
+    outs = [torch.full((n,), float("nan"), device=dev) for n in lengths]
+    tc.batch_decompress_decode_rows_batch(tc.RowBatch(outs), idxs, vals, k, use_dct=use_dct)
+    for i, n in enumerate(lengths):
+        sl = [rb.payload_slice(i, idxs[p], vals[p], k) for p in range(P)]
+        pi, pv = [a for a, _ in sl], [b for _, b in sl]
+        norms = torch.stack([torch.norm(v, p=2) for v in pv])  # src/tplr/neurons.py:346
+        dense = comp.batch_decompress(outs[i], pi, pv, (n // 64, 64), 64, block_norms=norms)
+        want = tr.decode(dense, use_dct=use_dct)
+        assert np.abs((outs[i] - want).cpu().numpy()).max() <= 1e-6 * float(want.abs().max())
+        ref = orc.batch_decompress([a.cpu().numpy() for a in pi], [b.cpu().numpy() for b in pv], (n // 64, 64), 64)
+        ref = orc.dct1d(ref, inverse=True) if use_dct else ref
+        assert np.abs(outs[i].cpu().numpy() - ref.reshape(-1)).max() <= 1e-5 * np.abs(ref).max()
+    # the same tensors as views of one flat buffer: read and written in place, same results
+    flat_in = torch.cat(grads)
+    views = list(flat_in.split(lengths))
+    vb = tc.RowBatch(views)
+    assert vb.flat is not None and vb.flat.data_ptr() == flat_in.data_ptr() and rb.flat is None
+    i2, v2 = tc.encode_compress_rows_batch(vb, k, use_dct=use_dct)
+    assert torch.equal(i2, idx12) and torch.equal(v2, val)
+    flat_out = torch.full((sum(lengths),), float("nan"), device=dev)
+    tc.batch_decompress_decode_rows_batch(tc.RowBatch(list(flat_out.split(lengths))), idxs, vals, k, use_dct=use_dct,
+                                          validate=False)
+    assert torch.equal(flat_out, torch.cat(outs))
+    # an index beyond the row length: torch's scatter raises, so does the checked form
+    bad = tc.pack_12bit_indices(torch.full((rb.total_rows, k), 64, dtype=torch.int64, device=dev).contiguous())
+    with pytest.raises(RuntimeError):
+        tc.batch_decompress_decode_rows_batch(tc.RowBatch(outs), [bad] + idxs[1:], vals, k, use_dct=use_dct)
