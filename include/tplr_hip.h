@@ -178,6 +178,17 @@ int tplr_scatter_rows(const uint8_t* d_idx12, const int64_t* d_idx64, const floa
                       int64_t n_rows, int64_t k_per_row, int64_t row_len, int reduce_mode,
                       float* d_out, int32_t* d_err, void* stream);
 
+/* The same for P peers' flat payloads at once, without concatenating them: row g of d_out
+ * (n_rows x row_len) takes the peers' entries for row g in peer order, peer p's values times
+ * d_scale[t * n_peers + p], t the tensor of d_desc (chunk_begin = first row, as for the chunk
+ * batches) that row g belongs to; d_scale NULL = no factors (then d_desc may be NULL).
+ * Replaces batch_decompress (src/tplr/compress.py:483-580) for layouts that are not 64x64 chunks
+ * - the 1-D parameters: rows of 64 - over a whole set of parameters in one launch.  k even;
+ * d_err as above. */
+int tplr_aggregate_rows(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale, int n_peers,
+                        int k, const tplr_tensor_desc* d_desc, int n_tensors, int64_t n_rows, int64_t row_len,
+                        int reduce_mode, float* d_out, int32_t* d_err, void* stream);
+
 /* ---- peer statistics (src/tplr/compress.py:526-535, :553-556) ---------------------
  * d_sumsq[p * n_slices + s] = sum of squares of the s-th of n_slices equal runs of payload p's
  * n values (h_val: HOST array of n_peers DEVICE pointers).  n_slices > 1 lets a few peers with

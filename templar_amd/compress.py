@@ -671,9 +671,32 @@ class TopKCompressor:
                 return LazyAggregate(idxs, vals, scale, xshape, k, normalise, p.dtype)
             out = _aggregate_chunks(idxs, vals, scale, xshape[0], xshape[1], k, normalise=normalise, use_dct=False)
             return out if p.dtype == torch.float32 else out.to(p.dtype)
-        # generic layout (1-D tensors, un-chunked rows): unpack, scale, concatenate in peer order
-        # (reference :559-575), then one row scatter
+        # generic layout (1-D tensors, un-chunked rows)
         n_rows, row_len = _row_layout(xshape)
+        sent = vals[0].numel() // k if k else 0
+        if (not normalise and k >= 2 and k % 2 == 0 and 0 < sent <= n_rows and row_len <= _lib.TPLR_MAX_ROW
+                and len(vals) <= _lib.TPLR_MAX_PEERS and all(v.numel() == sent * k and v.shape[-1] == k for v in vals)
+                and all(i.numel() * 2 == sent * k * 3 for i in idxs)):
+            # all peers in one launch: entries added in peer order, as the concatenation is (reference :559-580)
+            lib = _lib.load()
+            P = len(vals)
+            out = torch.empty((n_rows, row_len), dtype=torch.float32, device=dev)
+            if sent < n_rows:
+                out[sent:].zero_()  # torch's scatter lets the index cover fewer rows than the target
+            err = torch.zeros(1, dtype=torch.int32, device=dev)
+            ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+            vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
+            with _on(dev):
+                st = lib.tplr_aggregate_rows(ip, vp, _ptr(scale), P, k, _ptr(_flat_desc(sent, dev)), 1, sent, row_len,
+                                             _lib.REDUCE_MEAN, _ptr(out), _ptr(err), _stream(dev))
+            _lib.check(st, "tplr_aggregate_rows")
+            bad = int(err.item())  # the reference's scatter raises on an out-of-range index as well
+            if bad:
+                raise RuntimeError(f"index {bad} is out of bounds for dimension -1 with size {row_len}")
+            out = out.reshape(xshape)
+            return out if p.dtype == torch.float32 else out.to(p.dtype)
+        # peers of different sizes, per-row normalisation: unpack, scale, concatenate in peer order
+        # (reference :559-575), then one row scatter
         parts_i, parts_v = [], []
         for pi, (i_data, v) in enumerate(zip(idxs, vals)):
             v2 = v.reshape(-1, v.shape[-1])
@@ -1113,14 +1136,21 @@ def batch_decompress_decode_rows_batch(out: RowBatch, idxs: Sequence[torch.Tenso
             raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
         if v.dtype != torch.float32 or v.numel() != R * k or i.numel() * 2 != R * k * 3:
             raise RuntimeError(f"flat payload mismatch: {i.numel()} index bytes / {v.numel()} values for {R} rows, k={k}")
-    v = torch.stack([x.reshape(R, k) for x in vals])                                  # (P, R, k)
-    if clip_norm:
-        clip = peer_clip_scales_batch(out, [v[p] for p in range(P)], k)               # (T, P), two launches
-        v = v * clip.t()[:, out.segment].unsqueeze(-1)
-    idx = unpack_12bit_indices(torch.cat([i.reshape(-1) for i in idxs]), (P, R, k))   # one launch for all peers
-    cat_i = idx.permute(1, 0, 2).reshape(R, P * k).contiguous()                       # peer order inside a row
-    cat_v = v.permute(1, 0, 2).reshape(R, P * k).contiguous()
-    rows = _scatter_rows(cat_i, cat_v, R, P * k, _CH, validate=validate)
+    vals = [_val_on(x, dev) for x in vals]
+    idxs = [_idx_on(i, dev) for i in idxs]
+    scale = peer_clip_scales_batch(out, vals, k) if clip_norm else None               # (T, P), two launches
+    rows = torch.empty((R, _CH), dtype=torch.float32, device=dev)
+    err = torch.zeros(1, dtype=torch.int32, device=dev) if validate else None
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+    vp = (C.c_void_p * P)(*[x.data_ptr() for x in vals])
+    with _on(dev):
+        st = lib.tplr_aggregate_rows(ip, vp, _ptr(scale), P, k, _ptr(out.table), T, R, _CH, _lib.REDUCE_MEAN, _ptr(rows),
+                                     _ptr(err), _stream(dev))
+    _lib.check(st, "tplr_aggregate_rows")
+    if validate:
+        bad = int(err.item())  # torch's scatter raises on an out-of-range index as well
+        if bad:
+            raise RuntimeError(f"index {bad} is out of bounds for dimension -1 with size {_CH}")
     if use_dct:
         dec = out.flat.view(R, _CH) if out.flat is not None else torch.empty_like(rows)
         with _on(dev):

@@ -1976,6 +1976,126 @@ int tplr_decode_aggregate_batch(const uint8_t* const* h_idx12, const float* cons
                          normalise, use_dct, d_sumsq, stream);
 }
 
+// Rows of any length up to TPLR_MAX_ROW from P peers' flat payloads: row g of the result takes, element
+// by element, the sum (or the mean over the senders) of the peers' entries for row g, each peer's values
+// times its factor for the tensor the row belongs to, added in peer order and, inside a peer, in entry
+// order - the order scatter_reduce_ on the concatenation uses (src/tplr/compress.py:559-580).  One wave
+// per row.  Entries of one peer that name the same element (a top-k has none) are added one after the
+// other; an index outside the row is dropped and reported.
+__global__ __launch_bounds__(64) void k_aggregate_rows(const PeerPtrs pp, const float* __restrict__ scale, int P, int k,
+                                                       const tplr_tensor_desc* __restrict__ table, int n_tensors,
+                                                       int row_len, int reduce_mode, float* __restrict__ out,
+                                                       int32_t* __restrict__ err) {
+    __shared__ float acc[TPLR_MAX_ROW];
+    __shared__ uint32_t cnt[TPLR_MAX_ROW];
+    __shared__ uint32_t tag[TPLR_MAX_ROW];
+    const int lane = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    for (int i = lane; i < row_len; i += 64) {
+        acc[i] = 0.f;
+        cnt[i] = 0;
+    }
+    int t = 0;
+    if (scale && table) {  // the tensor this row belongs to: the last one that begins at or before it
+        int lo = 0, hi = n_tensors;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (table[mid].chunk_begin <= row)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        t = lo;
+    }
+    wave_lds_fence();
+    const int64_t idx_stride = k + (k >> 1);
+    const int batches = (k + 63) >> 6;  // 64 entries at a time
+    // turn `it` = (peer, batch of 64 entries): the entries of the next turn are requested before this
+    // turn's are added, so that a row does not wait for one memory round trip per peer
+    auto fetch = [&](int it, int& me, float& a) {
+        me = -1;
+        a = 0.f;
+        if (it >= P * batches) return;
+        const int p = it / batches, j = (it - p * batches) * 64 + lane;
+        if (j < k) {
+            const gbyte* irow = (const gbyte*)pp.idx[p] + row * idx_stride;
+            const gfloat* vrow = (const gfloat*)pp.val[p] + row * k;
+            const float s = scale ? scale[static_cast<int64_t>(t) * P + p] : 1.0f;
+            me = static_cast<int>(load_idx12(irow, j));
+            a = vrow[j] * s;
+        }
+    };
+    int me_next;
+    float a_next;
+    fetch(0, me_next, a_next);
+    for (int it = 0; it < P * batches; ++it) {
+        int me = me_next;
+        const float a = a_next;
+        fetch(it + 1, me_next, a_next);
+        if (me >= row_len) {
+            if (err) atomicMax(err, me);
+            me = -1;
+        }
+        // the usual case: the 64 entries name distinct elements
+        if (me >= 0) tag[me] = static_cast<uint32_t>(lane);
+        wave_lds_fence();
+        const bool clash = me >= 0 && tag[me] != static_cast<uint32_t>(lane);
+        if (__ballot(clash) == 0) {
+            if (me >= 0) {
+                acc[me] += a;
+                cnt[me] += 1;
+            }
+        } else {
+            // rank among the earlier lanes that name the same element; one rank per turn
+            int rank = 0;
+            for (int i = 0; i < 63; ++i) {
+                const int other = __shfl(me, i);
+                rank += (i < lane && other == me && me >= 0) ? 1 : 0;
+            }
+            int maxrank = rank;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const int o = __shfl_xor(maxrank, off);
+                maxrank = o > maxrank ? o : maxrank;
+            }
+            for (int r = 0; r <= maxrank; ++r) {
+                if (me >= 0 && rank == r) {
+                    acc[me] += a;
+                    cnt[me] += 1;
+                }
+                wave_lds_fence();
+            }
+        }
+        wave_lds_fence();
+    }
+    float* orow = out + row * row_len;
+    for (int i = lane; i < row_len; i += 64) {
+        const uint32_t c = cnt[i];
+        const float v = acc[i];
+        orow[i] = (reduce_mode == TPLR_REDUCE_MEAN && c > 1) ? v / static_cast<float>(c) : v;
+    }
+}
+
+int tplr_aggregate_rows(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale, int n_peers,
+                        int k, const tplr_tensor_desc* d_desc, int n_tensors, int64_t n_rows, int64_t row_len,
+                        int reduce_mode, float* d_out, int32_t* d_err, void* stream) {
+    if (!h_idx12 || !h_val || !d_out || n_peers < 1 || n_rows < 0 || row_len < 1 || k < 2 || (k & 1) ||
+        (reduce_mode != TPLR_REDUCE_MEAN && reduce_mode != TPLR_REDUCE_SUM) || (d_scale && (!d_desc || n_tensors < 1)))
+        return TPLR_E_BADARG;
+    if (n_peers > TPLR_MAX_PEERS || row_len > TPLR_MAX_ROW || k > TPLR_MAX_ROW || n_rows > 0x7fffffff) return TPLR_E_TOOMANY;
+    if (n_rows == 0) return 0;
+    PeerPtrs pp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        pp.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
+        pp.val[p] = p < n_peers ? h_val[p] : nullptr;
+        if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
+    }
+    hipLaunchKernelGGL(k_aggregate_rows, dim3(static_cast<unsigned>(n_rows)), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), pp, d_scale, n_peers, k, d_desc, n_tensors,
+                       static_cast<int>(row_len), reduce_mode, d_out, d_err);
+    return launch_status();
+}
+
 int tplr_scatter_rows(const uint8_t* d_idx12, const int64_t* d_idx64, const float* d_val, int64_t n_rows,
                       int64_t k_per_row, int64_t row_len, int reduce_mode, float* d_out, int32_t* d_err,
                       void* stream) {
