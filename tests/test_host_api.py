@@ -198,6 +198,10 @@ def test_entry_points_reject_bad_arguments_before_any_launch():
     assert lib.tplr_dequantize_peers(ptrs, 2, 6, p, p, 4, ptrs, None) == E.TPLR_E_BADARG       # n not a multiple of 4
     assert lib.tplr_quantize_batch(p, 32, p, 1, 4, C.c_float(6.0), 0, p, p, p, p, p, None) == E.TPLR_E_BADARG  # no slices
     assert lib.tplr_quantize_batch(p + 4, 32, p, 1, 4, C.c_float(6.0), 1, p, p, p, p, p, None) == E.TPLR_E_BADARG
+    assert lib.tplr_aggregate_rows(ptrs, ptrs, None, 2, 31, None, 0, 4, 64, 0, p, None, None) == E.TPLR_E_BADARG
+    assert lib.tplr_aggregate_rows(ptrs, ptrs, p, 2, 32, None, 0, 4, 64, 0, p, None, None) == E.TPLR_E_BADARG  # factors without a table
+    assert lib.tplr_aggregate_rows(many, many, None, 129, 32, None, 0, 4, 64, 0, p, None, None) == E.TPLR_E_TOOMANY
+    assert lib.tplr_aggregate_rows(ptrs, ptrs, None, 2, 32, None, 0, 4, 5000, 0, p, None, None) == E.TPLR_E_TOOMANY
     assert lib.tplr_segment_sumsq(ptrs, 2, 32, p, 1, 0, p, None) == E.TPLR_E_BADARG
     assert lib.tplr_clip_scales(None, 2, 0, p, None, None) == E.TPLR_E_BADARG
     for code in (0, E.TPLR_E_BADARG, E.TPLR_E_ODD, E.TPLR_E_SHAPE, E.TPLR_E_TOOMANY, 1):
