@@ -1095,6 +1095,13 @@ class RowBatch:
     def __len__(self) -> int:
         return len(self.tensors)
 
+    @property
+    def total_chunks(self) -> int:  # the flat-payload routines count rows of payload, whatever their length
+        return self.total_rows
+
+    def xshape(self, i: int) -> tuple[int, int]:
+        return (self.rows[i], _CH)
+
     def payload_slice(self, i: int, idx12: torch.Tensor, val: torch.Tensor, k: int):
         """Tensor i's part of a flat payload, in the reference's per-parameter form (xshape (rows, 64))."""
         b, n = self.offsets[i], self.rows[i]
@@ -1163,6 +1170,48 @@ def batch_decompress_decode_rows_batch(out: RowBatch, idxs: Sequence[torch.Tenso
         out.flat.copy_(rows.reshape(-1))
     else:
         torch._foreach_copy_(out.tensors, list(rows.reshape(-1).split([t.numel() for t in out.tensors])))
+
+
+@torch.no_grad()
+def error_feedback_step_rows_batch(ef: RowBatch, grad: RowBatch, decay: float, topk: int, *, use_dct: bool = True,
+                                   compressor: "TopKCompressor | None" = None, null_round: bool = False):
+    """error_feedback_step_batch for the 1-D parameters: the loop body of src/tplr/neurons.py:147-171
+    for all of them in about ten launches.  Returns (idx12, val, quant) as its 2-D counterpart does."""
+    lib = _lib.load()
+    if len(ef) != len(grad) or ef.rows != grad.rows:
+        raise ValueError("error-feedback and gradient sets differ in shape")
+    k = _clamp_k(_CH, topk)
+    dev, R, T = ef.device, ef.total_rows, len(ef)
+    if null_round:
+        torch._foreach_zero_(ef.tensors)                       # :148-149
+    elif ef.flat is not None and grad.flat is not None:
+        ef.flat.mul_(decay).add_(grad.flat)                    # :151-152, two roundings
+    else:
+        torch._foreach_mul_(ef.tensors, decay)
+        torch._foreach_add_(ef.tensors, grad.tensors)
+    idx12, val = encode_compress_rows_batch(ef, k, use_dct=use_dct)      # :155-159
+    quant, sent = None, val
+    if compressor is not None and compressor.use_quantization:
+        codes, shift, scale, lookup = quantize_batch(ef, val, k, compressor.n_bins, compressor.range_in_sigmas)
+        sent = dequantize_batch(ef, codes.reshape(-1), None, k, tables=(lookup, shift))
+        half = compressor.n_bins // 2
+        quant = [(codes[b:b + n], (shift[i], sc, half, lookup[i], torch.float32))
+                 for i, (b, n, sc) in enumerate(zip(ef.offsets, ef.rows, scale.tolist()))]
+    # :162-171: the sent part back through decompress + decode, subtracted from the error feedback
+    rows = torch.empty((R, _CH), dtype=torch.float32, device=dev)
+    ip, vp = (C.c_void_p * 1)(idx12.data_ptr()), (C.c_void_p * 1)(sent.data_ptr())
+    with _on(dev):
+        st = lib.tplr_aggregate_rows(ip, vp, None, 1, k, None, 0, R, _CH, _lib.REDUCE_MEAN, _ptr(rows), None, _stream(dev))
+        _lib.check(st, "tplr_aggregate_rows")
+        if use_dct:
+            dec = torch.empty_like(rows)
+            _lib.check(lib.tplr_dct1d(_ptr(rows), R, 1, _ptr(dec), _stream(dev)), "tplr_dct1d")
+            rows = dec
+    if ef.flat is not None:
+        ef.flat.sub_(rows.reshape(-1))
+    else:
+        torch._foreach_sub_(ef.tensors, list(rows.reshape(-1).split([t.numel() for t in ef.tensors])))
+    return idx12, val, quant
 
 
 def check_compressed_indices(param_name: str, idxs, totalk: int, allowed_topk: int | None = None,
@@ -1240,19 +1289,24 @@ def quantize_batch(batch: TensorBatch, val: torch.Tensor, k: int, n_bins: int = 
 
 
 @torch.no_grad()
-def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[QuantParamsT], k: int,
-                     out: torch.Tensor | None = None) -> torch.Tensor:
+def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[QuantParamsT] | None, k: int,
+                     out: torch.Tensor | None = None, *, tables: tuple[torch.Tensor, torch.Tensor] | None = None
+                     ) -> torch.Tensor:
     """One peer's flat payload of 8-bit codes -> fp32 values (total_chunks, k), every parameter
     with its own (shift, lookup): TopKCompressor.maybe_dequantize_values' per-parameter loop
     (reference :646-696, src/tplr/neurons.py:325) in one launch.  qparams[i] is parameter i's
     5-tuple as the reference's compress returns it."""
     lib = _lib.load()
     dev, n = batch.device, batch.total_chunks
-    if len(qparams) != len(batch):
+    if tables is None and len(qparams) != len(batch):
         raise IndexError(f"Mismatch in val lengths: dequant({len(qparams)}) vs original({len(batch)})")
     if codes.dtype != torch.uint8 or codes.numel() != n * k:
         raise RuntimeError(f"{codes.numel()} codes of {codes.dtype} for {n} chunks of k={k}")
-    lookup, shift, n_bins = _qparam_tables(qparams, dev)
+    if tables is not None:  # (lookup (T, n_bins), shift (T,)) already on the device, as quantize_batch returns them
+        lookup, shift = tables
+        n_bins = int(lookup.shape[1])
+    else:
+        lookup, shift, n_bins = _qparam_tables(qparams, dev)
     if out is None:
         out = torch.empty((n, k), dtype=torch.float32, device=dev)
     with _on(dev):
@@ -1442,6 +1496,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

@@ -920,3 +920,44 @@ def test_row_batch_matches_per_parameter_calls_and_oracle(dev, use_dct):
     bad = tc.pack_12bit_indices(torch.full((rb.total_rows, k), 64, dtype=torch.int64, device=dev).contiguous())
     with pytest.raises(RuntimeError):
         tc.batch_decompress_decode_rows_batch(tc.RowBatch(outs), [bad] + idxs[1:], vals, k, use_dct=use_dct)
+
+
+@pytest.mark.parametrize("use_dct,bins,flat", [(True, 0, False), (True, 4, True), (False, 256, False), (False, 0, True)])
+def test_error_feedback_step_for_the_1d_parameters(dev, use_dct, bins, flat):
+    # src/tplr/neurons.py:147-171 per parameter, restated with the oracle's pieces on rows of 64
+    lengths, k, decay = [128, 64, 1024], 32, 0.9
+    efs = [t3((n,), 300 + i) for i, n in enumerate(lengths)]
+    grads = [t3((n,), 310 + i) * 0.5 for i, n in enumerate(lengths)]
+    if flat:
+        fe, fg = torch.cat(efs).to(dev), torch.cat(grads).to(dev)
+        d_ef, d_gr = list(fe.split(lengths)), list(fg.split(lengths))
+    else:
+        d_ef, d_gr = [e.clone().to(dev) for e in efs], [g.to(dev) for g in grads]
+    comp = tc.TopKCompressor(use_quantization=bins > 0, quantization_bins=bins or 256, quantization_range=6)
+    eb, gb = tc.RowBatch(d_ef), tc.RowBatch(d_gr)
+    assert (eb.flat is not None) == flat
+    idx12, val, quant = tc.error_feedback_step_rows_batch(eb, gb, decay, k, use_dct=use_dct, compressor=comp)
+    assert (quant is None) == (bins == 0)
+    for i, n in enumerate(lengths):
+        acc = ((efs[i] * decay) + grads[i]).numpy()
+        rows = acc.reshape(-1, 64)
+        coef = orc.dct1d(rows) if use_dct else rows
+        got_i, got_v = eb.payload_slice(i, idx12, val, k)
+        # selection on the device's own coefficients (its transform differs from the oracle's in the last bits)
+        dev_coef = tc.ChunkingTransformer(_Stub([torch.empty(n)]), 64).encode(torch.from_numpy(acc).to(dev), use_dct=use_dct)
+        assert np.abs(dev_coef.cpu().numpy() - coef).max() <= TOL * np.abs(coef).max()
+        want_i, want_v = orc.topk_rows(dev_coef.cpu().numpy(), k)
+        assert np.array_equal(tc.unpack_12bit_indices(got_i, got_v.shape).cpu().numpy(), want_i)
+        assert np.array_equal(got_v.cpu().numpy(), want_v)
+        sent = want_v
+        if bins:
+            wq, wqp = orc.quantize(want_v, bins, 6.0)
+            assert np.array_equal(quant[i][0].cpu().numpy(), wq) and quant[i][1][1] == wqp[1]
+            sent = orc.dequantize(wq, wqp)
+        dense = orc.decompress(orc.pack12(want_i), sent, (n // 64, 64), 64)
+        recon = orc.dct1d(dense, inverse=True) if use_dct else dense
+        want_new = acc - recon.reshape(-1)
+        assert np.abs(d_ef[i].cpu().numpy() - want_new).max() <= TOL * np.abs(acc).max()
+    # a null round clears the error feedback and sends zeros
+    i0, v0, _ = tc.error_feedback_step_rows_batch(eb, gb, decay, k, use_dct=use_dct, null_round=True)
+    assert float(v0.abs().max()) == 0.0 and all(float(e.abs().max()) == 0.0 for e in d_ef)
