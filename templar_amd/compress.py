@@ -906,6 +906,11 @@ class TensorBatch:
         t = self.tensors[i]
         return (t.shape[0] // _CH, t.shape[1] // _CH, _CH, _CH)
 
+    def payload_rows(self, i: int) -> int:
+        """Rows of payload (chunks) of tensor i."""
+        t = self.tensors[i]
+        return (t.shape[0] // _CH) * (t.shape[1] // _CH)
+
     def payload_slice(self, i: int, idx12: torch.Tensor, val: torch.Tensor, k: int):
         """Tensor i's part of a flat payload, in the reference's per-parameter form."""
         y, x, _, _ = self.xshape(i)
@@ -1101,6 +1106,9 @@ class RowBatch:
 
     def xshape(self, i: int) -> tuple[int, int]:
         return (self.rows[i], _CH)
+
+    def payload_rows(self, i: int) -> int:
+        return self.rows[i]
 
     def payload_slice(self, i: int, idx12: torch.Tensor, val: torch.Tensor, k: int):
         """Tensor i's part of a flat payload, in the reference's per-parameter form (xshape (rows, 64))."""
@@ -1347,7 +1355,7 @@ class PayloadStage:
         self.dev = torch.empty(max_peers * self.stride, dtype=torch.uint8, device=batch.device)
         self.values = torch.empty((max_peers, n, k), dtype=torch.float32, device=batch.device) if quantized else None
         self._copied: torch.cuda.Event | None = None  # the last host-to-device copy out of `host`
-        self._val_sizes = [batch.xshape(i)[0] * batch.xshape(i)[1] * k for i in range(len(batch))]
+        self._val_sizes = [batch.payload_rows(i) * k for i in range(len(batch))]
         self._idx_sizes = [v // 2 * 3 for v in self._val_sizes]
         self._threads = max(1, min(64, host_threads if host_threads else min(8, os.cpu_count() or 1)))
 

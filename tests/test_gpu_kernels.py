@@ -958,6 +958,19 @@ def test_error_feedback_step_for_the_1d_parameters(dev, use_dct, bins, flat):
         recon = orc.dct1d(dense, inverse=True) if use_dct else dense
         want_new = acc - recon.reshape(-1)
         assert np.abs(d_ef[i].cpu().numpy() - want_new).max() <= TOL * np.abs(acc).max()
+    if bins:
+        # the payloads as a receiver holds them (per-parameter host lists) staged flat again
+        T = len(lengths)
+        h_idx = [[eb.payload_slice(i, idx12, val, k)[0].cpu()] for i in range(T)]
+        h_val = [[quant[i][0].cpu()] for i in range(T)]
+        h_qp = [[(quant[i][1][0].cpu(), quant[i][1][1], quant[i][1][2], quant[i][1][3].cpu(), torch.float32)] for i in range(T)]
+        fi, fv = tc.PayloadStage(eb, k, 2, quantized=True).load(h_idx, h_val, h_qp)
+        assert torch.equal(fi[0], idx12)
+        for i in range(T):
+            b0 = eb.offsets[i]
+            want = orc.dequantize(quant[i][0].cpu().numpy(), (float(quant[i][1][0]), quant[i][1][1], quant[i][1][2],
+                                                                quant[i][1][3].cpu().numpy()))
+            assert np.array_equal(fv[0][b0:b0 + eb.rows[i]].cpu().numpy(), want)
     # a null round clears the error feedback and sends zeros
     i0, v0, _ = tc.error_feedback_step_rows_batch(eb, gb, decay, k, use_dct=use_dct, null_round=True)
     assert float(v0.abs().max()) == 0.0 and all(float(e.abs().max()) == 0.0 for e in d_ef)
