@@ -1444,11 +1444,11 @@ class PayloadStage:
 
 
 @torch.no_grad()
-def index_stats_batch(batch: "TensorBatch | Sequence[int]", idxs: Sequence[torch.Tensor], k: int):
+def index_stats_batch(batch: "TensorBatch | RowBatch | Sequence[int]", idxs: Sequence[torch.Tensor], k: int):
     """Checks on P peers' packed index streams in one launch.
 
-    `batch` is a TensorBatch (rows = its 64x64 chunks), or a list of row counts per parameter
-    for payloads whose rows are not chunks.  Returns (pair, dup, top):
+    `batch` is a TensorBatch (rows = its 64x64 chunks), a RowBatch, or a list of row counts per
+    parameter for payloads whose rows are not chunks.  Returns (pair, dup, top):
       pair (T, P, P) int64: pair[t, i, j] for i < j = entries of peer i that also occur in the same
           row of peer j, summed over parameter t's rows - what check_uid_index_overlap
           (src/tplr/neurons.py:1373-1378) sums before dividing by k and averaging over rows;
@@ -1463,7 +1463,7 @@ def index_stats_batch(batch: "TensorBatch | Sequence[int]", idxs: Sequence[torch
         raise NotImplementedError(f"{P} peers: the index statistics kernel takes up to 32")
     dev = idxs[0].device
     _need_device(idxs[0], "index_stats_batch")
-    if isinstance(batch, TensorBatch):
+    if isinstance(batch, (TensorBatch, RowBatch)):
         table, T, total = batch.table, len(batch), batch.total_chunks
     else:
         counts = [int(c) for c in batch]

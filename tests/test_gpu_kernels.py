@@ -905,6 +905,10 @@ def test_row_batch_matches_per_parameter_calls_and_oracle(dev, use_dct):
         ref = orc.batch_decompress([a.cpu().numpy() for a in pi], [b.cpu().numpy() for b in pv], (n // 64, 64), 64)
         ref = orc.dct1d(ref, inverse=True) if use_dct else ref
         assert np.abs(outs[i].cpu().numpy() - ref.reshape(-1)).max() <= 1e-5 * np.abs(ref).max()
+    # index statistics take the row batch as they take a chunk batch
+    pair, dup, top = tc.index_stats_batch(rb, idxs, k)
+    pair2, dup2, top2 = tc.index_stats_batch(rb.rows, idxs, k)
+    assert torch.equal(pair, pair2) and torch.equal(dup, dup2) and torch.equal(top, top2) and int(top.max()) < 64
     # the same tensors as views of one flat buffer: read and written in place, same results
     flat_in = torch.cat(grads)
     views = list(flat_in.split(lengths))
