@@ -189,6 +189,11 @@ int tplr_aggregate_rows(const uint8_t* const* h_idx12, const float* const* h_val
                         int k, const tplr_tensor_desc* d_desc, int n_tensors, int64_t n_rows, int64_t row_len,
                         int reduce_mode, float* d_out, int32_t* d_err, void* stream);
 
+/* The elementwise steps of the miner's loop body on a flat run of n values (the 1-D parameters):
+ * subtract == 0: d_a <- d_a * decay + d_b, two roundings, as mul_ then add_
+ * (src/tplr/neurons.py:151-152); subtract != 0: d_a <- d_a - d_b (:171). */
+int tplr_flat_update(float* d_a, const float* d_b, int64_t n, float decay, int subtract, void* stream);
+
 /* ---- peer statistics (src/tplr/compress.py:526-535, :553-556) ---------------------
  * d_sumsq[p * n_slices + s] = sum of squares of the s-th of n_slices equal runs of payload p's
  * n values (h_val: HOST array of n_peers DEVICE pointers).  n_slices > 1 lets a few peers with

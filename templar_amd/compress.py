@@ -1190,14 +1190,17 @@ def error_feedback_step_rows_batch(ef: RowBatch, grad: RowBatch, decay: float, t
         raise ValueError("error-feedback and gradient sets differ in shape")
     k = _clamp_k(_CH, topk)
     dev, R, T = ef.device, ef.total_rows, len(ef)
+    # tensors that are not views of one buffer are gathered into one, worked on there and copied back
+    ef_flat = ef.flat if ef.flat is not None else torch.cat(ef.tensors)
     if null_round:
-        torch._foreach_zero_(ef.tensors)                       # :148-149
-    elif ef.flat is not None and grad.flat is not None:
-        ef.flat.mul_(decay).add_(grad.flat)                    # :151-152, two roundings
+        ef_flat.zero_()                                        # :148-149
     else:
-        torch._foreach_mul_(ef.tensors, decay)
-        torch._foreach_add_(ef.tensors, grad.tensors)
-    idx12, val = encode_compress_rows_batch(ef, k, use_dct=use_dct)      # :155-159
+        g_flat = grad.flat if grad.flat is not None else torch.cat(grad.tensors)
+        with _on(dev):                                         # :151-152, two roundings
+            _lib.check(lib.tplr_flat_update(_ptr(ef_flat), _ptr(g_flat), ef_flat.numel(), C.c_float(decay), 0,
+                                            _stream(dev)), "tplr_flat_update")
+    work = ef if ef.flat is not None else RowBatch(list(ef_flat.split([t.numel() for t in ef.tensors])))
+    idx12, val = encode_compress_rows_batch(work, k, use_dct=use_dct)    # :155-159
     quant, sent = None, val
     if compressor is not None and compressor.use_quantization:
         codes, shift, scale, lookup = quantize_batch(ef, val, k, compressor.n_bins, compressor.range_in_sigmas)
@@ -1215,10 +1218,10 @@ def error_feedback_step_rows_batch(ef: RowBatch, grad: RowBatch, decay: float, t
             dec = torch.empty_like(rows)
             _lib.check(lib.tplr_dct1d(_ptr(rows), R, 1, _ptr(dec), _stream(dev)), "tplr_dct1d")
             rows = dec
-    if ef.flat is not None:
-        ef.flat.sub_(rows.reshape(-1))
-    else:
-        torch._foreach_sub_(ef.tensors, list(rows.reshape(-1).split([t.numel() for t in ef.tensors])))
+        _lib.check(lib.tplr_flat_update(_ptr(ef_flat), _ptr(rows), ef_flat.numel(), C.c_float(0.0), 1, _stream(dev)),
+                   "tplr_flat_update")
+    if ef.flat is None:
+        torch._foreach_copy_(ef.tensors, list(ef_flat.split([t.numel() for t in ef.tensors])))
     return idx12, val, quant
 
 

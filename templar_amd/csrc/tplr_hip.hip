@@ -2096,6 +2096,35 @@ int tplr_aggregate_rows(const uint8_t* const* h_idx12, const float* const* h_val
     return launch_status();
 }
 
+// Momentum update and error-feedback subtraction on a flat run of values (the 1-D parameters, which do not
+// go through the chunk kernels): a <- a * decay + b with two roundings, as mul_ then add_
+// (src/tplr/neurons.py:151-152), or a <- a - b (:171).
+__global__ __launch_bounds__(256) void k_flat_update(float* __restrict__ a, const float* __restrict__ b, int64_t n,
+                                                     float decay, int subtract) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+        const float x = a[i], y = b[i];
+        float r;
+        if (subtract) {
+            r = x - y;
+        } else {
+            const float m = x * decay;
+            r = m + y;
+        }
+        a[i] = r;
+    }
+}
+
+int tplr_flat_update(float* d_a, const float* d_b, int64_t n, float decay, int subtract, void* stream) {
+    if (n < 0 || (n > 0 && (!d_a || !d_b))) return TPLR_E_BADARG;
+    if (n == 0) return 0;
+    int64_t blocks = (n + 255) / 256;
+    blocks = blocks > 4096 ? 4096 : blocks;
+    hipLaunchKernelGGL(k_flat_update, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       d_a, d_b, n, decay, subtract);
+    return launch_status();
+}
+
 int tplr_scatter_rows(const uint8_t* d_idx12, const int64_t* d_idx64, const float* d_val, int64_t n_rows,
                       int64_t k_per_row, int64_t row_len, int reduce_mode, float* d_out, int32_t* d_err,
                       void* stream) {
