@@ -751,6 +751,10 @@ class TopKCompressor:
     def _dequantize_values(self, val: torch.Tensor, qparams: QuantParamsT) -> torch.Tensor:
         if val.dtype != torch.uint8:
             return val
+        if val.is_cuda:
+            fast = self._dequantize_peers([val], [qparams], val.device)
+            if fast is not None:
+                return fast[0]
         shift, _, _, lookup, orig_dtype = qparams
         if isinstance(lookup, torch.Tensor):
             lookup = lookup.to(val.device)
