@@ -252,19 +252,18 @@ def test_full_size_index_statistics_against_bitmaps(dev, P, k):
         assert torch.equal(top[:, p].long(), want_top)
 
 
-@pytest.mark.parametrize("use_dct", [False, True])
-def test_full_set_aggregate_against_torch_scatter_reduce(dev, use_dct):
+@pytest.mark.parametrize("use_dct,P,k", [(False, 15, 32), (True, 15, 32), (False, 20, 64), (True, 20, 64), (True, 31, 32)])
+def test_full_set_aggregate_against_torch_scatter_reduce(dev, use_dct, P, k):
     # the 1B set, 15 peers, every chunk: torch's own scatter_reduce_(mean, include_self=False) on the
     # concatenated payloads (the reference's op sequence, src/tplr/compress.py:559-580, run on the GPU),
     # then its einsum decode, against the one-launch aggregate
     from oracle import torch_cpu_path as tcp
 
-    P, k = 15, 32
     shapes = [s for s in workloads.CONFIGS["cfg3_llama1b"]["shapes"] if len(s) == 2]
     counts = [(a // 64) * (b // 64) for a, b in shapes]
     n = sum(counts)
     g = torch.Generator(device=dev)
-    g.manual_seed(4242)
+    g.manual_seed(4242 + P + k)
     base = torch.rand((n, 4096), device=dev, generator=g).topk(k, dim=-1).indices
     rows, packed, vals = [], [], []
     for p in range(P):
