@@ -295,7 +295,12 @@ def test_full_set_aggregate_against_torch_scatter_reduce(dev, use_dct, P, k):
         worst = max(worst, err)
         assert err <= (TOL if use_dct else 2e-6), (t, shape, err)
         if not use_dct:
-            assert torch.equal(outs[t] != 0, want != 0)
+            # elements no peer sent are exactly zero (torch adds with atomics in no fixed order, so an
+            # element whose contributions cancel may come out as 0 there and as a last-bit residue
+            # here, or the other way round: the pattern is taken from the indices, not from the values)
+            sent = torch.zeros((cnt, 4096), dtype=torch.bool, device=dev).scatter_(1, idx, True)
+            sent = sent.reshape(Y, X, 64, 64).permute(0, 2, 1, 3).reshape(Y * 64, X * 64)
+            assert float(outs[t][~sent].abs().max()) == 0.0
         begin += cnt
     assert worst > 0.0 or not use_dct
 
