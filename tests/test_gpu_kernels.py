@@ -978,3 +978,57 @@ def test_error_feedback_step_for_the_1d_parameters(dev, use_dct, bins, flat):
     # a null round clears the error feedback and sends zeros
     i0, v0, _ = tc.error_feedback_step_rows_batch(eb, gb, decay, k, use_dct=use_dct, null_round=True)
     assert float(v0.abs().max()) == 0.0 and all(float(e.abs().max()) == 0.0 for e in d_ef)
+
+
+# ---------------------------------------------------------------- under stream capture
+def test_whole_set_calls_replay_from_a_captured_graph(dev):
+    # the library allocates nothing and keeps no state: the whole-set launches can be recorded once
+    # and replayed.  Three replays with new data in the same buffers, each against the eager calls.
+    shapes = [(128, 192), (64, 64), (256, 128)]
+    k, P = 32, 3
+    grads = [torch.zeros(s, device=dev) for s in shapes]
+    batch = tc.TensorBatch(grads)
+    n = batch.total_chunks
+    idx12 = torch.zeros(n * (k // 2) * 3, dtype=torch.uint8, device=dev)
+    val = torch.zeros((n, k), device=dev)
+    peer_idx = [torch.zeros_like(idx12) for _ in range(P)]
+    peer_val = [torch.zeros_like(val) for _ in range(P)]
+    outs = [torch.zeros(s, device=dev) for s in shapes]
+    out_batch = tc.TensorBatch(outs)
+
+    def fill(seed):
+        for i, g in enumerate(grads):
+            g.copy_(t3(tuple(g.shape), seed + i, row_scale=True).to(dev))
+        for p in range(P):
+            pg = [0.5 * g + t3(tuple(g.shape), seed + 100 * (p + 1) + i, row_scale=True).to(dev) for i, g in enumerate(grads)]
+            a, b = tc.encode_compress_batch(tc.TensorBatch(pg), k)
+            peer_idx[p].copy_(a)
+            peer_val[p].copy_(b)
+
+    def work():
+        tc.encode_compress_batch(batch, k, idx12=idx12, val=val)
+        tc.batch_decompress_decode_batch(out_batch, peer_idx, peer_val, k, clip_norm=True)
+
+    fill(1)
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            work()  # warm-up outside the capture (first-use occupancy queries, allocator pools)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        work()
+    for rep in range(3):
+        fill(1000 * (rep + 2))
+        work()  # eager
+        torch.cuda.synchronize()
+        want = (idx12.clone(), val.clone(), [o.clone() for o in outs])
+        idx12.zero_(), val.zero_()
+        for o in outs:
+            o.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(idx12, want[0]) and torch.equal(val, want[1])
+        assert all(torch.equal(a, b) for a, b in zip(outs, want[2]))
