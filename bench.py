@@ -343,6 +343,17 @@ def main():
     aggk_ms, _ = event_ms(aggregate_kernel_only, agg_steps, 1)
     agg_pt_ms, _ = event_ms(aggregate_per_tensor, 3, 1)
     agg_rc_ms, _ = event_ms(aggregate_reference_calls, 3, 1)
+    # the same per-parameter loop recorded once into a HIP graph and replayed: what is left is device time
+    side_stream = torch.cuda.Stream(device=dev)
+    side_stream.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side_stream):
+        aggregate_per_tensor()
+    torch.cuda.current_stream(dev).wait_stream(side_stream)
+    torch.cuda.synchronize()
+    per_tensor_graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(per_tensor_graph):
+        aggregate_per_tensor()
+    agg_graph_ms, _ = event_ms(per_tensor_graph.replay, 5, 1)
     agg_bytes = n_chunks * (P * 11 * k // 2 + 16384)           # the fused kernel's launch
     agg_pass_bytes = workloads.aggregate_bytes(shapes, k, P)  # the whole set, norm vectors included
     # validator-side checks on the same payloads: pairwise index overlap, repeats, bounds
@@ -393,6 +404,7 @@ def main():
         "aggregate_2d_ms": round(agg2d_ms, 4),
         "per_tensor_launches": {"encode_ms": round(enc_pt_ms, 4), "aggregate_ms": round(agg_pt_ms, 4),
                                 "note": "same work as one fused launch per tensor through the reference-shaped API",
+                                "aggregate_graph_replay_ms": round(agg_graph_ms, 4),
                                 "reference_calls_encode_ms": round(enc_rc_ms, 4),
                                 "reference_calls_aggregate_ms": round(agg_rc_ms, 4),
                                 "reference_calls_note": "the reference's unchanged call sites: encode then compress, "
