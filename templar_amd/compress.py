@@ -1366,6 +1366,44 @@ class PayloadStage:
         self._idx_sizes = [v // 2 * 3 for v in self._val_sizes]
         self._threads = max(1, min(64, host_threads if host_threads else min(8, os.cpu_count() or 1)))
 
+    @torch.no_grad()
+    def offload(self, n_peers: int) -> None:
+        """The staged window back into the pinned host buffer in one copy (what
+        offload_gather_results, neurons/validator.py:94-160, does tensor by tensor to free the device
+        during evaluation).  The device buffer stays allocated; its contents may be overwritten
+        until `reload`."""
+        n = n_peers * self.stride
+        with _on(self.dev.device):
+            self.host[:n].copy_(self.dev[:n], non_blocking=True)
+            self._copied = torch.cuda.Event()
+            self._copied.record()
+
+    @torch.no_grad()
+    def reload(self, n_peers: int):
+        """The offloaded window onto the device again (neurons/validator.py:162-219), one copy; returns
+        the lists `load` returned.  De-quantised values are rebuilt by the caller's next `load` only when
+        the stage holds codes: here the codes come back and are expanded again."""
+        n = n_peers * self.stride
+        with _on(self.dev.device):
+            self.dev[:n].copy_(self.host[:n], non_blocking=True)
+        out_i, out_v = [], []
+        for p in range(n_peers):
+            ri, rv = self._regions(self.dev, p)
+            out_i.append(ri)
+            out_v.append(rv.view(-1, self.k))
+        if not self.quantized:
+            return out_i, out_v
+        lookup, shift = self._tables
+        lib = _lib.load()
+        dev, T, n_rows = self.dev.device, len(self.batch), self.batch.total_chunks
+        with _on(dev):
+            for p in range(n_peers):
+                st = lib.tplr_dequantize_batch(_ptr(out_v[p]), _ptr(lookup[p * T:(p + 1) * T]), _ptr(shift[p * T:(p + 1) * T]),
+                                               int(lookup.shape[1]), self.k, _ptr(self.batch.table), T, n_rows,
+                                               _ptr(self.values[p]), _stream(dev))
+                _lib.check(st, "tplr_dequantize_batch")
+        return out_i, [self.values[p] for p in range(n_peers)]
+
     def _regions(self, buf: torch.Tensor, p: int) -> tuple[torch.Tensor, torch.Tensor]:
         b = p * self.stride
         idx = buf[b:b + self.idx_bytes]

@@ -866,6 +866,15 @@ def test_payload_stage_equals_per_parameter_path(dev, quantized, where):
             ref = orc.decode2d(orc.batch_decompress([a.cpu().numpy() for a in di], [b.cpu().numpy() for b in dv],
                                                     batch.xshape(i), 4096), use_dct=True)
             assert np.abs(outs[i].cpu().numpy() - ref).max() <= 1e-5 * np.abs(ref).max()
+    # off the device and back (neurons/validator.py:94-219): one copy each way
+    keep_i, keep_v = [t.clone() for t in fi], [t.clone() for t in fv]
+    stage.offload(P)
+    torch.cuda.synchronize()
+    stage.dev.zero_()
+    if quantized:
+        stage.values.zero_()
+    ri, rv = stage.reload(P)
+    assert all(torch.equal(a, b) for a, b in zip(ri, keep_i)) and all(torch.equal(a, b) for a, b in zip(rv, keep_v))
     with pytest.raises(ValueError):
         tc.PayloadStage(batch, k, 2, quantized=quantized).load(idxs, vals, qps if quantized else None)
     with pytest.raises(IndexError):
