@@ -4,7 +4,8 @@
  *
  * Conventions
  *   - every pointer named d_* is DEVICE memory owned by the caller; the library
- *     allocates nothing and keeps no state between calls;
+ *     allocates nothing and keeps no state between calls (one exception, stated where
+ *     it is declared: tplr_quantize_batch_static works in a static device array);
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); all
  *     work is enqueued on it and the call returns without synchronising;
  *   - return value: 0 = ok, negative = TPLR_E_* (bad argument, nothing launched),
@@ -30,6 +31,7 @@ extern "C" {
 #define TPLR_E_ODD      (-2) /* number of 12-bit indices is odd                        */
 #define TPLR_E_SHAPE    (-3) /* dimension not a multiple of the chunk size             */
 #define TPLR_E_TOOMANY  (-4) /* more peers / larger row than the kernel supports       */
+#define TPLR_E_WORKSPACE (-5) /* needs more workspace than the library's static scratch */
 
 #define TPLR_CHUNK        64   /* chunk edge handled by the factorised transform       */
 #define TPLR_MAX_PEERS    128  /* peers per tplr_decode_aggregate call                 */
@@ -288,6 +290,21 @@ int tplr_dequantize_peers(const uint8_t* const* h_codes, int n_peers, int64_t n,
 int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
                         float range_in_sigmas, int n_slices, double* d_work, uint8_t* d_codes, float* d_shift,
                         float* d_scale, float* d_lookup, void* stream);
+
+/* tplr_quantize_batch for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc); it has no counterpart in the
+ * reference.  Same arguments and results without d_work: the partial sums go through a static
+ * device array inside the library, TPLR_STATIC_WORK_DOUBLES doubles (tplr_static_work_bytes()
+ * bytes, about 8 MB, held on every GPU the library runs on until the process ends).  The call
+ * allocates and frees nothing.  n_tensors * n_slices * (2 + 2 * n_bins) doubles must fit:
+ * otherwise TPLR_E_WORKSPACE and nothing is launched.  Every call on a GPU uses that GPU's one
+ * array, whose contents are irrelevant on entry: calls that overlap on one GPU (two streams, two
+ * threads) race and must be serialised by the caller. */
+#define TPLR_STATIC_WORK_DOUBLES (2048 * (2 + 2 * 256))
+int64_t tplr_static_work_bytes(void);
+int tplr_quantize_batch_static(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
+                               float range_in_sigmas, int n_slices, uint8_t* d_codes, float* d_shift,
+                               float* d_scale, float* d_lookup, void* stream);
 
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes
  * (a multiple of 16, both pointers 16-byte aligned) that moves exactly n_bytes each way.

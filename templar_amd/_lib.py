@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # TPLR_HIP_LIB selects another build of the same library (e.g. an instrumented one)
 LIB_PATH = os.environ.get("TPLR_HIP_LIB") or os.path.join(_HERE, "libtplr_hip.so")
 
-TPLR_E_BADARG, TPLR_E_ODD, TPLR_E_SHAPE, TPLR_E_TOOMANY = -1, -2, -3, -4
+TPLR_E_BADARG, TPLR_E_ODD, TPLR_E_SHAPE, TPLR_E_TOOMANY, TPLR_E_WORKSPACE = -1, -2, -3, -4, -5
 TPLR_MAX_PEERS = 128
 TPLR_MAX_ROW = 4096
 TPLR_MAX_K = 128
@@ -51,6 +51,8 @@ SIGNATURES = {
     "tplr_dequantize_batch": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp]),
     "tplr_dequantize_peers": (_i32, [_vp, _i32, _i64, _vp, _vp, _i32, _vp, _vp]),
     "tplr_quantize_batch": (_i32, [_vp, _i32, _vp, _i32, _i32, C.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "tplr_static_work_bytes": (_i64, []),
+    "tplr_quantize_batch_static": (_i32, [_vp, _i32, _vp, _i32, _i32, C.c_float, _i32, _vp, _vp, _vp, _vp, _vp]),
     "tplr_index_stats_batch": (_i32, [_vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp, _vp, _vp]),
 }
 

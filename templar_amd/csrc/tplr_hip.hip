@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <mutex>
 #include <thread>
 #include <vector>
 
@@ -1663,6 +1664,7 @@ const char* tplr_status_string(int status) {
         case TPLR_E_ODD: return "number of indices must be even";
         case TPLR_E_SHAPE: return "dimension is not a multiple of the chunk size";
         case TPLR_E_TOOMANY: return "too many peers or row too long";
+        case TPLR_E_WORKSPACE: return "workspace larger than the library's static scratch (tplr_static_work_bytes)";
         default: return status > 0 ? hipGetErrorString(static_cast<hipError_t>(status)) : "unknown status";
     }
 }
@@ -2269,16 +2271,9 @@ int tplr_dequantize_peers(const uint8_t* const* h_codes, int n_peers, int64_t n,
     return launch_status();
 }
 
-int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
-                        float range_in_sigmas, int n_slices, double* d_work, uint8_t* d_codes, float* d_shift,
-                        float* d_scale, float* d_lookup, void* stream) {
-    if (!d_val || !d_desc || !d_work || !d_codes || !d_shift || !d_scale || !d_lookup || n_tensors < 1 || k < 4 ||
-        (k & 3) || n_bins < 1 || n_bins > 256 || n_slices < 1 || n_slices > 1024)
-        return TPLR_E_BADARG;
-    if ((reinterpret_cast<uintptr_t>(d_val) & 15) || (reinterpret_cast<uintptr_t>(d_codes) & 3) ||
-        (reinterpret_cast<uintptr_t>(d_work) & 7))
-        return TPLR_E_BADARG;
-    if (static_cast<int64_t>(n_tensors) * n_slices > 0x7fffffff) return TPLR_E_TOOMANY;
+static int launch_quantize(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
+                           float range_in_sigmas, int n_slices, double* d_work, uint8_t* d_codes, float* d_shift,
+                           float* d_scale, float* d_lookup, void* stream) {
     const dim3 grid(static_cast<unsigned>(n_tensors) * n_slices), block(256);
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(k_quant_sum, grid, block, 0, st, d_val, k, d_desc, n_slices, d_work);
@@ -2288,6 +2283,27 @@ int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_des
     hipLaunchKernelGGL(k_quant_tables, dim3(static_cast<unsigned>(n_tensors)), block, 0, st, d_desc, k, n_tensors,
                        n_slices, n_bins, range_in_sigmas, d_work, d_shift, d_scale, d_lookup);
     return launch_status();
+}
+
+static int check_quantize(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
+                          int n_slices, const uint8_t* d_codes, const float* d_shift, const float* d_scale,
+                          const float* d_lookup) {
+    if (!d_val || !d_desc || !d_codes || !d_shift || !d_scale || !d_lookup || n_tensors < 1 || k < 4 || (k & 3) ||
+        n_bins < 1 || n_bins > 256 || n_slices < 1 || n_slices > 1024)
+        return TPLR_E_BADARG;
+    if ((reinterpret_cast<uintptr_t>(d_val) & 15) || (reinterpret_cast<uintptr_t>(d_codes) & 3)) return TPLR_E_BADARG;
+    if (static_cast<int64_t>(n_tensors) * n_slices > 0x7fffffff) return TPLR_E_TOOMANY;
+    return 0;
+}
+
+int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
+                        float range_in_sigmas, int n_slices, double* d_work, uint8_t* d_codes, float* d_shift,
+                        float* d_scale, float* d_lookup, void* stream) {
+    if (!d_work || (reinterpret_cast<uintptr_t>(d_work) & 7)) return TPLR_E_BADARG;
+    if (int s = check_quantize(d_val, k, d_desc, n_tensors, n_bins, n_slices, d_codes, d_shift, d_scale, d_lookup))
+        return s;
+    return launch_quantize(d_val, k, d_desc, n_tensors, n_bins, range_in_sigmas, n_slices, d_work, d_codes, d_shift,
+                           d_scale, d_lookup, stream);
 }
 
 int tplr_dequantize_batch(const uint8_t* d_codes, const float* d_lookup, const float* d_shift, int n_bins, int k,
@@ -2313,6 +2329,63 @@ int tplr_calib_copy(const void* d_src, void* d_dst, int64_t n_bytes, void* strea
     hipLaunchKernelGGL(k_calib_copy, dim3(256 * 16), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const v4f*>(d_src), static_cast<v4f*>(d_dst), n_bytes >> 4);
     return launch_status();
+}
+
+// ---- the quantiser without a caller-provided workspace ----------------------------------------
+// The partial sums of tplr_quantize_batch live in a file-scope device array instead.  The array's
+// name is a host-side handle, not a device address: its address on the current device comes from
+// hipGetSymbolAddress, once per device, and only that pointer is handed to kernels.
+}  // extern "C"
+
+static __device__ __align__(256) double scratch[TPLR_STATIC_WORK_DOUBLES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_lock;
+double* scratch_ptr[kMaxDevices];  // per device: every GPU holds its own copy of the array
+
+// the array's address on the current device; nullptr with *status set when it cannot be had
+double* scratch_on_current_device(int* status) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        *status = static_cast<int>(e);
+        return nullptr;
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        *status = TPLR_E_TOOMANY;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            *status = e != hipSuccess ? static_cast<int>(e) : TPLR_E_BADARG;
+            return nullptr;
+        }
+        scratch_ptr[dev] = static_cast<double*>(p);
+    }
+    return scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" {
+
+int64_t tplr_static_work_bytes(void) { return static_cast<int64_t>(TPLR_STATIC_WORK_DOUBLES) * 8; }
+
+int tplr_quantize_batch_static(const float* d_val, int k, const tplr_tensor_desc* d_desc, int n_tensors, int n_bins,
+                               float range_in_sigmas, int n_slices, uint8_t* d_codes, float* d_shift, float* d_scale,
+                               float* d_lookup, void* stream) {
+    if (int s = check_quantize(d_val, k, d_desc, n_tensors, n_bins, n_slices, d_codes, d_shift, d_scale, d_lookup))
+        return s;
+    const int64_t need = static_cast<int64_t>(n_tensors) * n_slices * (2 + 2 * static_cast<int64_t>(n_bins));
+    if (need > TPLR_STATIC_WORK_DOUBLES) return TPLR_E_WORKSPACE;
+    int status = 0;
+    double* work = scratch_on_current_device(&status);
+    if (!work) return status;
+    return launch_quantize(d_val, k, d_desc, n_tensors, n_bins, range_in_sigmas, n_slices, work, d_codes, d_shift,
+                           d_scale, d_lookup, stream);
 }
 
 }  // extern "C"
