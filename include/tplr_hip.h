@@ -152,7 +152,10 @@ int tplr_encode_topk_pack_batch(const tplr_tensor_desc* d_desc, int n_tensors, i
  * decode(use_dct=False) makes of it, a pure re-layout, :281).
  * h_idx12 / h_val are HOST arrays of n_peers DEVICE pointers: payload p holds
  * n_chunks*k*3/2 index bytes and (n_chunks, k) values.  d_sumsq (nullable) receives
- * n_chunks partial sums of squares of the output, one per chunk. */
+ * n_chunks partial sums of squares of the output, one per chunk.
+ * A payload row may name a coefficient more than once (a top-k selection never does): every
+ * entry is then added, in entry order, and counted, as scatter_reduce_ does; such chunks take
+ * an exact, slower path inside the same launch. */
 int tplr_decode_aggregate(const uint8_t* const* h_idx12, const float* const* h_val,
                           const float* d_peer_scale, int n_peers, int k,
                           int64_t R, int64_t C, int reduce_mode, int normalise, int use_dct,

@@ -145,3 +145,30 @@ def batch_decompress(idxs, vals, xshape, totalk: int, *, block_norms=None, norma
         done.append(v)
     unpacked = [unpack12(i, v.shape) for i, v in zip(idxs, vals)]
     return decompress(torch.cat(unpacked, dim=-1), torch.cat(done, dim=-1), xshape, totalk)
+
+
+# ---- the statistical quantiser (:582-644) ----------------------------------------------------
+def quantize(val: torch.Tensor, n_bins: int = 256, range_in_sigmas: float = 6.0):
+    """TopKCompressor._quantize_values op for op: codes (uint8) and (shift, scale, offset, lookup, dtype)."""
+    offset = n_bins // 2                                                    # :593
+    shift = val.mean()                                                      # :594
+    centered = val - shift                                                  # :595
+    std = centered.norm() / math.sqrt(centered.numel() - 1)                 # :597
+    scale = range_in_sigmas * std / n_bins                                  # :598
+    if scale == 0 or torch.isnan(scale) or torch.isinf(scale):              # :599-600
+        scale = torch.tensor(1.0, dtype=centered.dtype, device=val.device)
+    centered_fp32 = centered.to(torch.float32)                              # :602
+    qval = (centered_fp32 / scale + offset).round().clamp(0, n_bins - 1).to(torch.uint8)   # :603-608
+    sums = torch.zeros(n_bins, dtype=torch.float32, device=qval.device)
+    counts = torch.zeros(n_bins, dtype=torch.float32, device=qval.device)
+    sums.scatter_add_(0, qval.flatten().long(), centered_fp32.flatten())    # :614
+    counts.scatter_add_(0, qval.flatten().long(), torch.ones_like(centered_fp32.flatten()))  # :615-617
+    lookup = torch.where(counts > 0, sums / counts, torch.zeros_like(sums))  # :619
+    return qval, (shift, float(scale), offset, lookup, val.dtype)           # :620-621
+
+
+def dequantize(qval: torch.Tensor, qparams) -> torch.Tensor:
+    """TopKCompressor._dequantize_values (:637-643)."""
+    shift, _, _, lookup, orig_dtype = qparams
+    return (lookup.to(qval.device)[qval.long()] + shift).to(orig_dtype)
+

@@ -292,8 +292,11 @@ static int cmp_f32(const void* a, const void* b) {
 float orc_clip_scales(const float* norms, int P, float* scale) {
     float* s = (float*)malloc(sizeof(float) * (size_t)P);
     memcpy(s, norms, sizeof(float) * (size_t)P);
+    int any_nan = 0;
+    for (int p = 0; p < P; ++p) any_nan |= norms[p] != norms[p];
     qsort(s, (size_t)P, sizeof(float), cmp_f32);
-    const float med = s[(P - 1) / 2];
+    /* torch.median (:535): the lower of the two middle values; NaN if any norm is NaN */
+    const float med = any_nan ? NAN : s[(P - 1) / 2];
     free(s);
     for (int p = 0; p < P; ++p) {
         const float f = med / (norms[p] + 1e-8f);

@@ -453,8 +453,17 @@ def _peer_scales(vals: Sequence[torch.Tensor], block_norms: torch.Tensor | None,
     scale = torch.empty(P, dtype=torch.float32, device=dev)
     with _on(dev):
         if block_norms is not None:
-            norms = block_norms.to(device=dev, dtype=torch.float32).contiguous()
-            st = lib.tplr_clip_scales(_ptr(norms), P, 0, _ptr(scale), None, _stream(dev))
+            norms = block_norms.to(device=dev, dtype=torch.float32).reshape(-1).contiguous()
+            n_norms = norms.numel()
+            # the reference takes the median of every entry (:535) and indexes norms[i] per peer (:554)
+            if n_norms < P:
+                raise IndexError(f"index {n_norms} is out of bounds for dimension 0 with size {n_norms}")
+            if n_norms > _lib.TPLR_MAX_PEERS:
+                raise NotImplementedError(f"{n_norms} block norms: the clip kernel takes up to {_lib.TPLR_MAX_PEERS}")
+            if n_norms > P:
+                scale = torch.empty(n_norms, dtype=torch.float32, device=dev)
+            st = lib.tplr_clip_scales(_ptr(norms), n_norms, 0, _ptr(scale), None, _stream(dev))
+            scale = scale[:P]
         else:
             ptrs = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
             n = vals[0].numel()

@@ -99,8 +99,12 @@ __device__ __forceinline__ void load_chunk_rows(float (&v)[64], const void* chun
         v[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4, r * ld4, 2));
 }
 
-__device__ __forceinline__ void store_chunk_rows(const float (&v)[64], void* chunk0, int64_t ld, int lane) {
-    const __amdgpu_buffer_rsrc_t rs = chunk_rsrc(chunk0, ld);
+// drop (wave-uniform): the stores are issued against a range of zero bytes, whose bounds check
+// discards them - the instruction stream stays the same for a chunk that must not be written
+__device__ __forceinline__ void store_chunk_rows(const float (&v)[64], void* chunk0, int64_t ld, int lane,
+                                                 bool drop = false) {
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        chunk0, 0, drop ? 0 : static_cast<int>((63 * ld + 64) * 4), 0x00020000);
     const int ld4 = static_cast<int>(ld) * 4;
 #pragma unroll
     for (int r = 0; r < 64; ++r)
@@ -469,6 +473,22 @@ __device__ __forceinline__ uint32_t load_idx12(BytePtr row, int j) {
 typedef uint16_t __attribute__((aligned(1))) unaligned_u16;
 using gu16 = __attribute__((address_space(1))) unaligned_u16;
 
+// The fast scatter adds one peer's entries with a plain read-add-write per wave instruction, which is
+// only right when the instruction's destinations are distinct.  A top-k selection has no repeats,
+// but payloads come from other machines: so the read is an exchange that leaves a marker in the
+// slot until the sum is written back.  A lane that reads the marker has met another lane of its own
+// instruction - a repeated index in that peer's row - and the chunk is done again on the exact
+// path (exact_scatter in the kernel).  The marker is a signalling NaN: a slot otherwise holds zero
+// or the result of an addition, which never has these bits.
+constexpr uint32_t kClaimMark = 0x7fa5a5a5u;
+constexpr int kMarkWords = 64;                       // one bit per chunk of a wave's range:
+constexpr int kMaxChunksPerWave = kMarkWords * 32;   // the longest range a wave can keep marks for
+__device__ __forceinline__ float tile_claim(float* slot) {
+    return __builtin_bit_cast(float, __hip_atomic_exchange(reinterpret_cast<uint32_t*>(slot), kClaimMark,
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT));
+}
+__device__ __forceinline__ bool is_claim_mark(float x) { return __builtin_bit_cast(uint32_t, x) == kClaimMark; }
+
 // Contribution counters, one per coefficient, packed into 32-bit words that LDS atomics update,
 // every tile row in words of its own: 4 bits each when at most 15 peers can hit a coefficient
 // (8 words per row, 2 KB), 5 bits up to 31 peers (6 per word, 11 words per row, 2.75 KB) - both
@@ -508,17 +528,25 @@ template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false>
 __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
-                                                            int64_t total, int reduce_mode, int normalise,
-                                                            float* __restrict__ sumsq) {
+                                                            int64_t first, int64_t total, int reduce_mode,
+                                                            int normalise, float* __restrict__ sumsq) {
+    // this launch covers the chunks first .. first + total - 1 of the batch
     __shared__ __align__(16) float tile[kTileFloats];
     using Cnt = Counters<kCntBits>;
     __shared__ __align__(16) uint32_t cnt[Cnt::kAlloc];
+    // the marks live in the counters' rounding slack where there is enough of it (5-bit counters:
+    // the kernel then still fits eight times into a compute unit's LDS), else in words of their own
+    constexpr bool kMarksInSlack = Cnt::kAlloc - Cnt::kWords >= kMarkWords;
+    __shared__ uint32_t own_marks[kMarksInSlack ? 1 : kMarkWords];
+    uint32_t* const marks = kMarksInSlack ? cnt + Cnt::kWords : own_marks;
     constexpr bool kFast = kUnits > 0;
     constexpr int kRegs = kFast ? kUnits : 1;
     const int lane = threadIdx.x;
     int64_t g0, g1;
     my_range(total, g0, g1);
     if (g0 >= g1) return;
+    g0 += first;
+    g1 += first;
 
     const int64_t idx_stride = k + (k >> 1);
     // the inverse transform below is 32x the orthonormal one: its input carries the exact 2^-5
@@ -580,8 +608,10 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
 #pragma unroll
         for (int q = 0; q < 16; ++q) row[q] = z;
         const uint4 zi = make_uint4(0, 0, 0, 0);
+        static_assert(Cnt::kWords % 4 == 0, "counters are cleared 16 bytes at a time");
 #pragma unroll
-        for (int q = 0; q < Cnt::kAlloc / 256; ++q) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
+        for (int q = 0; q < Cnt::kAlloc / 256; ++q)
+            if (q * 64 + lane < Cnt::kWords / 4) reinterpret_cast<uint4*>(cnt)[q * 64 + lane] = zi;
         wave_lds_fence();
     };
 
@@ -590,9 +620,27 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     // LDS instructions of a wave execute in order, so every destination receives its
     // contributions in peer order.  The fast path therefore needs no atomic for the sums; the
     // generic path keeps them.
+    // `repeat` collects, per lane, whether the chunk being scattered has to be done again on the
+    // exact path: a repeated index inside one wave instruction, or a counter about to wrap.
+    bool repeat = false;
+    // Chunks found that way are not stored; they are marked - bit i of `marks` for the i-th chunk of
+    // the wave's range - and done again after the main loop.
+    marks[lane] = 0;
+    auto mark_redo = [&](int64_t g) {  // wave-uniform call, rare
+        const int i = static_cast<int>(g - g0);
+        if (lane == 0) marks[i >> 5] |= 1u << (i & 31);
+    };
     auto add_entry = [&](uint32_t ixe, float val) {
+        // Generic path: atomics add every entry, but entries of one instruction that name the same
+        // coefficient are added in the hardware's order, not in entry order, and the 8-bit counter
+        // wraps at 256.  Another lane of this instruction has been here <=> the counter field this
+        // lane's atomic returns differs from what a read before the instruction saw.
+        uint32_t* cw = &cnt[Cnt::word(ixe)];
+        const uint32_t sh = Cnt::shift(ixe);
+        const uint32_t seen = *cw;
         atomicAdd(&tile[tile_pos(ixe)], val);
-        atomicAdd(&cnt[Cnt::word(ixe)], 1u << Cnt::shift(ixe));
+        const uint32_t was = atomicAdd(cw, 1u << sh);
+        repeat |= (((seen ^ was) >> sh) & Cnt::kMask) != 0u || ((was >> sh) & Cnt::kMask) == Cnt::kMask;
     };
     auto scatter = [&](int64_t g, int t_now) {
         if (fast) {
@@ -603,10 +651,12 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                         const uint32_t e = (lane & 1) ? (ix[i] >> 4) : (ix[i] & 0xfffu);
                         const float x = a[i] * __builtin_bit_cast(float, __builtin_amdgcn_readlane(
                                                    __builtin_bit_cast(int, my_scale), i));
-                        // plain read-add-write: the floating-point LDS atomic costs about 3 cycles
+                        // claim, add, write back: the floating-point LDS atomic costs about 3 cycles
                         // per lane, six times this sequence
                         float* t = &tile[tile_pos(e)];
-                        *t = *t + x;
+                        const float cur = tile_claim(t);
+                        repeat |= is_claim_mark(cur);
+                        *t = cur + x;
                         atomicAdd(&cnt[Cnt::word(e)], 1u << Cnt::shift(e));
                     }
                 }
@@ -667,6 +717,76 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         wave_lds_fence();
     };
 
+    // ---- exact path for a chunk with repeated indices inside one peer's row (no top-k produces
+    // them; the reference sums every entry and divides by the number of entries,
+    // src/tplr/compress.py:472-474).  Entries are added in source order - peer by peer, and inside
+    // a peer in entry order, repeats one after the other - first the values, then, into the
+    // cleared tile, 1.0 per entry, which counts any number of contributions exactly.  Leaves the
+    // tile as the fast scatter and mean_pass would; needs 64 free registers.
+    auto exact_scatter = [&](int64_t g, int t_now) {
+        float sums[64];
+#pragma unroll 1
+        for (int phase = 0; phase < 2; ++phase) {
+            {
+                const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+                float4* row = reinterpret_cast<float4*>(tile + lane * kLd);
+#pragma unroll
+                for (int q = 0; q < 16; ++q) row[q] = z;
+                wave_lds_fence();
+            }
+#pragma unroll 1
+            for (int p = 0; p < P; ++p) {
+                const gfloat* vrow = (const gfloat*)pp.val[p] + g * k;
+                float nrm = 1.0f;
+                if (normalise) {
+                    float ss = 0.f;
+                    for (int j = lane; j < k; j += 64) ss += vrow[j] * vrow[j];
+                    nrm = __builtin_sqrtf(wave_sum_f32(ss)) + 1e-8f;
+                }
+                const float sc = scale ? scale[static_cast<int64_t>(t_now) * P + p] : 1.0f;
+#pragma unroll 1
+                for (int j0 = 0; j0 < k; j0 += 64) {
+                    const int j = j0 + lane;
+                    int me = -1;
+                    float x = 0.f;
+                    if (j < k) {
+                        uint32_t ixe;
+                        float ae;
+                        load_entry(p, j, g, ixe, ae);
+                        me = static_cast<int>(ixe);
+                        // the value as the path this kernel was built for forms it
+                        x = normalise ? (ae / nrm) * out_scale : fast ? ae * (sc * out_scale) : (ae * sc) * out_scale;
+                        if (phase) x = 1.0f;
+                    }
+                    // rank among the earlier lanes that name the same coefficient; one rank per turn
+                    int rank = 0;
+                    for (int i = 0; i < 63; ++i) {
+                        const int other = __shfl(me, i);
+                        rank += (i < lane && other == me && me >= 0) ? 1 : 0;
+                    }
+                    const int turns = static_cast<int>(wave_max_u32(static_cast<uint32_t>(rank)));
+                    for (int r = 0; r <= turns; ++r) {
+                        if (me >= 0 && rank == r) {
+                            float* t = &tile[tile_pos(static_cast<uint32_t>(me))];
+                            *t = *t + x;
+                        }
+                        wave_lds_fence();
+                    }
+                }
+            }
+            if (phase == 0) tile_rows_to_regs(sums, tile, lane);
+            wave_lds_fence();
+        }
+        // row `lane`: sums in registers, counts in the tile
+        float* row = tile + lane * kLd;
+#pragma unroll
+        for (int d = 0; d < 64; ++d) {
+            const float n = row[d];
+            row[d] = (reduce_mode == TPLR_REDUCE_MEAN && n > 1.0f) ? sums[d] / n : sums[d];
+        }
+        wave_lds_fence();
+    };
+
     // where a chunk's result goes
     // Without the transform the result is either the dense coefficient tensor (R/64, C/64, 64, 64)
     // (row stride 0 in the descriptor) or, with a row stride, the (R, C) tensor itself: decode
@@ -674,11 +794,73 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     struct Out {
         gfloat* chunk0;
         int64_t ld;
+        int t;  // the chunk's tensor: its clip factors
     };
     auto out_of = [&](const Cursor& cu, int64_t g) -> Out {
         return Out{(kUseDct || cu.ld > 0) ? cu.base + (cu.y * 64) * cu.ld + static_cast<int64_t>(cu.xc) * 64
                                           : cu.base + (g - cu.begin) * 4096,
-                   cu.ld};
+                   cu.ld, cu.t};
+    };
+
+    // ---- the chunks marked for the exact path, one at a time, after the wave's main loop
+    auto redo_chunk = [&](int64_t g) {
+        Cursor cs;
+        cursor_seek(cs, table, single, n_tensors, g);
+        const Out o = out_of(cs, g);
+        exact_scatter(g, cs.t);
+        float v[64];
+        gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(o.chunk0));
+        const int64_t ld = uniform64(o.ld);
+        const bool rows = kUseDct || ld > 0;  // wave-uniform
+        if (kUseDct) {
+            chunk_inverse<true>(v, tile, lane);
+        } else if (rows) {
+            tile_cols_to_regs(v, tile, lane);
+        } else {
+#pragma unroll
+            for (int q0 = 0; q0 < 16; ++q0) {
+                const int q = q0 * 64 + lane;
+                const float4 t = *reinterpret_cast<const float4*>(tile + (q >> 4) * kLd + ((q & 15) << 2));
+                v[4 * q0] = t.x, v[4 * q0 + 1] = t.y, v[4 * q0 + 2] = t.z, v[4 * q0 + 3] = t.w;
+            }
+        }
+        wave_lds_fence();
+        if constexpr (kSubtract) {
+            const __amdgpu_buffer_rsrc_t rs = chunk_rsrc((const void*)dst, ld);
+            const int ld4 = static_cast<int>(ld) * 4;
+#pragma unroll
+            for (int r = 0; r < 64; ++r)
+                v[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4, r * ld4, 0)) - v[r];
+        }
+        if (sumsq) {
+            float ss = 0.f;
+#pragma unroll
+            for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
+            ss = wave_sum_f32(ss);
+            if (lane == 0) sumsq[g] = ss;
+        }
+        if (rows) {
+            store_chunk_rows(v, (void*)dst, ld, lane);
+        } else {
+#pragma unroll
+            for (int q0 = 0; q0 < 16; ++q0)
+                reinterpret_cast<float4*>((float*)dst)[q0 * 64 + lane] =
+                    make_float4(v[4 * q0], v[4 * q0 + 1], v[4 * q0 + 2], v[4 * q0 + 3]);
+        }
+    };
+    auto redo_marked = [&]() {
+        wave_lds_fence();
+        const uint32_t mine = marks[lane];
+        if (__ballot(mine != 0u) == 0) return;  // wave-uniform: nothing marked, the usual case
+#pragma unroll 1
+        for (int l = 0; l < kMarkWords; ++l) {
+            uint32_t m = __builtin_amdgcn_readlane(static_cast<int>(mine), l);
+#pragma unroll 1
+            while (m) {
+                redo_chunk(g0 + (l * 32 + __builtin_ctz(m)));
+                m &= m - 1;
+            }
+        }
     };
 
     // =====================================================================================
@@ -746,11 +928,16 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 if (i < P) {  // wave-uniform
                     const uint32_t e = (lane & 1) ? (s0.ix[i] >> 4) : (s0.ix[i] & 0xfffu);
                     float* t = &tile[tile_pos(e)];
-                    *t = *t + s0.a[i] * unit_scale(s0.sc, i);
+                    const float was = tile_claim(t);
+                    repeat |= is_claim_mark(was);
+                    *t = was + s0.a[i] * unit_scale(s0.sc, i);
                     atomicAdd(&cnt[Cnt::word(e)], 1u << Cnt::shift(e));
                 }
             }
         }
+        bool skip0 = __ballot(repeat) != 0;  // chunk g: found to hold a repeated index, not stored
+        if (skip0) mark_redo(g0);
+        repeat = false;
         mean_pass();
         if (g0 + 1 < g1) {
             cursor_next(c, g0 + 1);
@@ -815,6 +1002,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 constexpr int s = (h * kSteps + kDctHooks - 1) / kDctHooks;
                 if constexpr (s < kSteps && (s * kDctHooks) / kSteps == h) {
                     if constexpr (s > 0) {
+                        repeat |= is_claim_mark(cur);
                         tile[pos] = cur + add;
                         set_load_unit(st, s - 1, g_load);
                     }
@@ -824,7 +1012,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                         const uint32_t e = __builtin_amdgcn_ubfe(st.ix[u], nib_shift, 12);
                         pos = on ? static_cast<int>(e + ((e >> 6) << 2)) : dummy_pos;
                         add = st.a[u] * unit_scale(sc_now, u);
-                        cur = tile[pos];
+                        cur = tile_claim(&tile[pos]);
                         atomicAdd(&cnt[on ? Cnt::word(e) : lane], on ? 1u << Cnt::shift(e) : 0u);
                     }
                 }
@@ -839,11 +1027,16 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
                 ss = wave_sum_f32(ss);
             }
-            mean_pass();
             // (the loop-carried destination may have been parked in vector registers: make it
             // scalar again, or every store becomes a loop over distinct descriptors)
-            store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane);
-            if (sumsq && lane == 0) sumsq[g] = ss;
+            const bool skip1 = g + 1 < g1 && __ballot(repeat) != 0;  // wave-uniform, false for top-k payloads
+            if (skip1) mark_redo(g + 1);
+            repeat = false;
+            mean_pass();
+            // a chunk that is to be done again is not stored: its descriptor gets a range of zero bytes
+            store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane, skip0);
+            if (sumsq && lane == 0 && !skip0) sumsq[g] = ss;
+            skip0 = skip1;
             o0 = o1;
             o1 = o2;
             o2 = o3;
@@ -852,6 +1045,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             step(g, s1);
             if (g + 1 < g1) step(g + 1, s0);
         }
+        redo_marked();
         return;
     }
 
@@ -865,6 +1059,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     if (fast) load_payload(g0, c.t);
     zero_tile();
     scatter(g0, c.t);
+    bool skip_cur = __ballot(repeat) != 0;  // chunk g: found to hold a repeated index, not stored
+    if (skip_cur) mark_redo(g0);
+    repeat = false;
     mean_pass();
     if (g0 + 1 < g1) {
         cursor_next(c, g0 + 1);
@@ -916,34 +1113,43 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
             ss = wave_sum_f32(ss);
         }
+        const bool skip_next = more && __ballot(repeat) != 0;  // wave-uniform, false for top-k payloads
+        if (skip_next) mark_redo(g + 1);
+        repeat = false;
         if (more) mean_pass();
 
         // (the loop-carried destination may have been parked in vector registers: make it scalar
         // again, or every store becomes a loop over distinct descriptors)
         gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0));
         if (kUseDct || out_cur.ld > 0) {
-            store_chunk_rows(v, (void*)dst, uniform64(out_cur.ld), lane);
-        } else {
+            store_chunk_rows(v, (void*)dst, uniform64(out_cur.ld), lane, skip_cur);
+        } else if (!skip_cur) {
 #pragma unroll
             for (int q0 = 0; q0 < 16; ++q0)
                 reinterpret_cast<float4*>((float*)dst)[q0 * 64 + lane] =
                     make_float4(v[4 * q0], v[4 * q0 + 1], v[4 * q0 + 2], v[4 * q0 + 3]);
         }
-        if (sumsq && lane == 0) sumsq[g] = ss;
+        if (sumsq && lane == 0 && !skip_cur) sumsq[g] = ss;
+        skip_cur = skip_next;
         out_cur = out_next;
         out_next = out_after;
         t_next = t_after;
     }
+    redo_marked();
 }
 
 // ef <- ef - (the payload's entries) for chunks that are not transformed (use_dct = 0): the
 // reconstruction is the payload itself, so only k elements per chunk change
-// (src/tplr/neurons.py:162-171 with decode a pure re-layout).
+// (src/tplr/neurons.py:162-171 with decode a pure re-layout).  k <= 64: one entry per lane.  What
+// is subtracted at a position is what decompress leaves there (src/tplr/compress.py:472-474):
+// the entry, or, when a row names a position more than once (no top-k does), the mean of those
+// entries, added in entry order.
 __global__ __launch_bounds__(64) void k_ef_subtract_sparse(const uint8_t* __restrict__ idx12,
                                                            const float* __restrict__ val, int k,
                                                            const tplr_tensor_desc* __restrict__ table,
                                                            const tplr_tensor_desc single, int n_tensors,
                                                            int64_t total) {
+    __shared__ uint16_t owner[4096];  // the last lane that named a position (never cleared: written before read)
     const int lane = threadIdx.x;
     int64_t g0, g1;
     my_range(total, g0, g1);
@@ -953,11 +1159,35 @@ __global__ __launch_bounds__(64) void k_ef_subtract_sparse(const uint8_t* __rest
     const int64_t idx_stride = k + (k >> 1);
     for (int64_t g = g0; g < g1; ++g) {
         gfloat* chunk0 = c.base + (c.y * 64) * c.ld + static_cast<int64_t>(c.xc) * 64;
-        for (int j = lane; j < k; j += 64) {
-            const uint32_t e = load_idx12(idx12 + g * idx_stride, j);
-            gfloat* t = chunk0 + static_cast<int64_t>(e >> 6) * c.ld + (e & 63);
-            *t = *t - val[g * k + j];
+        int me = -1;
+        float x = 0.f;
+        if (lane < k) {
+            me = static_cast<int>(load_idx12(idx12 + g * idx_stride, lane));
+            x = val[g * k + lane];
+            owner[me] = static_cast<uint16_t>(lane);
         }
+        wave_lds_fence();
+        const bool shared_pos = me >= 0 && owner[me] != lane;
+        bool first = true;
+        if (__ballot(shared_pos) != 0) {  // wave-uniform: some position is named twice
+            float sum = 0.f;
+            int n = 0;
+            for (int i = 0; i < 64; ++i) {
+                const int other = __shfl(me, i);
+                const float xo = __shfl(x, i);
+                if (other == me && me >= 0) {
+                    sum += xo;  // entry order, from zero, as the scatter adds them
+                    n += 1;
+                    first = first && i >= lane;
+                }
+            }
+            x = n > 1 ? sum / static_cast<float>(n) : sum;
+        }
+        if (me >= 0 && first) {
+            gfloat* t = chunk0 + static_cast<int64_t>(me >> 6) * c.ld + (me & 63);
+            *t = *t - x;
+        }
+        wave_lds_fence();
         if (g + 1 < g1) cursor_next(c, g + 1);
     }
 }
@@ -1573,13 +1803,23 @@ __global__ __launch_bounds__(128) void k_clip_scales(const float* __restrict__ n
             nv[i] = norm[off + i];
         }
     }
-    if (i == 0) med = 0.f;
     __syncthreads();
     if (i < P) {
+        // rank in a total order: ascending, NaN after everything, ties by peer - exactly one lane holds
+        // the middle rank.  torch.median (:535) gives NaN as soon as one norm is NaN, and the lower
+        // of the two middle values otherwise.
         int rank = 0;
+        bool any_nan = false;
         const float mine = nv[i];
-        for (int j = 0; j < P; ++j) rank += (nv[j] < mine || (nv[j] == mine && j < i)) ? 1 : 0;
-        if (rank == (P - 1) / 2) med = mine;  // torch.median: lower of the two middles
+        const bool mine_nan = mine != mine;
+        for (int j = 0; j < P; ++j) {
+            const float other = nv[j];
+            const bool other_nan = other != other;
+            any_nan |= other_nan;
+            const bool before = mine_nan ? (!other_nan || j < i) : (!other_nan && (other < mine || (other == mine && j < i)));
+            rank += before ? 1 : 0;
+        }
+        if (rank == (P - 1) / 2) med = any_nan ? __builtin_nanf("") : mine;
     }
     __syncthreads();
     if (i < P) {
@@ -1646,10 +1886,16 @@ static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_sc
                             int64_t total, int reduce_mode, int normalise, float* d_sumsq, void* stream) {
     static int resident = 0;  // per kernel variant
     if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
-    const int64_t need = ((total + 7) / 8) * 8;
-    const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
-    hipLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale, n_peers, k, d_desc,
-                       single, n_tensors, total, reduce_mode, normalise, d_sumsq);
+    // a wave keeps one mark per chunk of its range (chunks to be done again on the exact path), so
+    // one launch takes at most kMaxChunksPerWave chunks per wave: 68 GB of output on a whole device
+    const int64_t piece = static_cast<int64_t>(resident) * (kMaxChunksPerWave - 2);
+    for (int64_t first = 0; first < total; first += piece) {
+        const int64_t count = total - first < piece ? total - first : piece;
+        const int64_t need = ((count + 7) / 8) * 8;
+        const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
+        hipLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale, n_peers, k, d_desc,
+                           single, n_tensors, first, count, reduce_mode, normalise, d_sumsq);
+    }
     return launch_status();
 }
 

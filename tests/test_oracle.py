@@ -294,6 +294,83 @@ def test_quantiser_closed_form():
     assert qp[1] == 1.0 and np.allclose(orc.dequantize(q, qp), cst)
 
 
+def _audit_codes(v, q_a, shift_a, scale_a, q_b, shift_b, scale_b, n_bins):
+    """Two runs of the quantiser whose shift and scale differ in their last bits may code an entry
+    differently only if it sits on a bin boundary to within what those differences move it."""
+    diff = np.flatnonzero(q_a.reshape(-1) != q_b.reshape(-1))
+    if diff.size == 0:
+        return 0
+    x = v.reshape(-1)[diff].astype(np.float64)
+    t = (x - float(shift_a)) / float(scale_a) + n_bins // 2                       # position in bins
+    slack = (abs(float(shift_a) - float(shift_b)) / float(scale_a)
+             + np.abs(t) * abs(float(scale_a) - float(scale_b)) / float(scale_a)
+             + 8 * np.finfo(np.float32).eps * (np.abs(t) + np.abs(x) / float(scale_a)))
+    assert (np.abs(q_a.reshape(-1)[diff].astype(int) - q_b.reshape(-1)[diff].astype(int)) == 1).all()
+    assert (np.abs(t - (np.floor(t) + 0.5)) <= slack).all(), (t, slack)
+    return diff.size
+
+
+@pytest.mark.parametrize("n_bins", [4, 256])
+@pytest.mark.parametrize("kind", ["normal", "offset", "heavy"])
+def test_quantiser_against_torch_op_sequence(n_bins, kind):
+    # the reference's own torch ops (fp32 mean, norm / sqrt(n - 1), round, scatter_add_) against the oracle,
+    # which carries its sums in double: shift and scale agree to rounding, codes agree except on audited
+    # bin boundaries, the per-bin means to rounding
+    rng = np.random.default_rng(11 + n_bins)
+    v = {"normal": rng.standard_normal((37, 32)) * 0.02,
+         "offset": rng.standard_normal((64, 32)) * 1e-3 + 1.0,
+         "heavy": rng.standard_t(3, size=(50, 64)) * 1e-4}[kind].astype(np.float32)
+    q_t, (shift_t, scale_t, off_t, lut_t, dt) = tcp.quantize(torch.from_numpy(v), n_bins, 6.0)
+    q_o, (shift_o, scale_o, off_o, lut_o) = orc.quantize(v, n_bins, 6.0)
+    assert off_t == off_o == n_bins // 2 and dt == torch.float32
+    assert abs(float(shift_t) - shift_o) <= 4e-7 * max(abs(shift_o), np.abs(v).max() / np.sqrt(v.size))
+    assert abs(scale_t - scale_o) <= 1e-6 * scale_o
+    n_diff = _audit_codes(v, q_t.numpy(), float(shift_t), scale_t, q_o, shift_o, scale_o, n_bins)
+    assert n_diff <= max(2, v.size // 100)
+    used = np.unique(q_o)
+    same = [b for b in used if (q_t.numpy() == b).sum() == (q_o == b).sum()]
+    assert np.allclose(lut_t.numpy()[same], lut_o[same], rtol=1e-4, atol=1e-6 * np.abs(v).max())
+    # de-quantisation: same table and codes in, same values out
+    want = tcp.dequantize(torch.from_numpy(q_o), (torch.tensor(shift_o), scale_o, off_o, torch.from_numpy(lut_o), dt))
+    assert np.array_equal(orc.dequantize(q_o, (shift_o, scale_o, off_o, lut_o)), want.numpy())
+
+
+@pytest.mark.parametrize("n_bins", [4, 256])
+def test_quantiser_ties_and_constants_equal_torch(n_bins):
+    # exact halves: range 0 makes the scale fall back to exactly 1 (:599-600) and dyadic, symmetric values make
+    # the mean exactly 0 in any summation order, so position = value + n_bins / 2 with ties at every x.5:
+    # torch.round rounds them to even (:605), and so must the oracle - every code equal
+    half = np.arange(-n_bins // 2 - 3, n_bins // 2 + 4, dtype=np.float32) + np.float32(0.5)
+    v = np.concatenate([half, -half, np.array([0.0, 0.25, -0.25, 0.75, -0.75], np.float32)]).astype(np.float32)
+    q_t, (shift_t, scale_t, _, lut_t, _) = tcp.quantize(torch.from_numpy(v), n_bins, 0.0)
+    q_o, (shift_o, scale_o, _, lut_o) = orc.quantize(v, n_bins, 0.0)
+    assert float(shift_t) == shift_o == 0.0 and scale_t == scale_o == 1.0
+    assert np.array_equal(q_t.numpy(), q_o)
+    assert np.array_equal(q_o, np.clip(np.rint(v + n_bins // 2), 0, n_bins - 1).astype(np.uint8))
+    # n_bins / 2 is even: both neighbouring halves round to it
+    assert q_o[np.flatnonzero(v == 0.5)[0]] == n_bins // 2 and q_o[np.flatnonzero(v == -0.5)[0]] == n_bins // 2
+    assert np.allclose(lut_t.numpy(), lut_o, rtol=1e-6, atol=0)
+    # a constant tensor: scale 1, every code n_bins / 2, de-quantised back to the constant
+    cst = np.full((6, 32), 0.375, np.float32)
+    q_t, (shift_t, scale_t, _, lut_t, _) = tcp.quantize(torch.from_numpy(cst), n_bins, 6.0)
+    q_o, (shift_o, scale_o, _, lut_o) = orc.quantize(cst, n_bins, 6.0)
+    assert float(shift_t) == shift_o == 0.375 and scale_t == scale_o == 1.0
+    assert np.array_equal(q_t.numpy(), q_o) and (q_o == n_bins // 2).all()
+    assert np.array_equal(orc.dequantize(q_o, (shift_o, scale_o, n_bins // 2, lut_o)), cst)
+
+
+def test_clip_scales_with_non_finite_norms_match_torch():
+    # torch.median gives NaN as soon as one norm is NaN (:535); an infinite norm is simply the largest
+    for norms in ([1.0, float("nan")], [float("nan"), 1.0], [3.0, float("nan"), 1.0, 2.0], [float("inf"), 1.0, 2.0, 5.0],
+                  [float("inf"), float("inf"), 1.0], [float("nan"), float("inf"), 2.0, 1.0, 4.0]):
+        med, scale = orc.clip_scales(norms)
+        t = torch.tensor(norms)
+        want_med = torch.median(t)
+        want = torch.clamp(want_med / (t + 1e-8), max=1).numpy()
+        assert np.array_equal(np.float32(med), want_med.numpy(), equal_nan=True), norms
+        assert np.array_equal(scale, want, equal_nan=True), norms
+
+
 def test_golden_fixture_is_reproduced():
     z = np.load(os.path.join(GOLD, "codec_small.npz"))
     coef = orc.encode2d(z["x"])
