@@ -1,5 +1,6 @@
-"""Full-size checks on the GPU: the 1B gradient set (294 144 chunks, benchmark configurations 3 and 4)
-and the 72B block (config 5, k = 64) through the batch entry points of the C ABI.
+"""Full-size checks on the GPU: the 150M set (config 2), the 1B gradient set (294 144 chunks, benchmark
+configurations 3 and 4) and the 72B block (config 5, k = 64, encode and 15-peer decode) through the batch
+entry points of the C ABI; config 1 has a file of its own (tests/test_gpu_config1.py).
 
 The CPU oracle cannot cover these sizes in test time, so the checks are properties that do not
 depend on size (plus a strided sample that does go through the oracle):
@@ -57,7 +58,7 @@ def _check_rows(idx12, val, n, k):
     return idx
 
 
-@pytest.mark.parametrize("name", ["cfg3_llama1b", "cfg5_72b_block"])
+@pytest.mark.parametrize("name", ["cfg2_llama150m", "cfg3_llama1b", "cfg5_72b_block"])
 def test_full_set_encode_properties(dev, name):
     grads, k = _set(name, dev)
     batch = tc.TensorBatch(grads)
@@ -252,14 +253,17 @@ def test_full_size_index_statistics_against_bitmaps(dev, P, k):
         assert torch.equal(top[:, p].long(), want_top)
 
 
-@pytest.mark.parametrize("use_dct,P,k", [(False, 15, 32), (True, 15, 32), (False, 20, 64), (True, 20, 64), (True, 31, 32)])
-def test_full_set_aggregate_against_torch_scatter_reduce(dev, use_dct, P, k):
-    # the 1B set, 15 peers, every chunk: torch's own scatter_reduce_(mean, include_self=False) on the
-    # concatenated payloads (the reference's op sequence, src/tplr/compress.py:559-580, run on the GPU),
-    # then its einsum decode, against the one-launch aggregate
+@pytest.mark.parametrize("name,use_dct,P,k", [("cfg3_llama1b", False, 15, 32), ("cfg3_llama1b", True, 15, 32),
+                                              ("cfg3_llama1b", False, 20, 64), ("cfg3_llama1b", True, 20, 64),
+                                              ("cfg3_llama1b", True, 31, 32), ("cfg2_llama150m", True, 15, 32),
+                                              ("cfg2_llama150m", False, 15, 32), ("cfg5_72b_block", True, 15, 64)])
+def test_full_set_aggregate_against_torch_scatter_reduce(dev, name, use_dct, P, k):
+    # a whole set (the 1B set, the 150M set, the 72B block on its own shapes), every chunk: torch's own
+    # scatter_reduce_(mean, include_self=False) on the concatenated payloads (the reference's op sequence,
+    # src/tplr/compress.py:559-580, run on the GPU), then its einsum decode, against the one-launch aggregate
     from oracle import torch_cpu_path as tcp
 
-    shapes = [s for s in workloads.CONFIGS["cfg3_llama1b"]["shapes"] if len(s) == 2]
+    shapes = [s for s in workloads.CONFIGS[name]["shapes"] if len(s) == 2]
     counts = [(a // 64) * (b // 64) for a, b in shapes]
     n = sum(counts)
     g = torch.Generator(device=dev)
@@ -305,14 +309,15 @@ def test_full_set_aggregate_against_torch_scatter_reduce(dev, use_dct, P, k):
     assert worst > 0.0 or not use_dct
 
 
-def test_full_set_transform_and_selection_against_torch(dev):
-    # every tensor of the 1B set: the chunked transform against torch's einsum with the reference's
+@pytest.mark.parametrize("name", ["cfg3_llama1b", "cfg2_llama150m", "cfg5_72b_block"])
+def test_full_set_transform_and_selection_against_torch(dev, name):
+    # every tensor of a set: the chunked transform against torch's einsum with the reference's
     # FFT-built basis (the reference's op sequence on the GPU), and the fused kernel's payload against
     # torch.topk on this library's own coefficients - magnitudes bit for bit, values gathered at the
     # selected indices bit for bit
     from oracle import torch_cpu_path as tcp
 
-    grads, k = _set("cfg3_llama1b", dev)
+    grads, k = _set(name, dev)
     batch = tc.TensorBatch(grads)
     idx12, val = tc.encode_compress_batch(batch, k, use_dct=True)
     f, _ = tcp.basis(64)
