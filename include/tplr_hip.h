@@ -294,6 +294,18 @@ int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_des
                         float range_in_sigmas, int n_slices, double* d_work, uint8_t* d_codes, float* d_shift,
                         float* d_scale, float* d_lookup, void* stream);
 
+/* ---- per-tensor L2 normalisation of an aggregate ----------------------------------------------
+ * The reference has no such step inside tplr.compress; the benchmark's aggregation workload words it
+ * ("scatter-summed, inverse DCT, mean over peers, then L2-normalised per tensor"), and the per-chunk
+ * d_sumsq output of tplr_decode_aggregate_batch exists for it.
+ * tplr_tensor_rnorm: d_factor[t] = 1 / (sqrt(sum of tensor t's d_sumsq entries) + eps), the entries
+ * added in a fixed order (d_desc: chunk_begin and chunk counts).
+ * tplr_scale_batch: every element of tensor t times d_factor[t], in place (d_desc as for the aggregate). */
+int tplr_tensor_rnorm(const float* d_sumsq, const tplr_tensor_desc* d_desc, int n_tensors, float eps, float* d_factor,
+                      void* stream);
+int tplr_scale_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, const float* d_factor,
+                     void* stream);
+
 /* tplr_quantize_batch for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc); it has no counterpart in the
  * reference.  Same arguments and results without d_work: the partial sums go through a static

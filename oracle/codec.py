@@ -219,6 +219,17 @@ def batch_decompress(idx_packed_list, val_list, xshape, totalk: int, *, block_no
     return out.reshape(xshape)
 
 
+def aggregate_mean_normalised(idx_packed_list, val_list, xshape, totalk: int, *, use_dct: bool = True,
+                              eps: float = 1e-8) -> np.ndarray:
+    """The benchmark's wording of the aggregation workload (no counterpart inside tplr.compress): the peers'
+    payloads scatter-summed, inverse transform, divided by the number of peers, divided by the L2 norm
+    (+ eps) of the result.  Built from batch_decompress in sum mode and decode2d."""
+    P = len(val_list)
+    dense = batch_decompress(idx_packed_list, val_list, xshape, totalk, clip_norm=False, mean=False)
+    x = decode2d(dense, use_dct=use_dct).astype(np.float64) / P
+    return (x / (np.sqrt((x * x).sum()) + eps)).astype(np.float32)
+
+
 # ---------------------------------------------------------------- quantiser (:582-644)
 def quantize(val, n_bins: int = 256, range_in_sigmas: float = 6.0):
     v = _c(val, np.float32)

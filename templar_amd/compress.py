@@ -1003,6 +1003,28 @@ def batch_decompress_decode_batch(out: TensorBatch, idxs: Sequence[torch.Tensor]
 
 
 @torch.no_grad()
+def aggregate_mean_normalised_batch(out: TensorBatch, idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], k: int,
+                                    *, use_dct: bool = True, eps: float = 1e-8) -> torch.Tensor:
+    """The aggregation as the benchmark's workload words it: every peer's payload scatter-summed, inverse
+    transform, mean over the peers (the sum divided by their number, whoever sent a coefficient), then
+    every tensor divided by its L2 norm (+ eps).  Three launches: the aggregate in sum mode with the factor
+    1/P on every peer and per-chunk sums of squares, the per-tensor norms from those, one scaling pass.
+    tplr.compress itself has no such mode (batch_decompress takes the mean over the senders of each
+    coefficient, src/tplr/compress.py:472-474).  Returns the (T,) factors 1 / (norm + eps)."""
+    lib = _lib.load()
+    P, T, n, dev = len(vals), len(out), out.total_chunks, out.device
+    scale = torch.full((T, P), 1.0 / P, dtype=torch.float32, device=dev)
+    ss = torch.empty(n, dtype=torch.float32, device=dev)
+    batch_decompress_decode_batch(out, idxs, vals, k, scale=scale, use_dct=use_dct, mean=False, sumsq=ss)
+    factor = torch.empty(T, dtype=torch.float32, device=dev)
+    with _on(dev):
+        _lib.check(lib.tplr_tensor_rnorm(_ptr(ss), _ptr(out.table), T, C.c_float(eps), _ptr(factor), _stream(dev)),
+                   "tplr_tensor_rnorm")
+        _lib.check(lib.tplr_scale_batch(_ptr(out.table), T, n, _ptr(factor), _stream(dev)), "tplr_scale_batch")
+    return factor
+
+
+@torch.no_grad()
 def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, topk: int, *, use_dct: bool = True,
                               compressor: "TopKCompressor | None" = None, null_round: bool = False):
     """The miner's per-parameter loop of src/tplr/neurons.py:147-171 for a whole set of 2-D
@@ -1558,6 +1580,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

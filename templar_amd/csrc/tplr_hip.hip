@@ -1829,6 +1829,43 @@ __global__ __launch_bounds__(128) void k_clip_scales(const float* __restrict__ n
     if (i == 0 && median) median[blockIdx.x] = med;
 }
 
+// Per-tensor factor 1 / (||x_t|| + eps) from per-chunk sums of squares (as tplr_decode_aggregate_batch
+// writes them): one block per tensor, the chunks' sums added in a fixed order.
+__global__ __launch_bounds__(256) void k_tensor_rnorm(const float* __restrict__ sumsq,
+                                                      const tplr_tensor_desc* __restrict__ table, float eps,
+                                                      float* __restrict__ factor) {
+    __shared__ double part[4];
+    const tplr_tensor_desc d = table[blockIdx.x];
+    const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
+    const float* s = sumsq + d.chunk_begin;
+    double acc = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += 256) acc += static_cast<double>(s[i]);
+    acc = block256_sum_f64(acc, part, threadIdx.x);
+    if (threadIdx.x == 0) factor[blockIdx.x] = 1.0f / (static_cast<float>(sqrt(acc)) + eps);
+}
+
+// x <- x * factor[t] for every chunk of a batch (the per-tensor normalisation that follows an aggregate):
+// 16 KB read and written per chunk, persistent, one chunk's 64 row loads in flight ahead of its stores.
+__global__ __launch_bounds__(64) void k_scale_chunks(const tplr_tensor_desc* __restrict__ table, int n_tensors,
+                                                     int64_t total, const float* __restrict__ factor) {
+    const int lane = threadIdx.x;
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
+    Cursor c;
+    tplr_tensor_desc none = {};
+    cursor_seek(c, table, none, n_tensors, g0);
+    for (int64_t g = g0; g < g1; ++g) {
+        float v[64];
+        load_chunk_cols(v, c, lane);
+        const float f = factor[c.t];
+#pragma unroll
+        for (int r = 0; r < 64; ++r) v[r] *= f;
+        store_chunk_cols(v, (float*)c.base, c.ld, c.y, c.xc, lane);
+        if (g + 1 < g1) cursor_next(c, g + 1);
+    }
+}
+
 // Plain streaming copy (16 bytes per lane per step, grid-stride).  It exists so that hardware
 // traffic counters can be calibrated: it moves exactly n16 * 16 bytes each way.
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -2565,6 +2602,26 @@ int tplr_dequantize_batch(const uint8_t* d_codes, const float* d_lookup, const f
     hipLaunchKernelGGL(k_dequantize_batch, dim3(static_cast<unsigned>(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), d_codes, d_lookup, d_shift, n_bins, k, d_desc, n_tensors, n4,
                        d_val);
+    return launch_status();
+}
+
+int tplr_tensor_rnorm(const float* d_sumsq, const tplr_tensor_desc* d_desc, int n_tensors, float eps, float* d_factor,
+                      void* stream) {
+    if (!d_sumsq || !d_desc || !d_factor || n_tensors < 1) return TPLR_E_BADARG;
+    hipLaunchKernelGGL(k_tensor_rnorm, dim3(static_cast<unsigned>(n_tensors)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), d_sumsq, d_desc, eps, d_factor);
+    return launch_status();
+}
+
+int tplr_scale_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, const float* d_factor,
+                     void* stream) {
+    if (!d_desc || !d_factor || n_tensors < 1 || total_chunks < 0) return TPLR_E_BADARG;
+    if (total_chunks == 0) return 0;
+    static int resident = 0;
+    if (resident == 0) resident = persistent_grid(k_scale_chunks, int64_t{1} << 40);
+    const int64_t need = ((total_chunks + 7) / 8) * 8;
+    hipLaunchKernelGGL(k_scale_chunks, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), d_desc, n_tensors, total_chunks, d_factor);
     return launch_status();
 }
 

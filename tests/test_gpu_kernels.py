@@ -1041,3 +1041,32 @@ def test_whole_set_calls_replay_from_a_captured_graph(dev):
         torch.cuda.synchronize()
         assert torch.equal(idx12, want[0]) and torch.equal(val, want[1])
         assert all(torch.equal(a, b) for a, b in zip(outs, want[2]))
+
+
+@pytest.mark.parametrize("use_dct", [True, False])
+def test_aggregate_mean_over_peers_then_normalised_per_tensor(dev, use_dct):
+    # the benchmark's wording of the aggregation workload: scatter-sum, inverse transform, divide by the number
+    # of peers, divide every tensor by its L2 norm - against the oracle, tensor by tensor
+    P, k = 15, 32
+    shapes = [(128, 192), (64, 64), (256, 128)]
+    counts = [(a // 64) * (b // 64) for a, b in shapes]
+    n = sum(counts)
+    idxs, vals = make_peers(P, 1, n, k, 321)
+    outs = [torch.full(s, 3.0, device=dev) for s in shapes]
+    batch = tc.TensorBatch(outs)
+    di = [torch.from_numpy(i).to(dev) for i in idxs]
+    dv = [torch.from_numpy(v.reshape(n, k)).to(dev) for v in vals]
+    factor = tc.aggregate_mean_normalised_batch(batch, di, dv, k, use_dct=use_dct)
+    b0 = 0
+    for t, (shape, cnt) in enumerate(zip(shapes, counts)):
+        Y, X = shape[0] // 64, shape[1] // 64
+        ti = [orc.pack12(orc.unpack12(i, (n, k))[b0:b0 + cnt]) for i in idxs]
+        tv = [v.reshape(n, k)[b0:b0 + cnt].reshape(Y, X, k) for v in vals]
+        want = orc.aggregate_mean_normalised(ti, tv, (Y, X, 64, 64), 4096, use_dct=use_dct)
+        got = outs[t].cpu().numpy()
+        assert abs(float(np.sqrt((got.astype(np.float64) ** 2).sum())) - 1.0) <= 1e-5
+        assert np.abs(got - want).max() <= TOL * np.abs(want).max(), t
+        plain = orc.decode2d(orc.batch_decompress(ti, tv, (Y, X, 64, 64), 4096, clip_norm=False, mean=False), use_dct=use_dct)
+        assert abs(float(factor[t]) * np.sqrt((plain.astype(np.float64) ** 2).sum()) / P - 1.0) <= 1e-5
+        b0 += cnt
+

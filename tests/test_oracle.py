@@ -371,6 +371,31 @@ def test_clip_scales_with_non_finite_norms_match_torch():
         assert np.array_equal(scale, want, equal_nan=True), norms
 
 
+def test_aggregate_mean_normalised_is_the_normalised_mean_of_the_peers_reconstructions():
+    # the benchmark's wording of the aggregation: linear in the peers, so it equals the mean of the one-peer
+    # reconstructions (each built here with torch's scatter_add_ and scipy's inverse DCT), divided by its norm
+    rng = np.random.default_rng(21)
+    P, Y, X, k = 5, 2, 3, 32
+    idxs, vals = [], []
+    for p in range(P):
+        i, v = orc.topk_rows(rng.standard_normal((Y, X, 4096)).astype(np.float32), k)
+        idxs.append(i)
+        vals.append(v)
+    got = orc.aggregate_mean_normalised([orc.pack12(i) for i in idxs], vals, (Y, X, 64, 64), 4096)
+    acc = np.zeros((Y * 64, X * 64))
+    for i, v in zip(idxs, vals):
+        dense = torch.zeros(Y * X, 4096, dtype=torch.float64)
+        dense.scatter_add_(1, torch.from_numpy(i.reshape(Y * X, k).astype(np.int64)),
+                           torch.from_numpy(v.reshape(Y * X, k).astype(np.float64)))
+        chunks = scipy.fft.idctn(dense.numpy().reshape(Y, X, 64, 64), type=2, norm="ortho", axes=(2, 3))
+        acc += chunks.transpose(0, 2, 1, 3).reshape(Y * 64, X * 64)
+    want = acc / P
+    want = want / np.sqrt((want ** 2).sum())
+    assert got.dtype == np.float32 and got.shape == (Y * 64, X * 64)
+    assert abs(float(np.sqrt((got.astype(np.float64) ** 2).sum())) - 1.0) <= 1e-6
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()
+
+
 def test_golden_fixture_is_reproduced():
     z = np.load(os.path.join(GOLD, "codec_small.npz"))
     coef = orc.encode2d(z["x"])
