@@ -75,6 +75,22 @@ def event_ms(fn, steps, warmup):
     return start.elapsed_time(stop) / steps, wall
 
 
+def launch_stats(fn, steps):
+    """Per-call durations of `steps` further calls, each between its own pair of events on the current
+    stream: (median, min, max) in ms.  The clock governor ramps for the first calls after idle; the
+    spread shows whether a mean sits inside that ramp."""
+    import torch
+
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in pairs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    t = sorted(a.elapsed_time(b) for a, b in pairs)
+    return round(t[len(t) // 2], 4), round(t[0], 4), round(t[-1], 4)
+
+
 def cpu_baseline(workload_name, k, peers, budget_s):
     """Reference op sequence on torch CPU (oracle/torch_cpu_path.py) on a bounded sample:
     one transformer layer's worth of the 1B set (4 x 2048x2048, 2 x 8192x2048, 2048x8192)
@@ -212,11 +228,16 @@ def main():
     n_chunks = batch.total_chunks
     idx_buf = torch.empty(n_chunks * (k // 2) * 3, dtype=torch.uint8, device=dev)
     val_buf = torch.empty((n_chunks, k), dtype=torch.float32, device=dev)
-    # the norm vectors (64-element chunks) as one flat tensor: one transform + one select launch
-    flat_1d = torch.cat(one_d) if one_d else None
-    if flat_1d is not None:  # the norm vectors live back to back, as views of one flat buffer
-        one_d = list(flat_1d.split([g.numel() for g in one_d]))
+    # the norm vectors (rows of 64 elements), every one an allocation of its own as in a model: one launch
+    # reads them where they lie
+    flat_1d = None
     rows_1d = tc.RowBatch(one_d) if one_d and all(g.numel() % 64 == 0 for g in one_d) else None
+    if one_d and rows_1d is None:
+        flat_1d = torch.cat(one_d)
+    if rows_1d is not None:
+        k1 = min(k, 64)
+        idx_buf_1d = torch.empty(rows_1d.total_rows * (k1 // 2) * 3, dtype=torch.uint8, device=dev)
+        val_buf_1d = torch.empty((rows_1d.total_rows, k1), dtype=torch.float32, device=dev)
 
     def encode2d_only():
         tc.encode_compress_batch(batch, k, use_dct=True, idx12=idx_buf, val=val_buf)
@@ -224,7 +245,7 @@ def main():
     def encode_pass():
         encode2d_only()
         if rows_1d is not None:
-            tc.encode_compress_rows_batch(rows_1d, k, use_dct=True)
+            tc.encode_compress_rows_batch(rows_1d, k, use_dct=True, idx12=idx_buf_1d, val=val_buf_1d)
         elif flat_1d is not None:
             comp.compress(tr.encode(flat_1d, use_dct=True), k)
 
@@ -281,7 +302,9 @@ def main():
         enc_ms, enc_wall = event_ms(encode_pass, args.steps, args.warmup)
     enc_bytes = workloads.encode_bytes(shapes, k)
     if args.profile is None:
+        enc_spread = launch_stats(encode_pass, args.steps)
         enc2d_ms, _ = event_ms(encode2d_only, args.steps, 1)      # the fused 2-D kernel alone (dominant)
+        enc2d_spread = launch_stats(encode2d_only, args.steps)
         enc_pt_ms, _ = event_ms(encode_per_tensor, max(3, args.steps // 2), 1)
         enc_rc_ms, _ = event_ms(encode_reference_calls, 3, 1)
     enc2d_bytes = n_chunks * (16384 + 11 * k // 2)
@@ -341,6 +364,10 @@ def main():
     agg_ms, agg_wall = event_ms(aggregate_pass, agg_steps, 2)
     agg2d_ms, _ = event_ms(aggregate_2d_pass, agg_steps, 1)
     aggk_ms, _ = event_ms(aggregate_kernel_only, agg_steps, 1)
+    aggk_spread = launch_stats(aggregate_kernel_only, agg_steps)
+    # the aggregation as the benchmark's workload words it: sum over the peers, inverse transform, mean over
+    # the peers, every tensor divided by its L2 norm (three launches; tplr.compress itself has no such mode)
+    aggn_ms, _ = event_ms(lambda: tc.aggregate_mean_normalised_batch(out_batch, idxs, vals, k), agg_steps, 1)
     agg_pt_ms, _ = event_ms(aggregate_per_tensor, 3, 1)
     agg_rc_ms, _ = event_ms(aggregate_reference_calls, 3, 1)
     # the same per-parameter loop recorded once into a HIP graph and replayed: what is left is device time
@@ -402,6 +429,13 @@ def main():
         "aggregate_GBps": round(agg_pass_bytes / (agg_ms * 1e-3) / 1e9, 2),
         "aggregate_wall_ms": round(agg_wall, 4),
         "aggregate_2d_ms": round(agg2d_ms, 4),
+        "aggregate_sum_mean_normalised_ms": round(aggn_ms, 4),
+        "aggregate_sum_mean_normalised_note": "the workload's own wording: scatter-sum over the peers, inverse DCT, "
+                                              "divide by their number, divide each tensor by its L2 norm (aggregate in "
+                                              "sum mode + per-tensor norms + one scaling pass); aggregate_ms is the "
+                                              "reference's batch_decompress semantics",
+        "ms_per_step_spread": {"median": enc_spread[0], "min": enc_spread[1], "max": enc_spread[2],
+                               "what": "per-call durations of a further `steps` calls of the step, each between its own events"},
         "per_tensor_launches": {"encode_ms": round(enc_pt_ms, 4), "aggregate_ms": round(agg_pt_ms, 4),
                                 "note": "same work as one fused launch per tensor through the reference-shaped API",
                                 "aggregate_graph_replay_ms": round(agg_graph_ms, 4),
@@ -414,14 +448,20 @@ def main():
             "achieved": round(enc2d_bytes / (enc2d_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(enc2d_bytes / (enc2d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
             "traffic": MEASURED_TRAFFIC.get((args.workload, P, "encode")),
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload kept under profiles/, "
+                              "not measured by this run; null for other workloads",
             "launches_per_step": 1, "bytes_per_launch": enc2d_bytes, "ms_per_launch": round(enc2d_ms, 4),
+            "ms_per_launch_median": enc2d_spread[0], "ms_per_launch_min": enc2d_spread[1],
         },
         "roofline_aggregate": {
             "bound": "hbm", "kernel": "k_decode_aggregate",
             "achieved": round(agg_bytes / (aggk_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(agg_bytes / (aggk_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
             "traffic": MEASURED_TRAFFIC.get((args.workload, P, "aggregate")),
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload kept under profiles/, "
+                              "not measured by this run; null for other workloads",
             "launches_per_step": 1, "bytes_per_launch": agg_bytes, "ms_per_launch": round(aggk_ms, 4),
+            "ms_per_launch_median": aggk_spread[0], "ms_per_launch_min": aggk_spread[1],
         },
     }
     if miner is not None:

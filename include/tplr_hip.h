@@ -137,6 +137,15 @@ int tplr_encode_topk_pack(const float* d_x, int64_t R, int64_t C, int64_t ld_x, 
 int tplr_encode_topk_pack_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, int k,
                                 int use_dct, uint8_t* d_idx12, float* d_val, void* stream);
 
+/* The 1-D parameters of a set (norm vectors) in ONE launch: encode (rows of 64, the 64-point DCT-II of
+ * every row when use_dct != 0, src/tplr/compress.py:248-255) followed by compress (top-k per row, :402-416)
+ * for every tensor of d_desc, each read where it lies: `dense` = the tensor, x_chunks = its number of rows
+ * (elements / 64), y_chunks = 1, chunk_begin = the id of its first row in the flat payload (row g: indices
+ * at byte g*3k/2, values at float g*k).  total_groups = the sum over the tensors of ceil(rows / 64).
+ * k even, 2 <= k <= 64.  Same bits as tplr_dct1d followed by tplr_topk_pack with row_len 64. */
+int tplr_encode_rows_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_groups, int k, int use_dct,
+                           uint8_t* d_idx12, float* d_val, void* stream);
+
 /* ---- decode side -----------------------------------------------------------------
  * Fused TopKCompressor.batch_decompress + ChunkingTransformer.decode
  * (src/tplr/compress.py:483-580 then :259-292; caller: src/tplr/neurons.py:355-367).

@@ -36,6 +36,7 @@ SIGNATURES = {
     "tplr_topk_pack": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp]),
     "tplr_encode_topk_pack": (_i32, [_vp, _i64, _i64, _i64, _i32, _i32, _vp, _vp, _vp]),
     "tplr_encode_topk_pack_batch": (_i32, [_vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp]),
+    "tplr_encode_rows_batch": (_i32, [_vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp]),
     "tplr_decode_aggregate_batch": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp]),
     "tplr_segment_sumsq": (_i32, [_vp, _i32, _i32, _vp, _i32, _i32, _vp, _vp]),
     "tplr_clip_scales_batch": (_i32, [_vp, _i32, _i32, _i32, _vp, _vp, _vp]),

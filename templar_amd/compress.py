@@ -1129,8 +1129,9 @@ class RowBatch:
         desc = np.zeros(len(tensors), dtype=np.dtype([("dense", "<u8"), ("ld", "<i8"), ("chunk_begin", "<i8"),
                                                       ("x_chunks", "<i4"), ("y_chunks", "<i4")]))
         for i, (b, n) in enumerate(zip(self.offsets, self.rows)):
-            desc[i] = (0, 0, b, n, 1)
+            desc[i] = (tensors[i].data_ptr(), _CH, b, n, 1)
         self.table = torch.from_numpy(desc.view(np.uint8).copy()).to(dev)
+        self.total_groups = sum((n + _CH - 1) // _CH for n in self.rows)  # waves of up to 64 rows of one tensor
 
     def __len__(self) -> int:
         return len(self.tensors)
@@ -1152,21 +1153,25 @@ class RowBatch:
 
 
 @torch.no_grad()
-def encode_compress_rows_batch(batch: RowBatch, topk: int, *, use_dct: bool = True):
+def encode_compress_rows_batch(batch: RowBatch, topk: int, *, use_dct: bool = True, idx12: torch.Tensor | None = None,
+                               val: torch.Tensor | None = None):
     """encode + compress of every 1-D tensor of the set (src/tplr/neurons.py:155-159 per parameter) in
-    three launches: concatenate, 64-point transform of every row, top-k per row.  Returns the flat
-    payload (idx12 uint8, val (total_rows, k)); totalk is 64 for every row."""
+    one launch: every tensor is read where it lies, its rows of 64 go through the 64-point transform and the
+    top-k in registers.  Returns the flat payload (idx12 uint8, val (total_rows, k)); totalk is 64 for
+    every row."""
     lib = _lib.load()
     k = _clamp_k(_CH, topk)
     dev = batch.device
-    rows = (batch.flat if batch.flat is not None else torch.cat(batch.tensors)).reshape(-1, _CH)
-    if use_dct:
-        coef = torch.empty_like(rows)
-        with _on(dev):
-            st = lib.tplr_dct1d(_ptr(rows), rows.shape[0], 0, _ptr(coef), _stream(dev))
-        _lib.check(st, "tplr_dct1d")
-        rows = coef
-    return _topk_rows(rows, k)
+    n = batch.total_rows
+    if idx12 is None:
+        idx12 = torch.empty(n * (k // 2) * 3, dtype=torch.uint8, device=dev)
+    if val is None:
+        val = torch.empty((n, k), dtype=torch.float32, device=dev)
+    with _on(dev):
+        st = lib.tplr_encode_rows_batch(_ptr(batch.table), len(batch), batch.total_groups, k, int(use_dct), _ptr(idx12),
+                                        _ptr(val), _stream(dev))
+    _lib.check(st, "tplr_encode_rows_batch")
+    return idx12, val
 
 
 @torch.no_grad()

@@ -174,6 +174,7 @@ __device__ __forceinline__ void chunk_inverse(float (&v)[64], float* tile, int l
 // Pointers that come out of descriptor tables are not kernel arguments, so the compiler
 // cannot tell that they are global memory; say so, or it emits FLAT accesses (which also
 // count as LDS traffic and serialise against the tile).
+typedef float v4f __attribute__((ext_vector_type(4)));
 using gfloat = __attribute__((address_space(1))) float;
 using gbyte = __attribute__((address_space(1))) uint8_t;
 
@@ -403,6 +404,89 @@ __global__ __launch_bounds__(64) void k_topk_rows(const float* __restrict__ coef
     emit_selected(s, lane, k, row, idx12, val);
 }
 
+// The 1-D parameters of a set (norm vectors), every tensor a run of rows of 64 elements: transform,
+// top-k and pack of all of them in one launch, each tensor read where it lies.  One wave takes up to 64
+// rows of one tensor: staged through the tile, a row per lane in registers, the 64-point transform and
+// its scale exactly as k_dct1d applies them, then every lane sorts its own 64 coefficients in registers -
+// a bitonic network over 64-bit keys (magnitude, 63 - index), the canonical order of select_topk - and
+// writes its row's payload: the k leading indices, and their values fetched back from the tile.
+template <bool kUseDct>
+__global__ __launch_bounds__(64) void k_encode_rows(const tplr_tensor_desc* __restrict__ table, int n_tensors, int k,
+                                                    uint8_t* __restrict__ idx12, float* __restrict__ val) {
+    __shared__ __align__(16) float tile[kTileFloats];
+    const int lane = threadIdx.x;
+    // this wave's tensor and group of rows: tensor t has ceil(rows / 64) groups
+    int t = 0, grp = blockIdx.x;
+    for (; t < n_tensors; ++t) {
+        const int groups = (table[t].x_chunks + 63) >> 6;
+        if (grp < groups) break;
+        grp -= groups;
+    }
+    if (t >= n_tensors) return;
+    const tplr_tensor_desc d = table[t];
+    const int left = d.x_chunks - grp * 64;  // rows from this group's first to the tensor's end
+    const gfloat* src = (const gfloat*)d.dense + static_cast<int64_t>(grp) * 4096;
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+        const int q = c * 64 + lane;
+        const int r = q >> 4;
+        v4f x = {0.f, 0.f, 0.f, 0.f};
+        if (r < left) x = *reinterpret_cast<const __attribute__((address_space(1))) v4f*>(src + q * 4);
+        *reinterpret_cast<v4f*>(tile + r * kLd + ((q & 15) << 2)) = x;
+    }
+    wave_lds_fence();
+    float w[64];
+    tile_rows_to_regs(w, tile, lane);
+    if (kUseDct) {
+        dct64_fwd(w);
+#pragma unroll
+        for (int e = 0; e < 64; ++e) w[e] *= 0.17677669529663687f;  // one pass is sqrt(32) times the orthonormal transform
+    }
+    wave_lds_fence();
+    regs_to_tile_rows(w, tile, lane);
+    uint64_t key[64];
+#pragma unroll
+    for (int e = 0; e < 64; ++e)
+        key[e] = (static_cast<uint64_t>(mag_key(__builtin_bit_cast(uint32_t, w[e]))) << 32) | static_cast<uint32_t>(63 - e);
+    // bitonic sort, descending
+#pragma unroll
+    for (int size = 2; size <= 64; size <<= 1) {
+#pragma unroll
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+#pragma unroll
+            for (int i = 0; i < 64; ++i) {
+                const int l = i ^ stride;
+                if (l > i) {
+                    const bool up = (i & size) != 0 && size < 64;  // this run ascends
+                    const uint64_t a = key[i], b = key[l];
+                    const bool swap = up ? a > b : a < b;
+                    key[i] = swap ? b : a;
+                    key[l] = swap ? a : b;
+                }
+            }
+        }
+    }
+    wave_lds_fence();
+    if (lane >= left) return;
+    const int64_t row = d.chunk_begin + static_cast<int64_t>(grp) * 64 + lane;
+    float* vrow = val + row * k;
+    uint8_t* irow = idx12 + row * (k + (k >> 1));
+    const float* mine = tile + lane * kLd;
+#pragma unroll
+    for (int j = 0; j < 64; j += 2) {
+        if (j < k) {  // k is even
+            const uint32_t i0 = 63u - static_cast<uint32_t>(key[j]), i1 = 63u - static_cast<uint32_t>(key[j + 1]);
+            vrow[j] = mine[i0];
+            vrow[j + 1] = mine[i1];
+            const uint32_t pair = i0 | (i1 << 12);
+            uint8_t* o = irow + 3 * (j >> 1);
+            o[0] = static_cast<uint8_t>(pair);
+            o[1] = static_cast<uint8_t>(pair >> 8);
+            o[2] = static_cast<uint8_t>(pair >> 16);
+        }
+    }
+}
+
 // Persistent fused encode: every wave walks its slice of the chunk list.  The kernel is bound by
 // vector-ALU issue and by the latencies between its phases, so it is shaped for residency -
 // 8.5 KB + 1 KB of LDS and a register budget that admits three to four waves per SIMD - and
@@ -478,16 +562,21 @@ using gu16 = __attribute__((address_space(1))) unaligned_u16;
 // but payloads come from other machines: so the read is an exchange that leaves a marker in the
 // slot until the sum is written back.  A lane that reads the marker has met another lane of its own
 // instruction - a repeated index in that peer's row - and the chunk is done again on the exact
-// path (exact_scatter in the kernel).  The marker is a signalling NaN: a slot otherwise holds zero
-// or the result of an addition, which never has these bits.
-constexpr uint32_t kClaimMark = 0x7fa5a5a5u;
+// path (exact_scatter in the kernel).  The marker is the largest bit pattern there is (a NaN), so a
+// lane remembers having met it with one unsigned maximum per step; a slot otherwise holds zero or
+// the result of an addition, which has these bits only if a peer sent that very NaN - and then
+// the chunk merely takes the exact path for nothing.
+constexpr uint32_t kClaimMark = 0xffffffffu;
 constexpr int kMarkWords = 64;                       // one bit per chunk of a wave's range:
 constexpr int kMaxChunksPerWave = kMarkWords * 32;   // the longest range a wave can keep marks for
 __device__ __forceinline__ float tile_claim(float* slot) {
     return __builtin_bit_cast(float, __hip_atomic_exchange(reinterpret_cast<uint32_t*>(slot), kClaimMark,
                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT));
 }
-__device__ __forceinline__ bool is_claim_mark(float x) { return __builtin_bit_cast(uint32_t, x) == kClaimMark; }
+__device__ __forceinline__ uint32_t seen_mark(uint32_t seen, float x) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, x);
+    return seen > b ? seen : b;
+}
 
 // Contribution counters, one per coefficient, packed into 32-bit words that LDS atomics update,
 // every tile row in words of its own: 4 bits each when at most 15 peers can hit a coefficient
@@ -622,7 +711,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     // generic path keeps them.
     // `repeat` collects, per lane, whether the chunk being scattered has to be done again on the
     // exact path: a repeated index inside one wave instruction, or a counter about to wrap.
-    bool repeat = false;
+    uint32_t repeat = 0;  // kClaimMark <=> the chunk has to be done again
     // Chunks found that way are not stored; they are marked - bit i of `marks` for the i-th chunk of
     // the wave's range - and done again after the main loop.
     marks[lane] = 0;
@@ -640,7 +729,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         const uint32_t seen = *cw;
         atomicAdd(&tile[tile_pos(ixe)], val);
         const uint32_t was = atomicAdd(cw, 1u << sh);
-        repeat |= (((seen ^ was) >> sh) & Cnt::kMask) != 0u || ((was >> sh) & Cnt::kMask) == Cnt::kMask;
+        if ((((seen ^ was) >> sh) & Cnt::kMask) != 0u || ((was >> sh) & Cnt::kMask) == Cnt::kMask) repeat = kClaimMark;
     };
     auto scatter = [&](int64_t g, int t_now) {
         if (fast) {
@@ -655,7 +744,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                         // per lane, six times this sequence
                         float* t = &tile[tile_pos(e)];
                         const float cur = tile_claim(t);
-                        repeat |= is_claim_mark(cur);
+                        repeat = seen_mark(repeat, cur);
                         *t = cur + x;
                         atomicAdd(&cnt[Cnt::word(e)], 1u << Cnt::shift(e));
                     }
@@ -929,15 +1018,15 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                     const uint32_t e = (lane & 1) ? (s0.ix[i] >> 4) : (s0.ix[i] & 0xfffu);
                     float* t = &tile[tile_pos(e)];
                     const float was = tile_claim(t);
-                    repeat |= is_claim_mark(was);
+                    repeat = seen_mark(repeat, was);
                     *t = was + s0.a[i] * unit_scale(s0.sc, i);
                     atomicAdd(&cnt[Cnt::word(e)], 1u << Cnt::shift(e));
                 }
             }
         }
-        bool skip0 = __ballot(repeat) != 0;  // chunk g: found to hold a repeated index, not stored
+        bool skip0 = __ballot(repeat == kClaimMark) != 0;  // chunk g: found to hold a repeated index, not stored
         if (skip0) mark_redo(g0);
-        repeat = false;
+        repeat = 0;
         mean_pass();
         if (g0 + 1 < g1) {
             cursor_next(c, g0 + 1);
@@ -1002,7 +1091,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 constexpr int s = (h * kSteps + kDctHooks - 1) / kDctHooks;
                 if constexpr (s < kSteps && (s * kDctHooks) / kSteps == h) {
                     if constexpr (s > 0) {
-                        repeat |= is_claim_mark(cur);
+                        repeat = seen_mark(repeat, cur);
                         tile[pos] = cur + add;
                         set_load_unit(st, s - 1, g_load);
                     }
@@ -1029,9 +1118,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             }
             // (the loop-carried destination may have been parked in vector registers: make it
             // scalar again, or every store becomes a loop over distinct descriptors)
-            const bool skip1 = g + 1 < g1 && __ballot(repeat) != 0;  // wave-uniform, false for top-k payloads
+            const bool skip1 = g + 1 < g1 && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
             if (skip1) mark_redo(g + 1);
-            repeat = false;
+            repeat = 0;
             mean_pass();
             // a chunk that is to be done again is not stored: its descriptor gets a range of zero bytes
             store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane, skip0);
@@ -1059,9 +1148,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     if (fast) load_payload(g0, c.t);
     zero_tile();
     scatter(g0, c.t);
-    bool skip_cur = __ballot(repeat) != 0;  // chunk g: found to hold a repeated index, not stored
+    bool skip_cur = __ballot(repeat == kClaimMark) != 0;  // chunk g: found to hold a repeated index, not stored
     if (skip_cur) mark_redo(g0);
-    repeat = false;
+    repeat = 0;
     mean_pass();
     if (g0 + 1 < g1) {
         cursor_next(c, g0 + 1);
@@ -1113,9 +1202,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
             ss = wave_sum_f32(ss);
         }
-        const bool skip_next = more && __ballot(repeat) != 0;  // wave-uniform, false for top-k payloads
+        const bool skip_next = more && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
         if (skip_next) mark_redo(g + 1);
-        repeat = false;
+        repeat = 0;
         if (more) mean_pass();
 
         // (the loop-carried destination may have been parked in vector registers: make it scalar
@@ -1868,7 +1957,6 @@ __global__ __launch_bounds__(64) void k_scale_chunks(const tplr_tensor_desc* __r
 
 // Plain streaming copy (16 bytes per lane per step, grid-stride).  It exists so that hardware
 // traffic counters can be calibrated: it moves exactly n16 * 16 bytes each way.
-typedef float v4f __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(256) void k_calib_copy(const v4f* __restrict__ src, v4f* __restrict__ dst, int64_t n16) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
@@ -2143,6 +2231,22 @@ int tplr_encode_topk_pack_batch(const tplr_tensor_desc* d_desc, int n_tensors, i
     if (total_chunks == 0) return 0;
     tplr_tensor_desc none = {};
     return launch_encode(d_desc, none, n_tensors, total_chunks, k, use_dct, d_idx12, d_val, stream);
+}
+
+int tplr_encode_rows_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_groups, int k, int use_dct,
+                           uint8_t* d_idx12, float* d_val, void* stream) {
+    if (!d_desc || n_tensors < 1 || total_groups < 0 || !d_idx12 || !d_val || k < 2 || (k & 1) || k > 64)
+        return TPLR_E_BADARG;
+    if (total_groups == 0) return 0;
+    if (total_groups > 0x7fffffff) return TPLR_E_TOOMANY;
+    const dim3 grid(static_cast<unsigned>(total_groups)), block(64);
+    if (use_dct)
+        hipLaunchKernelGGL(k_encode_rows<true>, grid, block, 0, static_cast<hipStream_t>(stream), d_desc, n_tensors, k,
+                           d_idx12, d_val);
+    else
+        hipLaunchKernelGGL(k_encode_rows<false>, grid, block, 0, static_cast<hipStream_t>(stream), d_desc, n_tensors, k,
+                           d_idx12, d_val);
+    return launch_status();
 }
 
 int tplr_ef_encode_topk_pack_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc* d_grad_desc,

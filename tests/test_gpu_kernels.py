@@ -1070,3 +1070,47 @@ def test_aggregate_mean_over_peers_then_normalised_per_tensor(dev, use_dct):
         assert abs(float(factor[t]) * np.sqrt((plain.astype(np.float64) ** 2).sum()) / P - 1.0) <= 1e-5
         b0 += cnt
 
+
+@pytest.mark.parametrize("use_dct", [True, False])
+@pytest.mark.parametrize("k", [2, 16, 32, 64])
+def test_rows_encode_in_one_launch_equals_transform_then_select(dev, k, use_dct):
+    # tplr_encode_rows_batch (every 1-D parameter where it lies, one launch) against tplr_dct1d followed by
+    # tplr_topk_pack on the concatenation: the same bytes, for separately allocated vectors of ragged lengths,
+    # with ties, zeros, denormals, infinities and NaNs among the elements
+    rng = np.random.default_rng(900 + k)
+    lengths = [64, 128, 768, 2048, 64 * 65, 64 * 3, 64 * 130]
+    host = []
+    for j, n in enumerate(lengths):
+        v = (rng.standard_t(3, size=n) * 10.0 ** (j % 3 - 2)).astype(np.float32)
+        v[rng.integers(0, n, n // 8)] = 0.0
+        v[rng.integers(0, n, n // 16)] = np.float32(0.5)      # exact ties, either sign
+        v[rng.integers(0, n, n // 16)] = np.float32(-0.5)
+        host.append(v)
+    host[1][:64] = 0.0                       # an all-zero row
+    host[2][5] = np.nan
+    host[2][70] = -np.nan
+    host[3][100] = np.inf
+    host[3][101] = -np.inf
+    host[4][64 * 64 + 3] = np.float32(1e-41)  # a denormal in the second group of a tensor
+    vecs = [torch.from_numpy(v).to(dev) for v in host]  # separate allocations
+    rb = tc.RowBatch(vecs)
+    assert rb.flat is None and rb.total_groups == 1 + 1 + 1 + 1 + 2 + 1 + 3
+    idx12, val = tc.encode_compress_rows_batch(rb, k, use_dct=use_dct)
+    rows = torch.cat(vecs).reshape(-1, 64)
+    lib = _lib.load()
+    if use_dct:
+        coef = torch.empty_like(rows)
+        with tc._on(dev):
+            assert lib.tplr_dct1d(tc._ptr(rows), rows.shape[0], 0, tc._ptr(coef), tc._stream(dev)) == 0
+        rows = coef
+    want_i, want_v = tc._topk_rows(rows, k)
+    assert val.shape == want_v.shape == (rb.total_rows, k)
+    assert torch.equal(idx12, want_i)
+    got_v, ref_v = val.cpu().numpy(), want_v.cpu().numpy()
+    assert np.array_equal(np.isnan(got_v), np.isnan(ref_v))  # (a NaN's payload bits are not compared)
+    fin = ~np.isnan(ref_v)
+    assert np.array_equal(got_v.view(np.uint32)[fin], ref_v.view(np.uint32)[fin])
+    # and the oracle's selection on those coefficients
+    oi, ov = orc.topk_rows(rows.cpu().numpy(), k)
+    assert np.array_equal(idx12.cpu().numpy(), orc.pack12(oi))
+
