@@ -1440,6 +1440,14 @@ class PayloadStage:
                 _lib.check(st, "tplr_dequantize_batch")
         return out_i, [self.values[p] for p in range(n_peers)]
 
+    def regions(self, p: int) -> tuple[torch.Tensor, torch.Tensor]:
+        """Peer p's place in the device buffer: (packed indices, values (n, k) or codes).  The peers'
+        places are equally spaced, which is what lets the aggregate kernels address them with scalar
+        arithmetic; payloads produced on the device (tests, benchmarks, a local peer) can be written here
+        directly."""
+        ri, rv = self._regions(self.dev, p)
+        return ri, rv.view(-1, self.k)
+
     def _regions(self, buf: torch.Tensor, p: int) -> tuple[torch.Tensor, torch.Tensor]:
         b = p * self.stride
         idx = buf[b:b + self.idx_bytes]

@@ -478,12 +478,16 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
     out.idx1 = 0;
     out.val1 = 0.0f;
     uint64_t e0, e1 = 0ull;
+    // (the slot address is formed here, from a copy of the lane id the optimiser cannot see through: hoisted
+    // out of a caller's chunk loop it would only be one more value to keep, or to spill, across the loop)
+    int slot_of_lane = lane;
+    asm volatile("" : "+v"(slot_of_lane));
     if (total <= 64) {
-        e0 = lane < static_cast<int>(total) ? cand[lane] : 0ull;
+        e0 = lane < static_cast<int>(total) ? cand[slot_of_lane] : 0ull;
         sort64_desc(e0, lane);
     } else {
-        e0 = cand[lane];
-        e1 = lane + 64 < static_cast<int>(total) ? cand[lane + 64] : 0ull;
+        e0 = cand[slot_of_lane];
+        e1 = lane + 64 < static_cast<int>(total) ? cand[slot_of_lane + 64] : 0ull;
         sort128_desc(e0, e1, lane);
     }
     // a slot unpacks to index, and to the value itself: sign bit on top of the magnitude bits
@@ -494,16 +498,20 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
         val = __uint_as_float(mag | (lo << 31)) * out_scale;
     };
     unpack(e0, out.idx0, out.val0);
-    if (k > 64) unpack(e1, out.idx1, out.val1);
+    if (kTwo && k > 64) unpack(e1, out.idx1, out.val1);  // (kTwo: the instantiation that serves k > 32)
     wave_lds_fence();
     return out;
 }
 
 // Write the selection of one row: values (row, k) and 12-bit packed indices.
+template <bool kTwo = true>
 __device__ __forceinline__ void emit_selected(const Selected& s, int lane, int k, int64_t row,
                                               uint8_t* __restrict__ idx12, float* __restrict__ val) {
     float* vrow = val + row * k;
     uint8_t* irow = idx12 + row * (k + (k >> 1));
+    // (lane-derived offsets are formed from a copy of the lane id the optimiser cannot see through, so that
+    // they are recomputed here instead of being kept, or spilled, across a caller's chunk loop)
+    asm volatile("" : "+v"(lane));
     if (lane < k) vrow[lane] = s.val0;
     const uint32_t p0 = __shfl_xor(s.idx0, 1);
     if (!(lane & 1) && lane < k) {
@@ -513,7 +521,7 @@ __device__ __forceinline__ void emit_selected(const Selected& s, int lane, int k
         o[1] = static_cast<uint8_t>(w >> 8);
         o[2] = static_cast<uint8_t>(w >> 16);
     }
-    if (k > 64) {
+    if (kTwo && k > 64) {
         if (lane + 64 < k) vrow[lane + 64] = s.val1;
         const uint32_t p1 = __shfl_xor(s.idx1, 1);
         if (!(lane & 1) && lane + 64 < k) {

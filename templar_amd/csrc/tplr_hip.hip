@@ -401,7 +401,7 @@ __global__ __launch_bounds__(64) void k_topk_rows(const float* __restrict__ coef
     tile_rows_to_regs(w, tile, lane);
     __syncthreads();
     const Selected s = select_topk<kTwo>(w, tile, cand, lane, k, 1.0f);
-    emit_selected(s, lane, k, row, idx12, val);
+    emit_selected<kTwo>(s, lane, k, row, idx12, val);
 }
 
 // The 1-D parameters of a set (norm vectors), every tensor a run of rows of 64 elements: transform,
@@ -532,7 +532,7 @@ __global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_de
         chunk_forward<kUseDct>(v, w, buf, lane);
         const Selected s =
             select_topk<kTwo, !kUseDct>(w, buf, cand, lane, k, kUseDct ? kDctPow2Scale : 1.0f, c1, c2);
-        emit_selected(s, lane, k, g, idx12, val);
+        emit_selected<kTwo>(s, lane, k, g, idx12, val);
     }
 }
 
@@ -613,16 +613,25 @@ struct Counters {
 // kSubtract (fast path with the transform only): the destination receives destination - result
 // instead of the result (the error-feedback update of src/tplr/neurons.py:171); its rows are
 // requested before the second pass and arrive during it.
-template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false>
+// kStrided (fast path): the peers' payloads are equally spaced in memory - peer p's index bytes at
+// pp.idx[0] + p * stride_idx, its values at pp.val[0] + p * stride_val floats, as a staged window lays
+// them out - so every payload address is scalar arithmetic on two base pointers instead of a pair of
+// lane broadcasts per peer and chunk.
+template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false, bool kStrided = false>
 __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
                                                             int64_t first, int64_t total, int reduce_mode,
-                                                            int normalise, float* __restrict__ sumsq) {
+                                                            int normalise, float* __restrict__ sumsq,
+                                                            int64_t stride_idx, int64_t stride_val) {
     // this launch covers the chunks first .. first + total - 1 of the batch
-    __shared__ __align__(16) float tile[kTileFloats];
     using Cnt = Counters<kCntBits>;
-    __shared__ __align__(16) uint32_t cnt[Cnt::kAlloc];
+    // kPark: lanes and units without an entry scatter "coefficient 4096 + lane", which the address
+    // arithmetic of real coefficients maps to 64 tile slots and 8 counter words past the chunk's own
+    // (one select per step instead of three); 4-bit counters only: a row of them is 8 whole words
+    constexpr bool kPark = kUnits > 0 && kUseDct && kCntBits == 4;
+    __shared__ __align__(16) float tile[kTileFloats + (kPark ? 64 : 0)];
+    __shared__ __align__(16) uint32_t cnt[Cnt::kAlloc + (kPark ? 8 : 0)];
     // the marks live in the counters' rounding slack where there is enough of it (5-bit counters:
     // the kernel then still fits eight times into a compute unit's LDS), else in words of their own
     constexpr bool kMarksInSlack = Cnt::kAlloc - Cnt::kWords >= kMarkWords;
@@ -642,7 +651,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     const float out_scale = kUseDct ? kDctPow2Scale : 1.0f;
     const bool lane_on = lane < k;       // fast path: this lane owns an entry
     const int le = lane_on ? lane : 0;   // the other lanes reload entry 0 and stay out of the scatter
-    const int lane_ioff = 3 * (le >> 1) + (le & 1);  // byte offset of entry `le` in a packed row
+    const uint32_t lane_ioff = 3u * (static_cast<uint32_t>(le) >> 1) + (le & 1);  // byte offset of entry `le` in a packed row
 
     // Fast path: lane p keeps peer p's two payload pointers and its clip factor for the current
     // tensor in registers; unit i gets them as scalars through v_readlane, so that the steady
@@ -669,17 +678,25 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
     };
     // unit i's entries of chunk g into its two registers
-    auto load_unit = [&](int i, int64_t g) {
-        const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
-        const gbyte* irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
-        const gfloat* vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
-        ix[i] = *(const gu16*)(irow + lane_ioff);
-        a[i] = vrow[le];
-    };
     auto load_payload = [&](int64_t g, int t) {  // fast path only
         load_scale(t);
+        // kStrided: peer after peer by scalar additions from chunk g's place in peer 0's payload
+        const gbyte* irow = (const gbyte*)pp.idx[0] + uniform64(g * idx_stride);
+        const gfloat* vrow = (const gfloat*)pp.val[0] + uniform64(g * k);
 #pragma unroll
-        for (int i = 0; i < kRegs; ++i) load_unit(i, g);
+        for (int i = 0; i < kRegs; ++i) {
+            if constexpr (!kStrided) {
+                const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
+                irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
+                vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
+            }
+            ix[i] = *(const gu16*)(irow + lane_ioff);
+            a[i] = vrow[le];
+            if (kStrided && i + 1 < P) {  // (unused units reload the last peer)
+                irow += stride_idx;
+                vrow += stride_val;
+            }
+        }
     };
     // entry j of peer p of chunk g (generic path and normalise)
     auto load_entry = [&](int p, int j, int64_t g, uint32_t& ixo, float& ao) {
@@ -985,10 +1002,31 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 st.t = t;
             }
         };
+        // kStrided: `next_i` / `next_v` walk from peer to peer by scalar additions; set_walk puts them on a
+        // chunk's place in peer 0's payload
+        const gbyte* next_i = (const gbyte*)pp.idx[0];
+        const gfloat* next_v = (const gfloat*)pp.val[0];
+        // (the peer count as the walk sees it: a copy the optimiser cannot see through, renewed per chunk, or it
+        // would keep "stride or 0" for every unit in scalar registers of its own across the loop, and spill them)
+        int walk_peers = P;
+        auto set_walk = [&](int64_t off_i, int64_t off_v) {
+            next_i = (const gbyte*)pp.idx[0] + off_i;
+            next_v = (const gfloat*)pp.val[0] + off_v;
+            asm volatile("" : "+s"(walk_peers));
+        };
         auto set_load_unit = [&](Set& st, int i, int64_t g) {
-            const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
-            const gbyte* irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
-            const gfloat* vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
+            const gbyte* irow = next_i;
+            const gfloat* vrow = next_v;
+            if constexpr (kStrided) {
+                if (i + 1 < walk_peers) {  // (unused units reload the last peer and stay out of the scatter)
+                    next_i += stride_idx;
+                    next_v += stride_val;
+                }
+            } else {
+                const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
+                irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
+                vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
+            }
             // Streaming loads: measured 7 % faster than cached ones for this kernel, although
             // index rows (1.5 k bytes) of neighbouring chunks share cache lines and those lines
             // then come in from memory more than once (+0.47 GB on the 1B set, 1.08 x the
@@ -998,6 +1036,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         };
         auto set_load = [&](Set& st, int64_t g, int t) {
             set_scale(st, t);
+            if constexpr (kStrided) set_walk(uniform64(g * idx_stride), uniform64(g * k));
 #pragma unroll
             for (int i = 0; i < kRegs; ++i) set_load_unit(st, i, g);
         };
@@ -1054,7 +1093,11 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             for (int r = 0; r < 64; ++r) __builtin_amdgcn_raw_buffer_store_b32(0, nowhere, lane * 4, r * 256, 2);
         }
 
-        const int dummy_pos = lane * kLd + kChunk;
+        // (kStrided) where the chunk loaded last sits in a payload; the loop's loads advance chunk by chunk
+        const int64_t loaded_last = g0 + 2 < g1 ? g0 + 2 : g1 - 1;
+        int64_t last_i = uniform64(loaded_last * idx_stride), last_v = uniform64(loaded_last * k);
+        const int dummy_pos = kPark ? kTileFloats + lane : lane * kLd + kChunk;
+        const uint32_t park = 4096u + lane;  // (kPark) maps to tile[kTileFloats + lane] and cnt[512 + lane / 8]
         const uint32_t nib_shift = (lane & 1) * 4;  // odd entries sit in the upper 12 bits of their 16
         // one chunk: `st` holds chunk g + 1 and is refilled with chunk g + 3
         auto step = [&](int64_t g, Set& st) {
@@ -1077,9 +1120,16 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 set_scale(st, c.t);
             }
             const int64_t g_load = more3 ? g + 3 : g1 - 1;
+            if constexpr (kStrided) {
+                if (more3) {
+                    last_i += idx_stride;
+                    last_v += k;
+                }
+                set_walk(last_i, last_v);
+            }
             constexpr int kSteps = kUnits + 1;
             constexpr int kAlways = kUnits > 8 ? kUnits - 8 : 1;  // units every served peer count uses
-            int pos = dummy_pos;
+            int pos = kPark ? dummy_pos * 4 : dummy_pos;  // (kPark: a byte offset)
             float cur = 0.f, add = 0.f;
             float before[kSubtract ? 64 : 1];
             if constexpr (kSubtract)
@@ -1092,17 +1142,31 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 if constexpr (s < kSteps && (s * kDctHooks) / kSteps == h) {
                     if constexpr (s > 0) {
                         repeat = seen_mark(repeat, cur);
-                        tile[pos] = cur + add;
+                        if constexpr (kPark)
+                            *reinterpret_cast<float*>(reinterpret_cast<char*>(tile) + pos) = cur + add;
+                        else
+                            tile[pos] = cur + add;
                         set_load_unit(st, s - 1, g_load);
                     }
                     if constexpr (s < kUnits) {
                         constexpr int u = s;
                         const bool on = lane_on && (u < kAlways || u < P);
-                        const uint32_t e = __builtin_amdgcn_ubfe(st.ix[u], nib_shift, 12);
-                        pos = on ? static_cast<int>(e + ((e >> 6) << 2)) : dummy_pos;
                         add = st.a[u] * unit_scale(sc_now, u);
-                        cur = tile_claim(&tile[pos]);
-                        atomicAdd(&cnt[on ? Cnt::word(e) : lane], on ? 1u << Cnt::shift(e) : 0u);
+                        if constexpr (kPark) {
+                            // byte addresses by hand: slot 4 e + 16 (e >> 6), counter word 4 (e >> 3), its
+                            // field 4 (e & 7) bits up - seven instructions from the packed index
+                            const uint32_t e = on ? __builtin_amdgcn_ubfe(st.ix[u], nib_shift, 12) : park;
+                            const uint32_t e4 = e << 2;
+                            pos = static_cast<int>(e4 + ((e >> 2) & 0x7f0u));
+                            cur = tile_claim(reinterpret_cast<float*>(reinterpret_cast<char*>(tile) + pos));
+                            atomicAdd(reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(cnt) + ((e >> 1) & 0xffcu)),
+                                      1u << (e4 & 28u));
+                        } else {
+                            const uint32_t e = __builtin_amdgcn_ubfe(st.ix[u], nib_shift, 12);
+                            pos = on ? static_cast<int>(e + ((e >> 6) << 2)) : dummy_pos;
+                            cur = tile_claim(&tile[pos]);
+                            atomicAdd(&cnt[on ? Cnt::word(e) : lane], on ? 1u << Cnt::shift(e) : 0u);
+                        }
                     }
                 }
             });
@@ -1962,6 +2026,61 @@ __global__ __launch_bounds__(256) void k_calib_copy(const v4f* __restrict__ src,
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
 
+// The memory side of k_decode_aggregate alone, for calibration: the same persistent grid and chunk
+// ranges, the same payload loads (every peer's two loads per chunk, streaming, requested two chunks
+// ahead) and the same 64 row stores per chunk, but no LDS work and no arithmetic beyond folding the
+// loaded values into what is stored.  Its duration is what the memory system needs for the
+// aggregate's traffic in this access pattern; with n_peers = 0 it is the pure fill of the outputs.
+__global__ __launch_bounds__(64, 2) void k_calib_aggregate(const PeerPtrs pp, int P, int k,
+                                                           const tplr_tensor_desc* __restrict__ table, int n_tensors,
+                                                           int64_t total) {
+    const int lane = threadIdx.x;
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
+    const int64_t idx_stride = k + (k >> 1);
+    const int le = lane < k ? lane : 0;
+    const uint32_t lane_ioff = 3u * (static_cast<uint32_t>(le) >> 1) + (le & 1);
+    constexpr int kU = 24;
+    uint32_t ix[2][kU];
+    float a[2][kU];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int i = 0; i < kU; ++i) ix[s][i] = 0, a[s][i] = 0.f;
+    auto load = [&](int s, int64_t g) {
+#pragma unroll
+        for (int i = 0; i < kU; ++i) {
+            if (i < P) {  // wave-uniform
+                const gbyte* irow = (const gbyte*)pp.idx[i] + g * idx_stride;
+                const gfloat* vrow = (const gfloat*)pp.val[i] + g * k;
+                ix[s][i] = __builtin_nontemporal_load((const gu16*)(irow + lane_ioff));
+                a[s][i] = __builtin_nontemporal_load(vrow + le);
+            }
+        }
+    };
+    Cursor c;
+    tplr_tensor_desc none = {};
+    cursor_seek(c, table, none, n_tensors, g0);
+    load(0, g0);
+    load(1, g0 + 1 < g1 ? g0 + 1 : g0);
+    auto chunk = [&](int64_t g, int s) {
+        float x = 0.f;
+#pragma unroll
+        for (int i = 0; i < kU; ++i) x += a[s][i] + __builtin_bit_cast(float, ix[s][i]);
+        load(s, g + 2 < g1 ? g + 2 : g1 - 1);
+        float v[64];
+#pragma unroll
+        for (int r = 0; r < 64; ++r) v[r] = x + static_cast<float>(r);
+        store_chunk_cols(v, (float*)c.base, c.ld, c.y, c.xc, lane);
+        if (g + 1 < g1) cursor_next(c, g + 1);
+    };
+    for (int64_t g = g0; g < g1; g += 2) {
+        chunk(g, 0);
+        if (g + 1 < g1) chunk(g + 1, 1);
+    }
+}
+
 }  // namespace tplr
 
 // =========================================================================================
@@ -2008,7 +2127,8 @@ static int launch_encode_as(Kernel kernel, const tplr_tensor_desc* d_desc, const
 template <typename Kernel>
 static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_scale, int n_peers, int k,
                             const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single, int n_tensors,
-                            int64_t total, int reduce_mode, int normalise, float* d_sumsq, void* stream) {
+                            int64_t total, int reduce_mode, int normalise, float* d_sumsq, void* stream,
+                            int64_t stride_idx = 0, int64_t stride_val = 0) {
     static int resident = 0;  // per kernel variant
     if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
     // a wave keeps one mark per chunk of its range (chunks to be done again on the exact path), so
@@ -2019,7 +2139,7 @@ static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_sc
         const int64_t need = ((count + 7) / 8) * 8;
         const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
         hipLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale, n_peers, k, d_desc,
-                           single, n_tensors, first, count, reduce_mode, normalise, d_sumsq);
+                           single, n_tensors, first, count, reduce_mode, normalise, d_sumsq, stride_idx, stride_val);
     }
     return launch_status();
 }
@@ -2290,7 +2410,7 @@ int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, co
     for (int p = 0; p < TPLR_MAX_PEERS; ++p) pp.idx[p] = nullptr, pp.val[p] = nullptr;
     pp.idx[0] = d_idx12;
     pp.val[0] = d_val;
-    return launch_decode_as(k_decode_aggregate<true, 8, 4, true>, pp, nullptr, 1, k, d_ef_desc, none, n_tensors,
+    return launch_decode_as(k_decode_aggregate<true, 8, 4, true, true>, pp, nullptr, 1, k, d_ef_desc, none, n_tensors,
                             total_chunks, TPLR_REDUCE_MEAN, 0, nullptr, stream);
 }
 
@@ -2305,8 +2425,25 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
     }
     // register-resident fast path: k <= 64 and at most 24 peers; 4-bit counters up to 15 peers, 5-bit beyond
     const int units = (k > 64 || normalise) ? 0 : n_peers <= 8 ? 8 : n_peers <= 15 ? 16 : n_peers <= 24 ? 24 : 0;
+    // equally spaced payloads (one staged buffer per window): scalar addressing
+    auto apart = [](const void* a, const void* b) {
+        return static_cast<int64_t>(reinterpret_cast<intptr_t>(a) - reinterpret_cast<intptr_t>(b));
+    };
+    const int64_t si = n_peers > 1 ? apart(pp.idx[1], pp.idx[0]) : 0;       // bytes
+    const int64_t sv4 = n_peers > 1 ? apart(pp.val[1], pp.val[0]) : 0;      // bytes, a multiple of 4
+    const int64_t sv = sv4 / 4;
+    bool strided = true;
+    for (int p = 1; p < n_peers; ++p)
+        strided = strided && apart(pp.idx[p], pp.idx[0]) == p * si && apart(pp.val[p], pp.val[0]) == p * sv4;
 #define TPLR_DECODE_CASE(U, BITS)                                                                                   \
     case U:                                                                                                         \
+        if (strided)                                                                                                \
+            return use_dct ? launch_decode_as(k_decode_aggregate<true, U, BITS, false, true>, pp, d_scale, n_peers,   \
+                                              k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq,  \
+                                              stream, si, sv)                                                        \
+                           : launch_decode_as(k_decode_aggregate<false, U, BITS, false, true>, pp, d_scale, n_peers,  \
+                                              k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq,  \
+                                              stream, si, sv);                                                       \
         return use_dct ? launch_decode_as(k_decode_aggregate<true, U, BITS>, pp, d_scale, n_peers, k, d_desc,         \
                                           single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream)         \
                        : launch_decode_as(k_decode_aggregate<false, U, BITS>, pp, d_scale, n_peers, k, d_desc,        \
@@ -2726,6 +2863,26 @@ int tplr_scale_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t tota
     const int64_t need = ((total_chunks + 7) / 8) * 8;
     hipLaunchKernelGGL(k_scale_chunks, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
                        static_cast<hipStream_t>(stream), d_desc, n_tensors, total_chunks, d_factor);
+    return launch_status();
+}
+
+int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_val, int n_peers, int k,
+                         const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, void* stream) {
+    if (!d_desc || n_tensors < 1 || total_chunks < 0 || n_peers < 0 || k < 2 || (k & 1) || k > 64) return TPLR_E_BADARG;
+    if (n_peers > 24) return TPLR_E_TOOMANY;
+    if (n_peers > 0 && (!h_idx12 || !h_val)) return TPLR_E_BADARG;
+    if (total_chunks == 0) return 0;
+    PeerPtrs pp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        pp.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
+        pp.val[p] = p < n_peers ? h_val[p] : nullptr;
+        if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
+    }
+    static int resident = 0;
+    if (resident == 0) resident = persistent_grid(k_decode_aggregate<true, 16, 4>, int64_t{1} << 40);  // the grid it stands in for
+    const int64_t need = ((total_chunks + 7) / 8) * 8;
+    hipLaunchKernelGGL(k_calib_aggregate, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), pp, n_peers, k, d_desc, n_tensors, total_chunks);
     return launch_status();
 }
 

@@ -131,8 +131,38 @@ def test_normalised_aggregate_with_repeats(dev):
     assert np.array_equal(got.cpu().numpy() != 0, want != 0)
 
 
-@pytest.mark.parametrize("P,k,use_dct", [(15, 32, True), (15, 32, False), (20, 64, True), (31, 32, True)])
-def test_whole_set_aggregate_with_repeats_in_some_rows(dev, P, k, use_dct):
+def staged(di, dv):
+    """The same payloads equally spaced in one buffer (a staged window): the kernels then address the peers
+    with scalar arithmetic, a code path of its own."""
+    P = len(di)
+    ib = torch.empty((P, di[0].numel() + 64), dtype=torch.uint8, device=di[0].device)
+    vb = torch.empty((P, dv[0].numel() + 16), dtype=torch.float32, device=dv[0].device)
+    out_i, out_v = [], []
+    for p in range(P):
+        ib[p, :di[p].numel()] = di[p]
+        vb[p, :dv[p].numel()] = dv[p].reshape(-1)
+        out_i.append(ib[p, :di[p].numel()])
+        out_v.append(vb[p, :dv[p].numel()].view(dv[p].shape))
+    return out_i, out_v
+
+
+@pytest.mark.parametrize("P,k", [(1, 32), (8, 32), (15, 32), (15, 64), (20, 64), (24, 32)])
+@pytest.mark.parametrize("use_dct", [True, False])
+def test_staged_window_gives_the_same_bits_as_separate_payloads(dev, P, k, use_dct):
+    Y, X = 5, 7
+    idxs, vals = peers_with_repeats(P, Y, X, k, 4000 + P + k, every=6)
+    di, dv = on_device(idxs, vals, dev)
+    si, sv = staged(di, dv)
+    assert all(b.data_ptr() - a.data_ptr() == si[1].data_ptr() - si[0].data_ptr() for a, b in zip(si, si[1:])) or P == 1
+    scale = torch.from_numpy((np.random.default_rng(9).random(P) * 0.5 + 0.5).astype(np.float32)).to(dev)
+    want = tc._aggregate_chunks(di, dv, scale, Y, X, k, normalise=False, use_dct=use_dct, rows=True)
+    got = tc._aggregate_chunks(si, sv, scale, Y, X, k, normalise=False, use_dct=use_dct, rows=True)
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+
+
+@pytest.mark.parametrize("P,k,use_dct,window", [(15, 32, True, False), (15, 32, True, True), (15, 32, False, False),
+                                                (15, 32, False, True), (20, 64, True, True), (31, 32, True, False)])
+def test_whole_set_aggregate_with_repeats_in_some_rows(dev, P, k, use_dct, window):
     # enough chunks that every wave walks several, a repeat planted in every 5th row: marked rows in the
     # middle of a wave's range, at its first and at its last chunk; the other rows go the fast way
     shapes = [(64 * 70, 64 * 48), (64 * 33, 64 * 64), (64, 64), (64 * 50, 64 * 40)]
@@ -140,6 +170,8 @@ def test_whole_set_aggregate_with_repeats_in_some_rows(dev, P, k, use_dct):
     n = sum(counts)
     idxs, vals = peers_with_repeats(P, 1, n, k, 77 + P + k, every=5)
     di, dv = on_device(idxs, vals, dev)
+    if window:
+        di, dv = staged(di, dv)
     outs = [torch.full(s, 7.0, device=dev) for s in shapes]
     batch = tc.TensorBatch(outs)
     scale = torch.from_numpy((np.random.default_rng(3).random((len(shapes), P)) * 0.5 + 0.5).astype(np.float32)).to(dev)
