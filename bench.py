@@ -41,8 +41,10 @@ HBM_PEAK_GBPS = 8000.0
 # x 2.000, WRITE_SIZE x 1.000).  The commands and raw figures are in the rocprofv3 summaries kept
 # with the sources.  Only the configuration they were measured on has an entry.
 MEASURED_TRAFFIC = {
-    ("cfg3_llama1b", 15, "encode"): 4_874_638_797,     # 1.001 x algorithmic
-    ("cfg3_llama1b", 15, "aggregate"): 6_068_590_299,  # 1.084 x: streaming loads re-fetch shared index lines
+    ("cfg3_llama1b", 15, "encode"): 4_871_455_590,     # 1.000 x algorithmic
+    ("cfg3_llama1b", 15, "aggregate"): 6_068_903_772,  # 1.085 x: streaming loads re-fetch shared index lines
+    ("cfg5_72b_block", 15, "encode"): 3_586_516_238,
+    ("cfg5_72b_block", 15, "aggregate"): 4_966_891_982,
 }
 
 
@@ -54,9 +56,12 @@ def parse():
     ap.add_argument("--workload", default="cfg3_llama1b", help="cfg1_2048x2048 | cfg2_llama150m | cfg3_llama1b | cfg5_72b_block")
     ap.add_argument("--peers", type=int, default=15)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--profile", choices=["encode", "aggregate", "miner", "copy"], default=None,
+    ap.add_argument("--topk", type=int, default=0, help="top-k per chunk instead of the workload's own (templar runs 64)")
+    ap.add_argument("--no-dct", action="store_true", help="chunks are selected and scattered untransformed (templar's use_dct=false)")
+    ap.add_argument("--profile", choices=["encode", "aggregate", "miner", "copy", "calib", "fill"], default=None,
                     help="run only that phase's batched launches --steps times (for rocprofv3) and print nothing; "
-                         "'copy' runs the library's calibration copy of 1 GiB instead (counter scaling)")
+                         "'copy' runs the library's calibration copy of 1 GiB instead (counter scaling); 'calib' / 'fill' "
+                         "run the memory-only form of the aggregate kernel with / without its payload loads")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline sample")
     return ap.parse_args()
 
@@ -225,8 +230,9 @@ def main():
         assert torch.equal(src, dst)
         return
     cfg = workloads.CONFIGS[args.workload]
-    k, shapes = cfg["k"], cfg["shapes"]
+    k, shapes = (args.topk or cfg["k"]), cfg["shapes"]
     P = args.peers
+    DCT = not args.no_dct
 
     class Shapes:
         def named_parameters(self):
@@ -257,22 +263,22 @@ def main():
         val_buf_1d = torch.empty((rows_1d.total_rows, k1), dtype=torch.float32, device=dev)
 
     def encode2d_only():
-        tc.encode_compress_batch(batch, k, use_dct=True, idx12=idx_buf, val=val_buf)
+        tc.encode_compress_batch(batch, k, use_dct=DCT, idx12=idx_buf, val=val_buf)
 
     def encode_pass():
         encode2d_only()
         if rows_1d is not None:
-            tc.encode_compress_rows_batch(rows_1d, k, use_dct=True, idx12=idx_buf_1d, val=val_buf_1d)
+            tc.encode_compress_rows_batch(rows_1d, k, use_dct=DCT, idx12=idx_buf_1d, val=val_buf_1d)
         elif flat_1d is not None:
-            comp.compress(tr.encode(flat_1d, use_dct=True), k)
+            comp.compress(tr.encode(flat_1d, use_dct=DCT), k)
 
     def encode_per_tensor():
         for g in two_d:
-            tc.encode_compress(g, k, use_dct=True)
+            tc.encode_compress(g, k, use_dct=DCT)
 
     def encode_reference_calls():  # the reference's own two calls per parameter, unchanged
         for g in two_d:
-            comp.compress(tr.encode(g, use_dct=True), k)
+            comp.compress(tr.encode(g, use_dct=DCT), k)
 
     if flat_1d is not None:
         tr.shape_dict[flat_1d.shape[0]] = 64
@@ -296,7 +302,7 @@ def main():
         # the same step through the Python entry point with templar's 4-bin quantiser on
         # (hparams.json:59-60): + one quantise and one de-quantise launch over the payload
         q4 = tc.TopKCompressor(use_quantization=True, quantization_bins=4, quantization_range=6)
-        _, ms_q = event_ms(lambda: tc.error_feedback_step_batch(eb, batch, 0.95, k, use_dct=True, compressor=q4),
+        _, ms_q = event_ms(lambda: tc.error_feedback_step_batch(eb, batch, 0.95, k, use_dct=DCT, compressor=q4),
                            max(3, steps // 4), 1)
         b1 = n_chunks * (2 * 16384 + 16384 + 11 * k // 2)
         b2 = n_chunks * (16384 + 11 * k // 2 + 16384)
@@ -314,12 +320,12 @@ def main():
     # held as a staged window (PayloadStage: one device buffer, the peers' payloads equally spaced), the form
     # in which a gathered window reaches the aggregate
     idxs, vals, idxs_1d, vals_1d = [], [], [], []
-    window = tc.PayloadStage(batch, k, P, quantized=False) if args.profile in (None, "aggregate") else None
+    window = tc.PayloadStage(batch, k, P, quantized=False) if args.profile in (None, "aggregate", "calib", "fill") else None
     for p in range(P if window is not None else 0):  # (a profile of another phase holds only that phase's launches)
         own = [workloads.student_t3(tuple(g.shape), 1000 * (p + 1) + j, row_scale=True, device=dev).add_(g, alpha=0.5)
                for j, g in enumerate(two_d)]
         i12, v = window.regions(p)
-        tc.encode_compress_batch(tc.TensorBatch(own), k, use_dct=True, idx12=i12, val=v)
+        tc.encode_compress_batch(tc.TensorBatch(own), k, use_dct=DCT, idx12=i12, val=v)
         torch.cuda.synchronize()
         idxs.append(i12)
         vals.append(v)
@@ -327,7 +333,7 @@ def main():
         if rows_1d is not None:  # the norm vectors' payloads, same recipe
             own = [workloads.student_t3(tuple(g.shape), 2000 * (p + 1) + j, row_scale=False, device=dev).add_(g, alpha=0.5)
                    for j, g in enumerate(one_d)]
-            i12, v = tc.encode_compress_rows_batch(tc.RowBatch(own), k, use_dct=True)
+            i12, v = tc.encode_compress_rows_batch(tc.RowBatch(own), k, use_dct=DCT)
             idxs_1d.append(i12)
             vals_1d.append(v)
     if args.profile == "miner":
@@ -352,18 +358,18 @@ def main():
     out_batch = batch
 
     def aggregate_2d_pass():
-        tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, clip_norm=True, use_dct=True)
+        tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, clip_norm=True, use_dct=DCT)
 
     def aggregate_pass():
         aggregate_2d_pass()
         if rows_1d is not None:
-            tc.batch_decompress_decode_rows_batch(rows_1d, idxs_1d, vals_1d, min(k, 64), clip_norm=True, use_dct=True,
+            tc.batch_decompress_decode_rows_batch(rows_1d, idxs_1d, vals_1d, min(k, 64), clip_norm=True, use_dct=DCT,
                                                   validate=False)
 
     scale = tc.peer_clip_scales_batch(out_batch, vals, k)
 
     def aggregate_kernel_only():
-        tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, scale=scale, use_dct=True)
+        tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, scale=scale, use_dct=DCT)
 
     # the reference's per-parameter form of the same payloads (lists of P tensors per parameter)
     per_param = []
@@ -373,20 +379,12 @@ def main():
 
     def aggregate_per_tensor():
         for i, (pi, pv, xs) in enumerate(per_param):
-            tc.batch_decompress_decode(pi, pv, xs, out=outs[i])
+            tc.batch_decompress_decode(pi, pv, xs, out=outs[i], use_dct=DCT)
 
     def aggregate_reference_calls():  # batch_decompress then decode per parameter, unchanged
         for i, (pi, pv, xs) in enumerate(per_param):
-            tr.decode(comp.batch_decompress(outs[i], pi, pv, xs, 4096, clip_norm=True), use_dct=True)
+            tr.decode(comp.batch_decompress(outs[i], pi, pv, xs, 4096, clip_norm=True), use_dct=DCT)
 
-    if args.profile == "aggregate":
-        event_ms(aggregate_pass, args.steps, args.warmup)
-        return
-    agg_steps = max(3, args.steps // 2)
-    agg_ms, agg_wall = event_ms(aggregate_pass, agg_steps, 2, settle=True)
-    agg2d_ms, _ = event_ms(aggregate_2d_pass, agg_steps, 1)
-    aggk_ms, _ = event_ms(aggregate_kernel_only, agg_steps, 1)
-    aggk_spread = launch_stats(aggregate_kernel_only, agg_steps)
     # what the memory system alone needs for this launch's traffic: the library's calibration kernel issues the
     # aggregate's loads and stores (same grid, ranges, instructions) without the scatter and the transform
     lib_c = _lib_mod.load()
@@ -398,6 +396,17 @@ def main():
         _lib_mod.check(lib_c.tplr_calib_aggregate(ip_c, vp_c, n_peers, k, out_batch.table.data_ptr(), len(out_batch),
                                                   n_chunks, cur_stream), "tplr_calib_aggregate")
 
+    if args.profile in ("calib", "fill"):
+        event_ms(lambda: calib(P if args.profile == "calib" else 0), args.steps, args.warmup)
+        return
+    if args.profile == "aggregate":
+        event_ms(aggregate_pass, args.steps, args.warmup)
+        return
+    agg_steps = max(3, args.steps // 2)
+    agg_ms, agg_wall = event_ms(aggregate_pass, agg_steps, 2, settle=True)
+    agg2d_ms, _ = event_ms(aggregate_2d_pass, agg_steps, 1)
+    aggk_ms, _ = event_ms(aggregate_kernel_only, agg_steps, 1)
+    aggk_spread = launch_stats(aggregate_kernel_only, agg_steps)
     ceiling = None
     agg_bytes = n_chunks * (P * 11 * k // 2 + 16384)           # the fused kernel's launch
     if P <= 24 and k <= 64:
@@ -466,7 +475,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: encode+top-k+pack of {len(shapes)} tensors "
                                f"({workloads.chunks_2d(shapes)} chunks 64x64, k={k}) and {P}-peer decode-aggregate",
-                   "chunk": 64, "topk": k, "peers": P, "use_dct": True},
+                   "chunk": 64, "topk": k, "peers": P, "use_dct": DCT},
         "clock_settle_s": SETTLE_S,
         "encode_wall_ms": round(enc_wall, 4),
         "aggregate_ms": round(agg_ms, 4),

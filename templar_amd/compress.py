@@ -233,6 +233,9 @@ class ChunkingTransformer:
     @torch.no_grad()
     def __init__(self, model, target_chunk, norm="ortho"):
         self.target_chunk = target_chunk
+        # the factorised 64-point kernels are the orthonormal transform; any other `norm` goes through the
+        # dense contraction with this instance's own bases
+        self._fast64 = norm == "ortho"
         self.shape_dict: dict[int, int] = {}
         self.f_dict: dict[int, torch.Tensor] = {}
         self.b_dict: dict[int, torch.Tensor] = {}
@@ -299,7 +302,7 @@ class ChunkingTransformer:
             if not use_dct:
                 return x.reshape(R // n1, n1, Cc // n2, n2).permute(0, 2, 1, 3)
             _need_device(x, "ChunkingTransformer.encode(use_dct=True)")
-            if n1 == _CH and n2 == _CH:
+            if n1 == _CH and n2 == _CH and self._fast64:
                 lib = _lib.load()
                 xin = x if (x.dtype == torch.float32 and x.stride(1) == 1 and x.stride(0) >= Cc) else _f32c(x)
                 out = torch.empty((R // _CH, Cc // _CH, _CH, _CH), dtype=torch.float32, device=x.device)
@@ -315,7 +318,7 @@ class ChunkingTransformer:
         if not use_dct:
             return rows
         _need_device(x, "ChunkingTransformer.encode(use_dct=True)")
-        if n1 == _CH:
+        if n1 == _CH and self._fast64:
             lib = _lib.load()
             xin = _f32c(rows)
             out = torch.empty_like(xin)
@@ -330,13 +333,15 @@ class ChunkingTransformer:
         """(y, x, h, w) -> (y*h, x*w), or (x, w) -> (x*w,); inverse DCT per chunk when use_dct
         (reference :259-292)."""
         if isinstance(x, LazyAggregate):
+            if use_dct and not self._fast64:  # (the fused kernel is the orthonormal transform)
+                return self.decode(x.dense(), use_dct=True)
             return x.decode(use_dct=use_dct)
         if x.dim() > 2:
             Y, X, h, w = x.shape
             if not use_dct:
                 return x.permute(0, 2, 1, 3).reshape(Y * h, X * w)
             _need_device(x, "ChunkingTransformer.decode(use_dct=True)")
-            if h == _CH and w == _CH:
+            if h == _CH and w == _CH and self._fast64:
                 lib = _lib.load()
                 xin = _f32c(x)
                 out = torch.empty((Y * h, X * w), dtype=torch.float32, device=x.device)
@@ -351,7 +356,7 @@ class ChunkingTransformer:
             return x.reshape(-1)
         _need_device(x, "ChunkingTransformer.decode(use_dct=True)")
         n1 = x.shape[1]
-        if n1 == _CH:
+        if n1 == _CH and self._fast64:
             lib = _lib.load()
             xin = _f32c(x)
             out = torch.empty_like(xin)
@@ -709,7 +714,12 @@ class TopKCompressor:
         parts_i, parts_v = [], []
         for pi, (i_data, v) in enumerate(zip(idxs, vals)):
             v2 = v.reshape(-1, v.shape[-1])
-            if normalise:
+            if normalise and v.dim() == 1:
+                # a single row of values: the reference divides by the norm itself, and only when it
+                # exceeds 1e-8 (:548-551)
+                nrm = torch.linalg.vector_norm(v)
+                v2 = torch.where(nrm > 1e-8, v2 / nrm, v2)
+            elif normalise:
                 v2 = v2 / (torch.linalg.vector_norm(v2, dim=1, keepdim=True) + 1e-8)
             elif scale is not None:
                 v2 = v2 * scale[pi]
@@ -1487,6 +1497,8 @@ class PayloadStage:
         if any(len(row) != P for row in idxs) or any(len(row) != P for row in vals):
             raise IndexError(f"every parameter needs {P} index and value entries")
         on_host = idxs[0][0].device.type == "cpu"
+        if any(t.device.type != idxs[0][0].device.type for row in list(idxs) + list(vals) for t in row):
+            raise ValueError("PayloadStage.load: the lists mix host and device tensors")
         if on_host and self._copied is not None:
             self._copied.synchronize()  # the previous window's copy still reads the pinned buffer
         if on_host:

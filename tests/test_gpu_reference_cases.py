@@ -188,3 +188,33 @@ class _Shapes:
     def named_parameters(self):
         for i, p in enumerate(self._p):
             yield f"p{i}", p
+
+
+def test_transformer_honours_an_unnormalised_basis(dev):
+    # ChunkingTransformer(model, 64, norm=None): the bases are the unnormalised DCT-II (2 sum x cos) and its
+    # inverse, as _dct / _idct build them (src/tplr/compress.py:710-788); 64-element chunks then go through the
+    # dense contraction with those bases, not through the orthonormal kernels
+    import scipy.fft
+    from types import SimpleNamespace
+
+    class M:
+        def named_parameters(self):
+            yield "w", SimpleNamespace(requires_grad=True, shape=(128, 192), dtype=torch.float32, device=dev)
+            yield "b", SimpleNamespace(requires_grad=True, shape=(128,), dtype=torch.float32, device=dev)
+
+    tr = ChunkingTransformer(M(), 64, norm=None)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((128, 192)).astype(np.float32)
+    coef = tr.encode(torch.from_numpy(x).to(dev), use_dct=True)
+    chunks = x.reshape(2, 64, 3, 64).transpose(0, 2, 1, 3)
+    want = scipy.fft.dctn(chunks.astype(np.float64), type=2, norm=None, axes=(2, 3))
+    assert coef.shape == (2, 3, 64, 64)
+    assert np.abs(coef.cpu().numpy() - want).max() <= 1e-5 * np.abs(want).max()
+    back = tr.decode(coef, use_dct=True)
+    assert np.abs(back.cpu().numpy() - x).max() <= 1e-5 * np.abs(x).max()
+    v = rng.standard_normal(128).astype(np.float32)
+    c1 = tr.encode(torch.from_numpy(v).to(dev), use_dct=True)
+    want1 = scipy.fft.dct(v.reshape(2, 64).astype(np.float64), type=2, norm=None, axis=1)
+    assert np.abs(c1.cpu().numpy() - want1).max() <= 1e-5 * np.abs(want1).max()
+    assert np.abs(tr.decode(c1, use_dct=True).cpu().numpy() - v).max() <= 1e-5 * np.abs(v).max()
+
