@@ -444,10 +444,17 @@ __global__ __launch_bounds__(64) void k_encode_rows(const tplr_tensor_desc* __re
     }
     wave_lds_fence();
     regs_to_tile_rows(w, tile, lane);
-    uint64_t key[64];
+    // Keys (magnitude bits, 63 - index) ordered as unsigned 64-bit integers - held as doubles: for positive,
+    // normal, finite doubles the two orders are the same, and a compare-exchange is then one v_max_f64 and one
+    // v_min_f64.  One is added to the exponent field so that a zero magnitude is a normal double, and NaNs share
+    // a magnitude key just below where that addition would reach the doubles' own infinities and NaNs.
+    double key[64];
 #pragma unroll
-    for (int e = 0; e < 64; ++e)
-        key[e] = (static_cast<uint64_t>(mag_key(__builtin_bit_cast(uint32_t, w[e]))) << 32) | static_cast<uint32_t>(63 - e);
+    for (int e = 0; e < 64; ++e) {
+        const uint32_t a = __builtin_bit_cast(uint32_t, w[e]) & 0x7fffffffu;
+        const uint32_t mag = (a > 0x7f800000u ? 0x7fdfffffu : a) + 0x00100000u;
+        key[e] = __builtin_bit_cast(double, (static_cast<uint64_t>(mag) << 32) | static_cast<uint32_t>(63 - e));
+    }
     // bitonic sort, descending
 #pragma unroll
     for (int size = 2; size <= 64; size <<= 1) {
@@ -458,10 +465,10 @@ __global__ __launch_bounds__(64) void k_encode_rows(const tplr_tensor_desc* __re
                 const int l = i ^ stride;
                 if (l > i) {
                     const bool up = (i & size) != 0 && size < 64;  // this run ascends
-                    const uint64_t a = key[i], b = key[l];
-                    const bool swap = up ? a > b : a < b;
-                    key[i] = swap ? b : a;
-                    key[l] = swap ? a : b;
+                    const double a = key[i], b = key[l];
+                    const double hi = __builtin_fmax(a, b), lo = __builtin_fmin(a, b);
+                    key[i] = up ? lo : hi;
+                    key[l] = up ? hi : lo;
                 }
             }
         }
@@ -475,7 +482,8 @@ __global__ __launch_bounds__(64) void k_encode_rows(const tplr_tensor_desc* __re
 #pragma unroll
     for (int j = 0; j < 64; j += 2) {
         if (j < k) {  // k is even
-            const uint32_t i0 = 63u - static_cast<uint32_t>(key[j]), i1 = 63u - static_cast<uint32_t>(key[j + 1]);
+            const uint32_t i0 = 63u - static_cast<uint32_t>(__builtin_bit_cast(uint64_t, key[j]));
+            const uint32_t i1 = 63u - static_cast<uint32_t>(__builtin_bit_cast(uint64_t, key[j + 1]));
             vrow[j] = mine[i0];
             vrow[j + 1] = mine[i1];
             const uint32_t pair = i0 | (i1 << 12);
