@@ -393,7 +393,7 @@ def main():
     cur_stream = torch.cuda.current_stream(dev).cuda_stream
 
     def calib(n_peers):
-        _lib_mod.check(lib_c.tplr_calib_aggregate(ip_c, vp_c, n_peers, k, out_batch.table.data_ptr(), len(out_batch),
+        _lib_mod.check(lib_c.tplr_calib_aggregate(ip_c, vp_c, n_peers, k, int(DCT), out_batch.table.data_ptr(), len(out_batch),
                                                   n_chunks, cur_stream), "tplr_calib_aggregate")
 
     if args.profile in ("calib", "fill"):

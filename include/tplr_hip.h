@@ -336,12 +336,13 @@ int tplr_quantize_batch_static(const float* d_val, int k, const tplr_tensor_desc
 int tplr_calib_copy(const void* d_src, void* d_dst, int64_t n_bytes, void* stream);
 
 /* Measurement aid, no counterpart in the reference: the memory side of tplr_decode_aggregate_batch alone.
- * Same grid, same chunk ranges, the same two streaming loads per peer and chunk (n_peers <= 24, k <= 64) and
- * the same 64 row stores per chunk into the tensors of d_desc, without the scatter and the transform; what
- * it stores is meaningless.  Its duration is the time the memory system needs for the aggregate's traffic in
- * that access pattern - the ceiling the real kernel is held against; n_peers = 0 gives the pure fill of the
- * outputs. */
-int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_val, int n_peers, int k,
+ * Same grid, same chunk ranges, the same streaming payload loads (n_peers <= 24, k <= 64) and the same 64 row
+ * stores per chunk into the tensors of d_desc, without the scatter and the transform; what it stores is
+ * meaningless.  use_dct selects whose loads it issues: with the transform the kernel fetches the packed indices
+ * once per group of four (k <= 32) or two chunks, without it once per chunk.  Its duration is the time the
+ * memory system needs for the aggregate's traffic in that access pattern - the ceiling the real kernel is held
+ * against; n_peers = 0 gives the pure fill of the outputs.  k >= 4 with use_dct. */
+int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_val, int n_peers, int k, int use_dct,
                          const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, void* stream);
 
 #ifdef __cplusplus

@@ -564,6 +564,8 @@ __device__ __forceinline__ uint32_t load_idx12(BytePtr row, int j) {
 
 typedef uint16_t __attribute__((aligned(1))) unaligned_u16;
 using gu16 = __attribute__((address_space(1))) unaligned_u16;
+typedef uint32_t __attribute__((aligned(1))) unaligned_u32;
+using gu32 = __attribute__((address_space(1))) unaligned_u32;
 
 // The fast scatter adds one peer's entries with a plain read-add-write per wave instruction, which is
 // only right when the instruction's destinations are distinct.  A top-k selection has no repeats,
@@ -993,15 +995,14 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     // about as long as one chunk; two chunks of distance keep the wave from waiting for them.
     // =====================================================================================
     if constexpr (kFast && kUseDct) {
-        struct Set {
-            uint32_t ix[kRegs];
+        struct Set {  // one chunk's values
             float a[kRegs];
             float sc;  // lane p: clip factor of peer p for tensor t, times 2^-5
             int t;
         };
         Set s0, s1;
 #pragma unroll
-        for (int i = 0; i < kRegs; ++i) s0.ix[i] = s1.ix[i] = 0, s0.a[i] = s1.a[i] = 0.f;
+        for (int i = 0; i < kRegs; ++i) s0.a[i] = s1.a[i] = 0.f;
         s0.sc = s1.sc = out_scale;
         s0.t = s1.t = -1;
         auto set_scale = [&](Set& st, int t) {  // wave-uniform branch, taken once per tensor
@@ -1010,41 +1011,84 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 st.t = t;
             }
         };
-        // kStrided: `next_i` / `next_v` walk from peer to peer by scalar additions; set_walk puts them on a
-        // chunk's place in peer 0's payload
-        const gbyte* next_i = (const gbyte*)pp.idx[0];
+        // kStrided: `next_v` walks from peer to peer by scalar additions; set_walk puts it on a chunk's place
+        // in peer 0's payload
         const gfloat* next_v = (const gfloat*)pp.val[0];
         // (the peer count as the walk sees it: a copy the optimiser cannot see through, renewed per chunk, or it
         // would keep "stride or 0" for every unit in scalar registers of its own across the loop, and spill them)
         int walk_peers = P;
-        auto set_walk = [&](int64_t off_i, int64_t off_v) {
-            next_i = (const gbyte*)pp.idx[0] + off_i;
+        auto set_walk = [&](int64_t off_v) {
             next_v = (const gfloat*)pp.val[0] + off_v;
             asm volatile("" : "+s"(walk_peers));
         };
         auto set_load_unit = [&](Set& st, int i, int64_t g) {
-            const gbyte* irow = next_i;
             const gfloat* vrow = next_v;
             if constexpr (kStrided) {
-                if (i + 1 < walk_peers) {  // (unused units reload the last peer and stay out of the scatter)
-                    next_i += stride_idx;
-                    next_v += stride_val;
-                }
+                if (i + 1 < walk_peers) next_v += stride_val;  // (unused units reload the last peer and stay out of the scatter)
             } else {
                 const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
-                irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
                 vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
             }
-            // Streaming loads: measured 7 % faster than cached ones for this kernel, although
-            // index rows (1.5 k bytes) of neighbouring chunks share cache lines and those lines
-            // then come in from memory more than once (+0.47 GB on the 1B set, 1.08 x the
-            // algorithmic traffic in total).
-            st.ix[i] = __builtin_nontemporal_load((const gu16*)(irow + lane_ioff));
-            st.a[i] = __builtin_nontemporal_load(vrow + le);
+            st.a[i] = __builtin_nontemporal_load(vrow + le);  // streaming: 7 % faster than cached here
+        };
+        // The packed indices come in once per group of G chunks instead of once per chunk.  A chunk's
+        // index row is 1.5 k bytes, so neighbouring rows share 128-byte lines, and a streaming load per chunk
+        // fetches those lines from memory again and again (3.3 x the index bytes at k = 32).  Here lane l takes
+        // the four bytes at 3 l of the group - the entries 2 l and 2 l + 1 of its G k entries, whatever k - with
+        // one load per peer and group, and entry j of the group's chunk c is fetched from lane (c k + j) / 2 with
+        // a lane permute when it is scattered.  `cur` is the group being scattered, `nxt` the one on its way:
+        // requested two chunks before its first use and moved to `cur` at that use.  A lane whose four bytes would
+        // end past the rows this launch may read starts one byte earlier and shifts that byte out on arrival.
+        const int G = k <= 32 ? 4 : 2;
+        const int64_t piece_end = first + total;
+        uint32_t cur[kRegs], nxt[kRegs];
+        uint32_t nxt_fix = 0;  // bits to shift out of `nxt` when it becomes `cur`
+        const bool tiny = piece_end * idx_stride < 4;  // one row of two entries is all there is: three bytes
+        auto group_load = [&](uint32_t (&dst)[kRegs], int64_t gs, auto first_call) -> uint32_t {
+            if (gs >= piece_end) gs = piece_end - 1;  // (a group nobody will scatter)
+            const int64_t room64 = (piece_end - gs) * idx_stride;
+            const int room = room64 < 4096 ? static_cast<int>(room64) : 4096;
+            // the last pair of the last row starts at room - 3: that lane and those past it read the last four
+            // bytes instead (when a row is three bytes, that begins in the row before: `tiny` is the case without one)
+            const int want = 3 * lane;
+            const int from = want < room - 4 ? want : room - 4;
+            const uint32_t fix = want == room - 3 ? 8u : 0u;
+            const uint32_t off = static_cast<uint32_t>(from + 1);
+            const gbyte* grow = (const gbyte*)pp.idx[0] + uniform64(gs * idx_stride - 1);
+            if constexpr (kStrided) asm volatile("" : "+s"(walk_peers));
+            if constexpr (decltype(first_call)::value) {
+                // (k = 2 makes groups of four rows and a launch of one row has one chunk: no other call is reached)
+                if (tiny) {
+#pragma unroll
+                    for (int i = 0; i < kRegs; ++i) {
+                        const gbyte* row = (const gbyte*)pp.idx[i < P ? i : P - 1];
+                        dst[i] = row[0] | (static_cast<uint32_t>(row[1]) << 8) | (static_cast<uint32_t>(row[2]) << 16);
+                    }
+                    return 0;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kRegs; ++i) {
+                if constexpr (!kStrided) {
+                    const int u = i < P ? i : P - 1;
+                    grow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + (gs * idx_stride - 1);
+                }
+                dst[i] = __builtin_nontemporal_load((const gu32*)(grow + off));
+                if constexpr (kStrided) {
+                    if (i + 1 < walk_peers) grow += stride_idx;
+                }
+            }
+            return fix;
+        };
+        // entry `le` of the group's chunk c sits in lane (c k + le) / 2, in its bits 0-11 or 12-23
+        const uint32_t pair_shift = (le & 1) * 12;
+        const uint32_t pair_lane4 = (static_cast<uint32_t>(le) >> 1) << 2;
+        auto group_entry = [&](uint32_t held, uint32_t from4) -> uint32_t {
+            return static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(static_cast<int>(from4), static_cast<int>(held)));
         };
         auto set_load = [&](Set& st, int64_t g, int t) {
             set_scale(st, t);
-            if constexpr (kStrided) set_walk(uniform64(g * idx_stride), uniform64(g * k));
+            if constexpr (kStrided) set_walk(uniform64(g * k));
 #pragma unroll
             for (int i = 0; i < kRegs; ++i) set_load_unit(st, i, g);
         };
@@ -1057,12 +1101,20 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         Out o0 = out_of(c, g0), o1 = o0, o2 = o0;  // destinations of chunks g, g + 1, g + 2
         // the first chunk: plain serial scatter
         set_load(s0, g0, c.t);
+        {
+            const uint32_t fix = group_load(cur, g0, std::true_type{});
+#pragma unroll
+            for (int i = 0; i < kRegs; ++i) cur[i] >>= fix;
+            if (G == 2) nxt_fix = group_load(nxt, g0 + 2, std::false_type{});
+        }
         zero_tile();
-        if (lane_on) {
+        {
 #pragma unroll
             for (int i = 0; i < kRegs; ++i) {
                 if (i < P) {  // wave-uniform
-                    const uint32_t e = (lane & 1) ? (s0.ix[i] >> 4) : (s0.ix[i] & 0xfffu);
+                    // (every lane takes part in the permute, also those without an entry)
+                    const uint32_t e = __builtin_amdgcn_ubfe(group_entry(cur[i], pair_lane4), pair_shift, 12);
+                    if (!lane_on) continue;
                     float* t = &tile[tile_pos(e)];
                     const float was = tile_claim(t);
                     repeat = seen_mark(repeat, was);
@@ -1103,12 +1155,24 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
 
         // (kStrided) where the chunk loaded last sits in a payload; the loop's loads advance chunk by chunk
         const int64_t loaded_last = g0 + 2 < g1 ? g0 + 2 : g1 - 1;
-        int64_t last_i = uniform64(loaded_last * idx_stride), last_v = uniform64(loaded_last * k);
+        int64_t last_v = uniform64(loaded_last * k);
         const int dummy_pos = kPark ? kTileFloats + lane : lane * kLd + kChunk;
         const uint32_t park = 4096u + lane;  // (kPark) maps to tile[kTileFloats + lane] and cnt[512 + lane / 8]
-        const uint32_t nib_shift = (lane & 1) * 4;  // odd entries sit in the upper 12 bits of their 16
         // one chunk: `st` holds chunk g + 1 and is refilled with chunk g + 3
-        auto step = [&](int64_t g, Set& st) {
+        auto step = [&](int64_t g, Set& st, auto odd) {
+            uint32_t from4 = 0;  // four times the lane that holds this lane's entry of chunk g + 1
+            {
+                const int j = static_cast<int>(g - g0);  // the chunk scattered below is number j + 1 of the range
+                if constexpr (decltype(odd)::value) {
+                    // groups begin at odd steps: G = 4 alternates "request" and "take over", G = 2 does both
+                    if (G == 2 || (j & 2)) {
+#pragma unroll
+                        for (int i = 0; i < kRegs; ++i) cur[i] = nxt[i] >> nxt_fix;
+                    }
+                    if (G == 2 || !(j & 2)) nxt_fix = group_load(nxt, g0 + ((j + 3) & ~(G - 1)), std::false_type{});
+                }
+                from4 = pair_lane4 + static_cast<uint32_t>(((j + 1) & (G - 1)) * 2 * k);
+            }
             float v[64];
             tile_rows_to_regs(v, tile, lane);
             dct64_inv(v);  // along d: v[l] = sum_d Y[lane][d] F[l][d]
@@ -1129,16 +1193,19 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             }
             const int64_t g_load = more3 ? g + 3 : g1 - 1;
             if constexpr (kStrided) {
-                if (more3) {
-                    last_i += idx_stride;
-                    last_v += k;
-                }
-                set_walk(last_i, last_v);
+                if (more3) last_v += k;
+                set_walk(last_v);
             }
             constexpr int kSteps = kUnits + 1;
             constexpr int kAlways = kUnits > 8 ? kUnits - 8 : 1;  // units every served peer count uses
             int pos = kPark ? dummy_pos * 4 : dummy_pos;  // (kPark: a byte offset)
-            float cur = 0.f, add = 0.f;
+            float cur_sum = 0.f, add = 0.f;
+            // units this lane scatters: a per-lane count compared per unit (a mask per unit, kept across the
+            // loop, would take sixteen scalar registers that are not there)
+            int my_units = lane_on ? P : 0;
+            asm volatile("" : "+v"(my_units));
+            // the register with the next unit's entry, on its way from another lane
+            uint32_t held = group_entry(cur[0], from4);
             float before[kSubtract ? 64 : 1];
             if constexpr (kSubtract)
                 load_chunk_rows(before, (const void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane);
@@ -1149,32 +1216,34 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 constexpr int s = (h * kSteps + kDctHooks - 1) / kDctHooks;
                 if constexpr (s < kSteps && (s * kDctHooks) / kSteps == h) {
                     if constexpr (s > 0) {
-                        repeat = seen_mark(repeat, cur);
+                        repeat = seen_mark(repeat, cur_sum);
                         if constexpr (kPark)
-                            *reinterpret_cast<float*>(reinterpret_cast<char*>(tile) + pos) = cur + add;
+                            *reinterpret_cast<float*>(reinterpret_cast<char*>(tile) + pos) = cur_sum + add;
                         else
-                            tile[pos] = cur + add;
+                            tile[pos] = cur_sum + add;
                         set_load_unit(st, s - 1, g_load);
                     }
                     if constexpr (s < kUnits) {
                         constexpr int u = s;
-                        const bool on = lane_on && (u < kAlways || u < P);
+                        const bool on = u < kAlways ? lane_on : u < my_units;
                         add = st.a[u] * unit_scale(sc_now, u);
+                        const uint32_t packed = __builtin_amdgcn_ubfe(held, pair_shift, 12);
                         if constexpr (kPark) {
                             // byte addresses by hand: slot 4 e + 16 (e >> 6), counter word 4 (e >> 3), its
                             // field 4 (e & 7) bits up - seven instructions from the packed index
-                            const uint32_t e = on ? __builtin_amdgcn_ubfe(st.ix[u], nib_shift, 12) : park;
+                            const uint32_t e = on ? packed : park;
                             const uint32_t e4 = e << 2;
                             pos = static_cast<int>(e4 + ((e >> 2) & 0x7f0u));
-                            cur = tile_claim(reinterpret_cast<float*>(reinterpret_cast<char*>(tile) + pos));
+                            cur_sum = tile_claim(reinterpret_cast<float*>(reinterpret_cast<char*>(tile) + pos));
                             atomicAdd(reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(cnt) + ((e >> 1) & 0xffcu)),
                                       1u << (e4 & 28u));
                         } else {
-                            const uint32_t e = __builtin_amdgcn_ubfe(st.ix[u], nib_shift, 12);
+                            const uint32_t e = packed;
                             pos = on ? static_cast<int>(e + ((e >> 6) << 2)) : dummy_pos;
-                            cur = tile_claim(&tile[pos]);
+                            cur_sum = tile_claim(&tile[pos]);
                             atomicAdd(&cnt[on ? Cnt::word(e) : lane], on ? 1u << Cnt::shift(e) : 0u);
                         }
+                        if constexpr (s + 1 < kUnits) held = group_entry(cur[s + 1], from4);
                     }
                 }
             });
@@ -1203,8 +1272,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             o2 = o3;
         };
         for (int64_t g = g0; g < g1; g += 2) {
-            step(g, s1);
-            if (g + 1 < g1) step(g + 1, s0);
+            step(g, s1, std::false_type{});
+            if (g + 1 < g1) step(g + 1, s0, std::true_type{});
         }
         redo_marked();
         return;
@@ -2034,11 +2103,11 @@ __global__ __launch_bounds__(256) void k_calib_copy(const v4f* __restrict__ src,
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
 
-// The memory side of k_decode_aggregate alone, for calibration: the same persistent grid and chunk
-// ranges, the same payload loads (every peer's two loads per chunk, streaming, requested two chunks
-// ahead) and the same 64 row stores per chunk, but no LDS work and no arithmetic beyond folding the
-// loaded values into what is stored.  Its duration is what the memory system needs for the
-// aggregate's traffic in this access pattern; with n_peers = 0 it is the pure fill of the outputs.
+// The memory side of the fast aggregate alone: same grid, same chunk ranges, the same payload loads and the
+// same 64 row stores per chunk, no scatter and no transform (what it stores is meaningless).  kGroup = 0: one
+// two-byte index load per peer and chunk, as the kernels without the transform issue them; kGroup = 4 or 2:
+// one four-byte load per peer and group of that many chunks, as the pipeline with the transform does.
+template <int kGroup>
 __global__ __launch_bounds__(64, 2) void k_calib_aggregate(const PeerPtrs pp, int P, int k,
                                                            const tplr_tensor_desc* __restrict__ table, int n_tensors,
                                                            int64_t total) {
@@ -2056,13 +2125,20 @@ __global__ __launch_bounds__(64, 2) void k_calib_aggregate(const PeerPtrs pp, in
     for (int s = 0; s < 2; ++s)
 #pragma unroll
         for (int i = 0; i < kU; ++i) ix[s][i] = 0, a[s][i] = 0.f;
-    auto load = [&](int s, int64_t g) {
+    auto load = [&](int s, int64_t g, auto with_group) {
+        // (a group's lanes as the kernel places them: four bytes at 3 * lane, kept inside the rows of this launch)
+        int64_t room = (total - g) * idx_stride - 4;
+        if (room < 0) room = 0;
+        const int64_t goff = 3 * lane < room ? 3 * lane : room;
 #pragma unroll
         for (int i = 0; i < kU; ++i) {
             if (i < P) {  // wave-uniform
                 const gbyte* irow = (const gbyte*)pp.idx[i] + g * idx_stride;
                 const gfloat* vrow = (const gfloat*)pp.val[i] + g * k;
-                ix[s][i] = __builtin_nontemporal_load((const gu16*)(irow + lane_ioff));
+                if constexpr (kGroup == 0)
+                    ix[s][i] = __builtin_nontemporal_load((const gu16*)(irow + lane_ioff));
+                else if constexpr (decltype(with_group)::value)
+                    ix[0][i] = __builtin_nontemporal_load((const gu32*)(irow + goff));
                 a[s][i] = __builtin_nontemporal_load(vrow + le);
             }
         }
@@ -2070,22 +2146,32 @@ __global__ __launch_bounds__(64, 2) void k_calib_aggregate(const PeerPtrs pp, in
     Cursor c;
     tplr_tensor_desc none = {};
     cursor_seek(c, table, none, n_tensors, g0);
-    load(0, g0);
-    load(1, g0 + 1 < g1 ? g0 + 1 : g0);
-    auto chunk = [&](int64_t g, int s) {
+    load(0, g0, std::true_type{});
+    load(1, g0 + 1 < g1 ? g0 + 1 : g0, std::false_type{});
+    auto chunk = [&](int64_t g, int s, auto with_group) {
         float x = 0.f;
 #pragma unroll
-        for (int i = 0; i < kU; ++i) x += a[s][i] + __builtin_bit_cast(float, ix[s][i]);
-        load(s, g + 2 < g1 ? g + 2 : g1 - 1);
+        for (int i = 0; i < kU; ++i) x += a[s][i] + __builtin_bit_cast(float, ix[kGroup ? 0 : s][i]);
+        load(s, g + 2 < g1 ? g + 2 : g1 - 1, with_group);
         float v[64];
 #pragma unroll
         for (int r = 0; r < 64; ++r) v[r] = x + static_cast<float>(r);
         store_chunk_cols(v, (float*)c.base, c.ld, c.y, c.xc, lane);
         if (g + 1 < g1) cursor_next(c, g + 1);
     };
-    for (int64_t g = g0; g < g1; g += 2) {
-        chunk(g, 0);
-        if (g + 1 < g1) chunk(g + 1, 1);
+    // the payload requested while chunk g is stored is that of chunk g + 2: a group starts there every kGroup chunks
+    if constexpr (kGroup == 4) {
+        for (int64_t g = g0; g < g1; g += 4) {
+            chunk(g, 0, std::false_type{});
+            if (g + 1 < g1) chunk(g + 1, 1, std::false_type{});
+            if (g + 2 < g1) chunk(g + 2, 0, std::true_type{});
+            if (g + 3 < g1) chunk(g + 3, 1, std::false_type{});
+        }
+    } else {
+        for (int64_t g = g0; g < g1; g += 2) {
+            chunk(g, 0, std::true_type{});
+            if (g + 1 < g1) chunk(g + 1, 1, std::false_type{});
+        }
     }
 }
 
@@ -2874,11 +2960,12 @@ int tplr_scale_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t tota
     return launch_status();
 }
 
-int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_val, int n_peers, int k,
+int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_val, int n_peers, int k, int use_dct,
                          const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, void* stream) {
     if (!d_desc || n_tensors < 1 || total_chunks < 0 || n_peers < 0 || k < 2 || (k & 1) || k > 64) return TPLR_E_BADARG;
     if (n_peers > 24) return TPLR_E_TOOMANY;
     if (n_peers > 0 && (!h_idx12 || !h_val)) return TPLR_E_BADARG;
+    if (use_dct && k < 4) return TPLR_E_BADARG;  // (a group's four-byte loads need rows of at least four bytes)
     if (total_chunks == 0) return 0;
     PeerPtrs pp;
     for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
@@ -2889,8 +2976,14 @@ int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_va
     static int resident = 0;
     if (resident == 0) resident = persistent_grid(k_decode_aggregate<true, 16, 4>, int64_t{1} << 40);  // the grid it stands in for
     const int64_t need = ((total_chunks + 7) / 8) * 8;
-    hipLaunchKernelGGL(k_calib_aggregate, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
-                       static_cast<hipStream_t>(stream), pp, n_peers, k, d_desc, n_tensors, total_chunks);
+    const dim3 grid(static_cast<unsigned>(need < resident ? need : resident));
+    const hipStream_t on = static_cast<hipStream_t>(stream);
+    if (!use_dct)
+        hipLaunchKernelGGL(k_calib_aggregate<0>, grid, dim3(64), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
+    else if (k <= 32)
+        hipLaunchKernelGGL(k_calib_aggregate<4>, grid, dim3(64), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
+    else
+        hipLaunchKernelGGL(k_calib_aggregate<2>, grid, dim3(64), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
     return launch_status();
 }
 

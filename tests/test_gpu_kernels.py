@@ -376,6 +376,47 @@ def test_aggregate_fused_with_inverse_dct(dev, P, k):
     assert relerr(tr.decode(dense, use_dct=True).cpu().numpy(), want) <= TOL
 
 
+@pytest.mark.parametrize("k", [2, 4, 6, 30, 32, 34, 62, 64])
+@pytest.mark.parametrize("Y,X", [(1, 1), (1, 2), (1, 3), (3, 3)])
+def test_aggregate_with_transform_short_payloads(dev, k, Y, X):
+    """The kernel fetches packed indices four bytes at a time for groups of rows: the last rows of a payload, rows of
+    three bytes (k = 2) and payloads of a single row must come out as any other (peers strided and not)."""
+    for P, strided in ((1, True), (3, True), (3, False)):
+        idxs, vals = make_peers(P, Y, X, k, 1000 * k + 10 * Y + X + P)
+        want = orc.decode2d(orc.batch_decompress(idxs, vals, (Y, X, 64, 64), 4096, clip_norm=False))
+        if strided:  # equally spaced in one allocation each, exactly sized: nothing behind the last row
+            ibuf = torch.from_numpy(np.stack([i.reshape(-1) for i in idxs])).to(dev)
+            vbuf = torch.from_numpy(np.stack([v.reshape(-1) for v in vals])).to(dev)
+            di = [ibuf[p].view(Y * X, -1) for p in range(P)]
+            dv = [vbuf[p].view(Y * X, k) for p in range(P)]
+        else:
+            di = [torch.from_numpy(i).to(dev) for i in idxs]
+            dv = [torch.from_numpy(v).to(dev) for v in vals]
+            di[-1] = torch.cat([torch.zeros(5, dtype=torch.uint8, device=dev), di[-1].reshape(-1)])[5:].view(Y * X, -1)
+        got = tc.batch_decompress_decode(di, dv, (Y, X, 64, 64), clip_norm=False)
+        assert relerr(got.cpu().numpy(), want) <= TOL, (P, strided)
+
+
+def test_aggregate_with_transform_many_chunks_per_wave(dev):
+    """More chunks than resident waves, so that every wave walks several index groups and ends inside one."""
+    k, P = 32, 2
+    Y, X = 4, 2100                               # 8400 chunks on some 2000 waves: ranges of four and five chunks
+    g = torch.Generator(device=dev); g.manual_seed(5)
+    idx = torch.rand((P, Y * X, 4096), device=dev, generator=g).topk(k, dim=-1).indices
+    val = torch.randn((P, Y * X, k), device=dev, generator=g)
+    di = [tc.pack_12bit_indices(idx[p].contiguous()) for p in range(P)]
+    dv = [val[p].contiguous() for p in range(P)]
+    got = tc.batch_decompress_decode(di, dv, (Y, X, 64, 64), clip_norm=False)
+    dense = torch.zeros((Y * X, 4096), device=dev)
+    cnt = torch.zeros((Y * X, 4096), device=dev)
+    for p in range(P):
+        dense.scatter_add_(1, idx[p], val[p])
+        cnt.scatter_add_(1, idx[p], torch.ones_like(val[p]))
+    dense = dense / cnt.clamp(min=1)
+    want = orc.decode2d(dense.view(Y, X, 64, 64).cpu().numpy())
+    assert relerr(got.cpu().numpy(), want) <= TOL
+
+
 def test_scatter_rows_generic(dev):
     rng = np.random.default_rng(8)
     comp = tc.TopKCompressor()
