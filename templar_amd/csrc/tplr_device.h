@@ -451,27 +451,44 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
     }
     uint32_t slot = incl - cnt;  // exclusive prefix of the per-lane counts
 
-    // compaction: each half of the wave in turn parks its rows in the staging buffer, so that a
-    // lane can fetch its own candidates with a run-time column index
-    float* row = buf + (lane & 31) * kLd;
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-        if ((lane >> 5) == half) {
-            regs_to_tile_rows(w, buf, lane & 31);
-            while (mhi | mlo) {
-                const bool hi = mhi != 0;
-                const uint32_t m = hi ? mhi : mlo;
-                const int z = __builtin_clz(m);
-                const uint32_t cleared = m & ~(0x80000000u >> z);
-                mhi = hi ? cleared : mhi;
-                mlo = hi ? mlo : cleared;
-                const int d = hi ? z : 32 + z;
-                const uint32_t bits = __float_as_uint(row[d]);
-                const uint32_t ix = lane * 64 + d;
-                cand[slot++] = (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - ix) << 1) | (bits >> 31);
-            }
+    // compaction: lanes park their rows in the staging buffer, so that a lane can fetch its own
+    // candidates with a run-time column index
+    auto compact = [&](const float* row) {
+        while (mhi | mlo) {
+            const bool hi = mhi != 0;
+            const uint32_t m = hi ? mhi : mlo;
+            const int z = __builtin_clz(m);
+            const uint32_t cleared = m & ~(0x80000000u >> z);
+            mhi = hi ? cleared : mhi;
+            mlo = hi ? mlo : cleared;
+            const int d = hi ? z : 32 + z;
+            const uint32_t bits = __float_as_uint(row[d]);
+            const uint32_t ix = lane * 64 + d;
+            cand[slot++] = (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - ix) << 1) | (bits >> 31);
+        }
+    };
+    // The threshold is the k-th largest lane maximum, so with k <= 32 and no ties there are exactly k lanes
+    // that hold candidates: their rows fit the buffer's 32 together, each at its rank among those lanes, and
+    // one pass serves all of them (its length is the largest number of candidates in one lane).  Otherwise
+    // each half of the wave takes its turn.
+    const uint64_t holders = __ballot(cnt != 0);
+    if (!kTwo && __popcll(holders) <= 32) {  // wave-uniform
+        if (cnt != 0) {
+            const int r = static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(holders >> 32),
+                                           __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(holders), 0u)));
+            regs_to_tile_rows(w, buf, r);
+            compact(buf + r * kLd);
         }
         wave_lds_fence();
+    } else {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            if ((lane >> 5) == half) {
+                regs_to_tile_rows(w, buf, lane & 31);
+                compact(buf + (lane & 31) * kLd);
+            }
+            wave_lds_fence();
+        }
     }
 
     Selected out;

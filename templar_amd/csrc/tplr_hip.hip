@@ -246,7 +246,10 @@ __device__ __forceinline__ void cursor_next(Cursor& c, int64_t g) {
 
 // the contiguous slice of [0, total) that workgroup `bid` of a grid of G (multiple of 8) owns;
 // workgroups b, b+8, b+16, ... run on the same XCD and take neighbouring slices
-__device__ __forceinline__ void my_range(int64_t total, int64_t& g0, int64_t& g1) {
+// `align` > 1 (a power of two): where slices are long (64 items and more), the boundaries between the
+// slices of one XCD fall on multiples of `align` counted from -`first`, i.e. on absolute multiples when
+// [0, total) stands for the items first .. first + total - 1 of a longer list
+__device__ __forceinline__ void my_range(int64_t total, int64_t& g0, int64_t& g1, int align = 1, int64_t first = 0) {
     const int64_t bid = blockIdx.x, S = gridDim.x >> 3;
     const int64_t xcd = bid & 7, slot = bid >> 3;
     const int64_t per = (total + 7) >> 3;
@@ -256,6 +259,12 @@ __device__ __forceinline__ void my_range(int64_t total, int64_t& g0, int64_t& g1
     const int64_t len = xe > xb ? xe - xb : 0;
     g0 = xb + len * slot / S;
     g1 = xb + len * (slot + 1) / S;
+    if (align > 1 && len >= 64 * S) {
+        if (slot > 0) g0 = ((g0 + first) & ~static_cast<int64_t>(align - 1)) - first;
+        if (slot + 1 < S) g1 = ((g1 + first) & ~static_cast<int64_t>(align - 1)) - first;
+        g0 = g0 < xb ? xb : g0;
+        g1 = g1 < xb ? xb : g1;
+    }
 }
 
 template <int kRow0 = 0, int kRow1 = 64>
@@ -651,7 +660,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     constexpr int kRegs = kFast ? kUnits : 1;
     const int lane = threadIdx.x;
     int64_t g0, g1;
-    my_range(total, g0, g1);
+    // (the pipeline with the transform fetches packed indices per group of four or two chunks: slices that
+    // begin on a multiple of that keep every group inside two 128-byte lines)
+    my_range(total, g0, g1, kUnits > 0 && kUseDct ? (k <= 32 ? 4 : 2) : 1, first);
     if (g0 >= g1) return;
     g0 += first;
     g1 += first;
@@ -1046,10 +1057,14 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         const bool tiny = piece_end * idx_stride < 4;  // one row of two entries is all there is: three bytes
         auto group_load = [&](uint32_t (&dst)[kRegs], int64_t gs, auto first_call) -> uint32_t {
             if (gs >= piece_end) gs = piece_end - 1;  // (a group nobody will scatter)
+            // bytes to read from: the group, or what is left of the rows of this launch.  The group's last pair
+            // is its last three bytes, and a fourth byte behind them would be the first of another 128-byte line
+            // every other group
             const int64_t room64 = (piece_end - gs) * idx_stride;
-            const int room = room64 < 4096 ? static_cast<int>(room64) : 4096;
-            // the last pair of the last row starts at room - 3: that lane and those past it read the last four
-            // bytes instead (when a row is three bytes, that begins in the row before: `tiny` is the case without one)
+            const int group_bytes = G * static_cast<int>(idx_stride);
+            const int room = room64 < group_bytes ? static_cast<int>(room64) : group_bytes;
+            // the last pair starts at room - 3: that lane and those past it read the last four bytes instead
+            // (when a row is three bytes, that begins in the row before: `tiny` is the case without one)
             const int want = 3 * lane;
             const int from = want < room - 4 ? want : room - 4;
             const uint32_t fix = want == room - 3 ? 8u : 0u;
@@ -2113,7 +2128,7 @@ __global__ __launch_bounds__(64, 2) void k_calib_aggregate(const PeerPtrs pp, in
                                                            int64_t total) {
     const int lane = threadIdx.x;
     int64_t g0, g1;
-    my_range(total, g0, g1);
+    my_range(total, g0, g1, kGroup ? kGroup : 1);
     if (g0 >= g1) return;
     const int64_t idx_stride = k + (k >> 1);
     const int le = lane < k ? lane : 0;
@@ -2127,8 +2142,9 @@ __global__ __launch_bounds__(64, 2) void k_calib_aggregate(const PeerPtrs pp, in
         for (int i = 0; i < kU; ++i) ix[s][i] = 0, a[s][i] = 0.f;
     auto load = [&](int s, int64_t g, auto with_group) {
         // (a group's lanes as the kernel places them: four bytes at 3 * lane, kept inside the rows of this launch)
-        int64_t room = (total - g) * idx_stride - 4;
-        if (room < 0) room = 0;
+        int64_t room = (total - g) * idx_stride;
+        if (kGroup && room > kGroup * idx_stride) room = kGroup * idx_stride;
+        room = room < 4 ? 0 : room - 4;
         const int64_t goff = 3 * lane < room ? 3 * lane : room;
 #pragma unroll
         for (int i = 0; i < kU; ++i) {
@@ -2227,7 +2243,8 @@ static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_sc
     if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
     // a wave keeps one mark per chunk of its range (chunks to be done again on the exact path), so
     // one launch takes at most kMaxChunksPerWave chunks per wave: 68 GB of output on a whole device
-    const int64_t piece = static_cast<int64_t>(resident) * (kMaxChunksPerWave - 2);
+    // (the margin covers the rounding of the slices and their alignment to index groups)
+    const int64_t piece = static_cast<int64_t>(resident) * (kMaxChunksPerWave - 8);
     for (int64_t first = 0; first < total; first += piece) {
         const int64_t count = total - first < piece ? total - first : piece;
         const int64_t need = ((count + 7) / 8) * 8;
