@@ -1990,7 +1990,7 @@ __global__ __launch_bounds__(1024) void k_peer_sumsq(const ValPtrs vp, int64_t n
 __global__ __launch_bounds__(1024) void k_segment_sumsq(const ValPtrs vp, int P, int k, int S,
                                                         const tplr_tensor_desc* __restrict__ table,
                                                         float* __restrict__ sumsq) {
-    constexpr int kT = 1024, kU = 16;
+    constexpr int kT = 1024;
     __shared__ float part[kT / 64];
     // block = (tensor t, peer p, slice sl); a slice is a run of whole chunks
     const int tp = blockIdx.x / S, sl = blockIdx.x - tp * S;
@@ -1998,28 +1998,43 @@ __global__ __launch_bounds__(1024) void k_segment_sumsq(const ValPtrs vp, int P,
     const tplr_tensor_desc d = table[t];
     const int64_t n_chunks = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
     const int64_t c0 = n_chunks * sl / S, c1 = n_chunks * (sl + 1) / S;
-    const int64_t n2 = (c1 - c0) * k / 2;
+    // a slice is often no more than a few loads per lane (64 KB for a 2048 x 2048 parameter cut in two): four
+    // independent streaming loads per trip, 16 bytes wide where rows of k values keep that alignment
     typedef float v2f __attribute__((ext_vector_type(2)));
-    const v2f* v = reinterpret_cast<const v2f*>(vp.val[p] + (d.chunk_begin + c0) * k);
-    float acc[kU];
-#pragma unroll
-    for (int u = 0; u < kU; ++u) acc[u] = 0.f;
+    const float* base = vp.val[p] + (d.chunk_begin + c0) * k;
+    const int64_t n = (c1 - c0) * k;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    auto sq4 = [](float a, v4f x) {
+        return __builtin_fmaf(x.w, x.w, __builtin_fmaf(x.z, x.z, __builtin_fmaf(x.y, x.y, __builtin_fmaf(x.x, x.x, a))));
+    };
     int64_t i = threadIdx.x;
-    for (; i + (kU - 1) * kT < n2; i += kU * kT) {
-        v2f x[kU];
+    if ((k & 3) == 0 && (reinterpret_cast<uintptr_t>(base) & 15) == 0) {
+        const v4f* v = reinterpret_cast<const v4f*>(base);
+        const int64_t n4 = n >> 2;
+        for (; i + 3 * kT < n4; i += 4 * kT) {
+            v4f x[4];
 #pragma unroll
-        for (int u = 0; u < kU; ++u) x[u] = __builtin_nontemporal_load(v + i + u * kT);
+            for (int u = 0; u < 4; ++u) x[u] = __builtin_nontemporal_load(v + i + u * kT);
 #pragma unroll
-        for (int u = 0; u < kU; ++u) acc[u] = __builtin_fmaf(x[u].y, x[u].y, __builtin_fmaf(x[u].x, x[u].x, acc[u]));
+            for (int u = 0; u < 4; ++u) acc[u] = sq4(acc[u], x[u]);
+        }
+        for (int u = 0; i < n4; i += kT, u = (u + 1) & 3) acc[u] = sq4(acc[u], __builtin_nontemporal_load(v + i));
+    } else {
+        const v2f* v = reinterpret_cast<const v2f*>(base);
+        const int64_t n2 = n >> 1;
+        for (; i + 3 * kT < n2; i += 4 * kT) {
+            v2f x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = __builtin_nontemporal_load(v + i + u * kT);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc[u] = __builtin_fmaf(x[u].y, x[u].y, __builtin_fmaf(x[u].x, x[u].x, acc[u]));
+        }
+        for (; i < n2; i += kT) {
+            const v2f x = __builtin_nontemporal_load(v + i);
+            acc[0] = __builtin_fmaf(x.y, x.y, __builtin_fmaf(x.x, x.x, acc[0]));
+        }
     }
-    for (; i < n2; i += kT) {
-        const v2f x = v[i];
-        acc[0] = __builtin_fmaf(x.y, x.y, __builtin_fmaf(x.x, x.x, acc[0]));
-    }
-#pragma unroll
-    for (int w = kU / 2; w > 0; w >>= 1)
-#pragma unroll
-        for (int u = 0; u < w; ++u) acc[u] += acc[u + w];
+    acc[0] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
     const float s = wave_sum_f32(acc[0]);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
     __syncthreads();
