@@ -421,6 +421,8 @@ def main():
     # the aggregation as the benchmark's workload words it: sum over the peers, inverse transform, mean over
     # the peers, every tensor divided by its L2 norm (three launches; tplr.compress itself has no such mode)
     aggn_ms, _ = event_ms(lambda: tc.aggregate_mean_normalised_batch(out_batch, idxs, vals, k), agg_steps, 1)
+    aggn2_ms, _ = event_ms(lambda: tc.aggregate_mean_normalised_batch(out_batch, idxs, vals, k, two_pass=True),
+                           agg_steps, 1)
     agg_pt_ms, _ = event_ms(aggregate_per_tensor, 3, 1)
     agg_rc_ms, _ = event_ms(aggregate_reference_calls, 3, 1)
     # the same per-parameter loop recorded once into a HIP graph and replayed: what is left is device time
@@ -484,9 +486,13 @@ def main():
         "aggregate_2d_ms": round(agg2d_ms, 4),
         "aggregate_sum_mean_normalised_ms": round(aggn_ms, 4),
         "aggregate_sum_mean_normalised_note": "the workload's own wording: scatter-sum over the peers, inverse DCT, "
-                                              "divide by their number, divide each tensor by its L2 norm (aggregate in "
-                                              "sum mode + per-tensor norms + one scaling pass); aggregate_ms is the "
+                                              "divide by their number, divide each tensor by its L2 norm; the norms "
+                                              "come from the payloads (orthonormal transform: one launch over the "
+                                              "payload, no dense traffic) and are folded into the factors of the one "
+                                              "aggregate launch; _two_pass_ms is the literal order (aggregate, norms "
+                                              "of the dense result, one scaling pass); aggregate_ms is the "
                                               "reference's batch_decompress semantics",
+        "aggregate_sum_mean_normalised_two_pass_ms": round(aggn2_ms, 4),
         "ms_per_step_spread": {"median": enc_spread[0], "min": enc_spread[1], "max": enc_spread[2],
                                "what": "per-call durations of a further `steps` calls of the step, each between its own events"},
         "per_tensor_launches": {"encode_ms": round(enc_pt_ms, 4), "aggregate_ms": round(agg_pt_ms, 4),

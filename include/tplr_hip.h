@@ -315,6 +315,21 @@ int tplr_tensor_rnorm(const float* d_sumsq, const tplr_tensor_desc* d_desc, int 
 int tplr_scale_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, const float* d_factor,
                      void* stream);
 
+/* The same normalisation without a pass over the dense tensors.  The transform is orthonormal, so the L2
+ * norm of a decoded tensor is the norm of its summed coefficients, which the payloads alone determine.
+ * tplr_aggregate_sumsq_batch: d_sumsq[g] = sum over the coefficients of chunk g of (sum over the peers'
+ * entries for that coefficient, each times d_scale[t * n_peers + p] when d_scale is given)^2; reads the
+ * payloads only (arguments as tplr_decode_aggregate_batch, any even k up to 4096, repeated indices added
+ * like any other entry).
+ * tplr_tensor_rnorm_scales: d_factor[t] (optional) = 1 / (sqrt(sum of tensor t's d_sumsq entries) * pre + eps)
+ * and d_scale[t * n_peers + p] = pre * d_factor[t] for every p: with pre = 1 / n_peers, the factors that make
+ * tplr_decode_aggregate_batch in TPLR_REDUCE_SUM mode write mean-over-peers / (its L2 norm + eps) directly. */
+int tplr_aggregate_sumsq_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale,
+                               int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
+                               int64_t total_chunks, float* d_sumsq, void* stream);
+int tplr_tensor_rnorm_scales(const float* d_sumsq, const tplr_tensor_desc* d_desc, int n_tensors, int n_peers,
+                             float pre, float eps, float* d_factor, float* d_scale, void* stream);
+
 /* tplr_quantize_batch for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc); it has no counterpart in the
  * reference.  Same arguments and results without d_work: the partial sums go through a static

@@ -55,6 +55,8 @@ SIGNATURES = {
     "tplr_quantize_batch": (_i32, [_vp, _i32, _vp, _i32, _i32, C.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
     "tplr_tensor_rnorm": (_i32, [_vp, _vp, _i32, C.c_float, _vp, _vp]),
     "tplr_scale_batch": (_i32, [_vp, _i32, _i64, _vp, _vp]),
+    "tplr_aggregate_sumsq_batch": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp]),
+    "tplr_tensor_rnorm_scales": (_i32, [_vp, _vp, _i32, _i32, C.c_float, C.c_float, _vp, _vp, _vp]),
     "tplr_static_work_bytes": (_i64, []),
     "tplr_quantize_batch_static": (_i32, [_vp, _i32, _vp, _i32, _i32, C.c_float, _i32, _vp, _vp, _vp, _vp, _vp]),
     "tplr_index_stats_batch": (_i32, [_vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp, _vp, _vp]),

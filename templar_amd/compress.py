@@ -1014,23 +1014,45 @@ def batch_decompress_decode_batch(out: TensorBatch, idxs: Sequence[torch.Tensor]
 
 @torch.no_grad()
 def aggregate_mean_normalised_batch(out: TensorBatch, idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], k: int,
-                                    *, use_dct: bool = True, eps: float = 1e-8) -> torch.Tensor:
+                                    *, use_dct: bool = True, eps: float = 1e-8, two_pass: bool = False) -> torch.Tensor:
     """The aggregation as the benchmark's workload words it: every peer's payload scatter-summed, inverse
     transform, mean over the peers (the sum divided by their number, whoever sent a coefficient), then
-    every tensor divided by its L2 norm (+ eps).  Three launches: the aggregate in sum mode with the factor
-    1/P on every peer and per-chunk sums of squares, the per-tensor norms from those, one scaling pass.
-    tplr.compress itself has no such mode (batch_decompress takes the mean over the senders of each
-    coefficient, src/tplr/compress.py:472-474).  Returns the (T,) factors 1 / (norm + eps)."""
+    every tensor divided by its L2 norm (+ eps).  tplr.compress itself has no such mode (batch_decompress
+    takes the mean over the senders of each coefficient, src/tplr/compress.py:472-474).
+    The transform is orthonormal, so a tensor's norm is that of its summed coefficients: one launch over the
+    payloads alone gives the per-chunk sums of squares, a small one the per-tensor factors, and the aggregate
+    in sum mode with those factors writes the normalised mean directly - the dense tensors are written once
+    and never read.  two_pass=True is the literal order instead (aggregate with the factor 1/P, norms from
+    the per-chunk sums of squares of the result, one scaling pass over the dense tensors).
+    Returns the (T,) factors 1 / (norm + eps)."""
     lib = _lib.load()
     P, T, n, dev = len(vals), len(out), out.total_chunks, out.device
-    scale = torch.full((T, P), 1.0 / P, dtype=torch.float32, device=dev)
     ss = torch.empty(n, dtype=torch.float32, device=dev)
-    batch_decompress_decode_batch(out, idxs, vals, k, scale=scale, use_dct=use_dct, mean=False, sumsq=ss)
     factor = torch.empty(T, dtype=torch.float32, device=dev)
+    if two_pass:
+        scale = torch.full((T, P), 1.0 / P, dtype=torch.float32, device=dev)
+        batch_decompress_decode_batch(out, idxs, vals, k, scale=scale, use_dct=use_dct, mean=False, sumsq=ss)
+        with _on(dev):
+            _lib.check(lib.tplr_tensor_rnorm(_ptr(ss), _ptr(out.table), T, C.c_float(eps), _ptr(factor), _stream(dev)),
+                       "tplr_tensor_rnorm")
+            _lib.check(lib.tplr_scale_batch(_ptr(out.table), T, n, _ptr(factor), _stream(dev)), "tplr_scale_batch")
+        return factor
+    if P > _lib.TPLR_MAX_PEERS:
+        raise NotImplementedError(f"{P} peers: the HIP aggregate kernel takes up to {_lib.TPLR_MAX_PEERS}")
+    for i, v in zip(idxs, vals):
+        if i.dtype != torch.uint8:
+            raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
+        if v.dtype != torch.float32 or v.numel() != n * k or i.numel() * 2 != n * k * 3 or not v.is_contiguous():
+            raise RuntimeError(f"flat payload mismatch: {i.numel()} index bytes / {v.numel()} values for {n} chunks, k={k}")
+    scale = torch.empty((T, P), dtype=torch.float32, device=dev)
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+    vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
     with _on(dev):
-        _lib.check(lib.tplr_tensor_rnorm(_ptr(ss), _ptr(out.table), T, C.c_float(eps), _ptr(factor), _stream(dev)),
-                   "tplr_tensor_rnorm")
-        _lib.check(lib.tplr_scale_batch(_ptr(out.table), T, n, _ptr(factor), _stream(dev)), "tplr_scale_batch")
+        _lib.check(lib.tplr_aggregate_sumsq_batch(ip, vp, None, P, k, _ptr(out.table), T, n, _ptr(ss), _stream(dev)),
+                   "tplr_aggregate_sumsq_batch")
+        _lib.check(lib.tplr_tensor_rnorm_scales(_ptr(ss), _ptr(out.table), T, P, C.c_float(1.0 / P), C.c_float(eps),
+                                                _ptr(factor), _ptr(scale), _stream(dev)), "tplr_tensor_rnorm_scales")
+    batch_decompress_decode_batch(out, idxs, vals, k, scale=scale, use_dct=use_dct, mean=False)
     return factor
 
 

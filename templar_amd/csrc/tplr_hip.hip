@@ -2126,6 +2126,163 @@ __global__ __launch_bounds__(64) void k_scale_chunks(const tplr_tensor_desc* __r
     }
 }
 
+// Per-chunk sum of squares of the peers' summed coefficients, from the payloads alone: nothing is transformed
+// and no dense element is written.  The transform is orthonormal, so a tensor's L2 norm after the inverse
+// transform is the norm of its summed coefficients, and a per-tensor normalisation can be folded into the
+// factors of the one aggregate launch that follows instead of taking a pass of its own over the dense tensors.
+// A unit is one peer's entries 64 m .. 64 m + 63 of the chunk (one wave instruction); units are taken kUnits
+// at a time, the next round's payload requested before this round is scattered.  Sums are plain
+// read-add-write through the claiming exchange (see tile_claim): entries of one instruction that name the
+// same coefficient send the chunk through floating-point atomics instead.  The tile is read back and cleared
+// 16 bytes per lane at a time, every lane adding its squares in a fixed order.
+// kOneRound: k <= 64 and at most kUnits peers - unit i is peer i, one round per chunk, no unit arithmetic.
+template <int kUnits, bool kOneRound>
+__global__ __launch_bounds__(64) void k_aggregate_sumsq(const PeerPtrs pp, const float* __restrict__ scale, int P,
+                                                        int k, const tplr_tensor_desc* __restrict__ table,
+                                                        int n_tensors, int64_t total, float* __restrict__ sumsq) {
+    __shared__ __align__(16) float tile[kChunk * kChunk];
+    const int lane = threadIdx.x;
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
+    const int64_t idx_stride = k + (k >> 1);
+    const int M = kOneRound ? 1 : (k + 63) >> 6;               // wave instructions per peer and chunk
+    const int U = P * M;                                       // units per chunk
+    const int nb = kOneRound ? 1 : (U + kUnits - 1) / kUnits;  // rounds per chunk
+    float4* const tile4 = reinterpret_cast<float4*>(tile);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) tile4[q * 64 + lane] = make_float4(0.f, 0.f, 0.f, 0.f);
+    wave_lds_fence();
+
+    uint32_t ix[2][kUnits];
+    float a[2][kUnits];
+    int t_of[2] = {0, 0};
+    Cursor c;
+    tplr_tensor_desc none = {};
+    cursor_seek(c, table, none, n_tensors, g0);
+    int64_t lg = g0;  // the round requested next: chunk and round number
+    int lr = 0;
+    auto unit_peer = [&](int u, int& m) -> int {  // wave-uniform
+        if constexpr (kOneRound) {
+            m = 0;
+            return u;
+        }
+        const int p = u / M;
+        m = u - p * M;
+        return p;
+    };
+    auto request = [&](auto sel) {
+        constexpr int s = decltype(sel)::value;
+        if (lg >= g1) return;
+        t_of[s] = c.t;
+#pragma unroll
+        for (int i = 0; i < kUnits; ++i) {
+            const int u = kOneRound ? i : lr * kUnits + i;
+            if (u < U) {  // wave-uniform
+                int m;
+                const int p = unit_peer(u, m);
+                const int j = m * 64 + lane;
+                const int je = j < k ? j : 0;
+                const gbyte* irow = (const gbyte*)pp.idx[p] + lg * idx_stride;
+                ix[s][i] = *(const gu16*)(irow + (3 * (je >> 1) + (je & 1)));
+                a[s][i] = ((const gfloat*)pp.val[p] + lg * k)[je];
+            }
+        }
+        if (++lr == nb) {
+            lr = 0;
+            if (++lg < g1) cursor_next(c, lg);
+        }
+    };
+
+    auto read_back = [&]() -> float {  // sum of squares of the tile, which it leaves cleared
+        wave_lds_fence();
+        float ss = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            const float4 t = tile4[q * 64 + lane];
+            ss = __builtin_fmaf(t.w, t.w, __builtin_fmaf(t.z, t.z, __builtin_fmaf(t.y, t.y, __builtin_fmaf(t.x, t.x, ss))));
+            tile4[q * 64 + lane] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        wave_lds_fence();
+        return wave_sum_f32(ss);
+    };
+
+    int64_t pg = g0;  // the round scattered next
+    int pr = 0;
+    uint32_t repeat = 0;
+    auto scatter = [&](auto sel) {
+        constexpr int s = decltype(sel)::value;
+        const int t = t_of[s];
+#pragma unroll
+        for (int i = 0; i < kUnits; ++i) {
+            const int u = kOneRound ? i : pr * kUnits + i;
+            if (u < U) {  // wave-uniform
+                int m;
+                const int p = unit_peer(u, m);
+                const int j = m * 64 + lane;
+                const float sc = scale ? scale[static_cast<int64_t>(t) * P + p] : 1.0f;
+                if (j < k) {
+                    const uint32_t e = (j & 1) ? (ix[s][i] >> 4) : (ix[s][i] & 0xfffu);
+                    const float cur = tile_claim(&tile[e]);
+                    repeat = seen_mark(repeat, cur);
+                    tile[e] = cur + a[s][i] * sc;
+                }
+            }
+        }
+        if (++pr < nb) return;
+        // the chunk is complete
+        float ss = read_back();
+        if (__ballot(repeat == kClaimMark) != 0) {  // wave-uniform, false for top-k payloads
+            for (int p = 0; p < P; ++p) {
+                const float sc = scale ? scale[static_cast<int64_t>(t) * P + p] : 1.0f;
+                const gbyte* irow = (const gbyte*)pp.idx[p] + pg * idx_stride;
+                const gfloat* vrow = (const gfloat*)pp.val[p] + pg * k;
+                for (int j = lane; j < k; j += 64) {
+                    const uint32_t w = *(const gu16*)(irow + (3 * (j >> 1) + (j & 1)));
+                    atomicAdd(&tile[(j & 1) ? (w >> 4) : (w & 0xfffu)], vrow[j] * sc);
+                }
+            }
+            ss = read_back();
+            repeat = 0;
+        }
+        if (lane == 0) sumsq[pg] = ss;
+        pr = 0;
+        ++pg;
+    };
+
+    request(std::integral_constant<int, 0>{});
+    while (pg < g1) {
+        request(std::integral_constant<int, 1>{});
+        scatter(std::integral_constant<int, 0>{});
+        if (pg >= g1) break;
+        request(std::integral_constant<int, 0>{});
+        scatter(std::integral_constant<int, 1>{});
+    }
+}
+
+// From those sums: tensor t's factor 1 / (sqrt(sum of its entries) * pre + eps), and pre times that factor
+// as the P aggregate factors of the tensor (pre = 1 / P makes the aggregate the normalised mean over P peers).
+__global__ __launch_bounds__(256) void k_tensor_rnorm_scales(const float* __restrict__ sumsq,
+                                                             const tplr_tensor_desc* __restrict__ table, float eps,
+                                                             float pre, int P, float* __restrict__ factor,
+                                                             float* __restrict__ scale) {
+    __shared__ double part[4];
+    __shared__ float f_all;
+    const tplr_tensor_desc d = table[blockIdx.x];
+    const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
+    const float* s = sumsq + d.chunk_begin;
+    double acc = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += 256) acc += static_cast<double>(s[i]);
+    acc = block256_sum_f64(acc, part, threadIdx.x);
+    if (threadIdx.x == 0) {
+        const float f = 1.0f / (static_cast<float>(sqrt(acc)) * pre + eps);
+        if (factor) factor[blockIdx.x] = f;
+        f_all = f * pre;
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < P; p += 256) scale[static_cast<int64_t>(blockIdx.x) * P + p] = f_all;
+}
+
 // Plain streaming copy (16 bytes per lane per step, grid-stride).  It exists so that hardware
 // traffic counters can be calibrated: it moves exactly n16 * 16 bytes each way.
 __global__ __launch_bounds__(256) void k_calib_copy(const v4f* __restrict__ src, v4f* __restrict__ dst, int64_t n16) {
@@ -2989,6 +3146,42 @@ int tplr_scale_batch(const tplr_tensor_desc* d_desc, int n_tensors, int64_t tota
     const int64_t need = ((total_chunks + 7) / 8) * 8;
     hipLaunchKernelGGL(k_scale_chunks, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
                        static_cast<hipStream_t>(stream), d_desc, n_tensors, total_chunks, d_factor);
+    return launch_status();
+}
+
+int tplr_aggregate_sumsq_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale,
+                               int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
+                               int64_t total_chunks, float* d_sumsq, void* stream) {
+    if (int s = check_decode(h_idx12, h_val, n_peers, k, TPLR_REDUCE_SUM)) return s;
+    if (!d_desc || !d_sumsq || n_tensors < 1 || total_chunks < 0) return TPLR_E_BADARG;
+    if (total_chunks == 0) return 0;
+    PeerPtrs pp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        pp.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
+        pp.val[p] = p < n_peers ? h_val[p] : nullptr;
+        if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
+    }
+    static int resident = 0;  // (the instantiations differ in registers, not in LDS, which bounds them)
+    if (resident == 0) resident = persistent_grid(k_aggregate_sumsq<16, true>, int64_t{1} << 40);
+    const int64_t need = ((total_chunks + 7) / 8) * 8;
+    const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
+    if (k <= 64 && n_peers <= 16)
+        hipLaunchKernelGGL((k_aggregate_sumsq<16, true>), grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale,
+                           n_peers, k, d_desc, n_tensors, total_chunks, d_sumsq);
+    else if (k <= 64 && n_peers <= 32)
+        hipLaunchKernelGGL((k_aggregate_sumsq<32, true>), grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale,
+                           n_peers, k, d_desc, n_tensors, total_chunks, d_sumsq);
+    else
+        hipLaunchKernelGGL((k_aggregate_sumsq<16, false>), grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale,
+                           n_peers, k, d_desc, n_tensors, total_chunks, d_sumsq);
+    return launch_status();
+}
+
+int tplr_tensor_rnorm_scales(const float* d_sumsq, const tplr_tensor_desc* d_desc, int n_tensors, int n_peers,
+                             float pre, float eps, float* d_factor, float* d_scale, void* stream) {
+    if (!d_sumsq || !d_desc || !d_scale || n_tensors < 1 || n_peers < 1) return TPLR_E_BADARG;
+    hipLaunchKernelGGL(k_tensor_rnorm_scales, dim3(static_cast<unsigned>(n_tensors)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), d_sumsq, d_desc, eps, pre, n_peers, d_factor, d_scale);
     return launch_status();
 }
 

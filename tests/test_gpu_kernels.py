@@ -1084,10 +1084,55 @@ def test_whole_set_calls_replay_from_a_captured_graph(dev):
         assert all(torch.equal(a, b) for a, b in zip(outs, want[2]))
 
 
+@pytest.mark.parametrize("P,k,repeats", [(15, 32, False), (1, 2, False), (20, 64, False), (3, 128, False), (40, 20, False),
+                                          (15, 32, True), (5, 128, True)])
+def test_sums_of_squares_of_the_summed_coefficients_from_the_payloads(dev, P, k, repeats):
+    # tplr_aggregate_sumsq_batch against the oracle's dense scatter-sum, chunk by chunk: one and several rounds of
+    # units, rows longer than a wave, clip factors, and repeated indices inside a row (atomic path)
+    shapes = [(128, 192), (64, 64), (192, 64)]
+    counts = [(a // 64) * (b // 64) for a, b in shapes]
+    n = sum(counts)
+    idxs, vals = make_peers(P, 1, n, k, 4000 + 10 * P + k)
+    rng = np.random.default_rng(17 * P + k)
+    if repeats:
+        for p in range(P):
+            ii = orc.unpack12(idxs[p], (n, k)).reshape(n, k).copy()
+            for r in range(0, n, 2):
+                ii[r, 1 + (p % (k - 1))] = ii[r, 0]          # a repeat inside one wave instruction
+                if k > 64:
+                    ii[r, 70] = ii[r, 3]                       # and one across two of them
+            idxs[p] = orc.pack12(ii)
+    batch = tc.TensorBatch([torch.empty(s, device=dev) for s in shapes])
+    di = [torch.from_numpy(i).to(dev) for i in idxs]
+    dv = [torch.from_numpy(v.reshape(n, k)).to(dev) for v in vals]
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in di])
+    vp = (C.c_void_p * P)(*[v.data_ptr() for v in dv])
+    for scaled in (False, True):
+        scale = rng.uniform(0.2, 1.0, size=(len(shapes), P)).astype(np.float32) if scaled else None
+        dscale = torch.from_numpy(scale).to(dev) if scaled else None
+        ss = torch.full((n,), -1.0, device=dev)
+        st = _lib.load().tplr_aggregate_sumsq_batch(ip, vp, dscale.data_ptr() if scaled else None, P, k,
+                                                    batch.table.data_ptr(), len(shapes), n, ss.data_ptr(), None)
+        assert st == 0
+        torch.cuda.synchronize()
+        got = ss.cpu().numpy()
+        b0 = 0
+        for t, cnt in enumerate(counts):
+            ti = [orc.pack12(orc.unpack12(i, (n, k)).reshape(n, k)[b0:b0 + cnt]) for i in idxs]
+            tv = [(v.reshape(n, k)[b0:b0 + cnt] * (scale[t, p] if scaled else np.float32(1))).reshape(1, cnt, k)
+                  for p, v in enumerate(vals)]
+            dense = orc.batch_decompress(ti, tv, (1, cnt, 64, 64), 4096, clip_norm=False, mean=False).astype(np.float64)
+            want = (dense.reshape(cnt, 4096) ** 2).sum(axis=1)
+            assert np.abs(got[b0:b0 + cnt] - want).max() <= 1e-5 * want.max(), (t, scaled)
+            b0 += cnt
+
+
+@pytest.mark.parametrize("two_pass", [False, True])
 @pytest.mark.parametrize("use_dct", [True, False])
-def test_aggregate_mean_over_peers_then_normalised_per_tensor(dev, use_dct):
+def test_aggregate_mean_over_peers_then_normalised_per_tensor(dev, use_dct, two_pass):
     # the benchmark's wording of the aggregation workload: scatter-sum, inverse transform, divide by the number
-    # of peers, divide every tensor by its L2 norm - against the oracle, tensor by tensor
+    # of peers, divide every tensor by its L2 norm - against the oracle, tensor by tensor; the norm taken from
+    # the payloads before the one aggregate launch (the default) and from the dense result (two_pass)
     P, k = 15, 32
     shapes = [(128, 192), (64, 64), (256, 128)]
     counts = [(a // 64) * (b // 64) for a, b in shapes]
@@ -1097,7 +1142,7 @@ def test_aggregate_mean_over_peers_then_normalised_per_tensor(dev, use_dct):
     batch = tc.TensorBatch(outs)
     di = [torch.from_numpy(i).to(dev) for i in idxs]
     dv = [torch.from_numpy(v.reshape(n, k)).to(dev) for v in vals]
-    factor = tc.aggregate_mean_normalised_batch(batch, di, dv, k, use_dct=use_dct)
+    factor = tc.aggregate_mean_normalised_batch(batch, di, dv, k, use_dct=use_dct, two_pass=two_pass)
     b0 = 0
     for t, (shape, cnt) in enumerate(zip(shapes, counts)):
         Y, X = shape[0] // 64, shape[1] // 64
