@@ -117,7 +117,8 @@ int tplr_dct2d_dense(const float* d_in, int64_t R, int64_t C, int h, int w,
 /* ---- top-k select + value gather + 12-bit pack -----------------------------------
  * Replaces TopKCompressor.compress without quantisation (src/tplr/compress.py:402-416)
  * on n_rows rows of row_len fp32 coefficients (row_len = 4096 for 2-D chunks, 64 for
- * 1-D tensors, anything <= TPLR_MAX_ROW otherwise).  k even, 2 <= k <= min(row_len, 128).
+ * 1-D tensors, anything <= TPLR_MAX_ROW otherwise).  k even, 2 <= k <= row_len (k > 128 sorts the
+ * whole row in LDS: exact, an order of magnitude slower than the select that serves k <= 128).
  * Outputs: d_idx12 = n_rows * k * 3/2 bytes, d_val = (n_rows, k) signed values.
  * This is the coefficient-input entry used for the bit-exact parity stage. */
 int tplr_topk_pack(const float* d_coef, int64_t n_rows, int64_t row_len, int k,

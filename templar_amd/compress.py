@@ -419,11 +419,8 @@ def _row_layout(xshape: tuple) -> tuple[int, int]:
 def _topk_rows(rows: torch.Tensor, k: int):
     """rows (n_rows, n) fp32 contiguous on device -> (packed idx uint8, val (n_rows, k))."""
     n_rows, n = rows.shape
-    if n > _lib.TPLR_MAX_ROW or k > _lib.TPLR_MAX_K:
-        raise NotImplementedError(
-            f"top-{k} of rows of {n}: the HIP select kernel handles rows up to {_lib.TPLR_MAX_ROW} and "
-            f"k up to {_lib.TPLR_MAX_K}"
-        )
+    if n > _lib.TPLR_MAX_ROW:  # (the 12-bit index ends there as well)
+        raise NotImplementedError(f"top-{k} of rows of {n}: the HIP select kernel handles rows up to {_lib.TPLR_MAX_ROW}")
     lib = _lib.load()
     idx = torch.empty(n_rows * (k // 2) * 3, dtype=torch.uint8, device=rows.device)
     val = torch.empty((n_rows, k), dtype=torch.float32, device=rows.device)
@@ -435,10 +432,21 @@ def _topk_rows(rows: torch.Tensor, k: int):
 
 
 def _encode_topk(x2d: torch.Tensor, R: int, Cc: int, ld: int, k: int, use_dct: bool):
-    if k > _lib.TPLR_MAX_K:
-        raise NotImplementedError(f"top-{k}: the HIP select kernel handles k up to {_lib.TPLR_MAX_K}")
     lib = _lib.load()
     n_chunks = (R // _CH) * (Cc // _CH)
+    if k > _lib.TPLR_MAX_K and n_chunks:
+        # more entries than the fused kernel's select holds: the chunked (transformed) tensor is written out
+        # and every chunk sorted whole - exact, far slower; no setting of templar's comes here
+        coef = torch.empty((n_chunks, _CH * _CH), dtype=torch.float32, device=x2d.device)
+        with _on(x2d.device):
+            if use_dct:
+                st = lib.tplr_dct2d_fwd(_ptr(x2d), R, Cc, ld, _ptr(coef), _stream(x2d.device))
+                _lib.check(st, "tplr_dct2d_fwd")
+            else:
+                coef.view(R // _CH, Cc // _CH, _CH, _CH).copy_(
+                    torch.as_strided(x2d, (R // _CH, Cc // _CH, _CH, _CH), (ld * _CH, _CH, ld, 1)))
+        idx, val = _topk_rows(coef, k)
+        return idx, val.view(R // _CH, Cc // _CH, k)
     idx = torch.empty(n_chunks * (k // 2) * 3, dtype=torch.uint8, device=x2d.device)
     val = torch.empty((R // _CH, Cc // _CH, k), dtype=torch.float32, device=x2d.device)
     if n_chunks:
@@ -604,7 +612,7 @@ class TopKCompressor:
         topk = _clamp_k(totalk, topk)
 
         view = _as_chunk_view(x)
-        if view is not None and topk <= _lib.TPLR_MAX_K:
+        if view is not None:
             R, Cc, ld = view  # the un-transformed chunk view of a dense tensor: select straight from it
             idx, val = _encode_topk(x, R, Cc, ld, topk, use_dct=False)
         else:
@@ -948,13 +956,18 @@ def encode_compress_batch(batch: TensorBatch, topk: int, *, use_dct: bool = True
     src/tplr/neurons.py:114-159).  Returns the flat payload (idx12 uint8, val (total_chunks, k))."""
     lib = _lib.load()
     k = _clamp_k(_CH * _CH, topk)
-    if k > _lib.TPLR_MAX_K:
-        raise NotImplementedError(f"top-{k}: the HIP select kernel handles k up to {_lib.TPLR_MAX_K}")
     n = batch.total_chunks
     if idx12 is None:
         idx12 = torch.empty(n * (k // 2) * 3, dtype=torch.uint8, device=batch.device)
     if val is None:
         val = torch.empty((n, k), dtype=torch.float32, device=batch.device)
+    if k > _lib.TPLR_MAX_K:  # tensor by tensor through the whole-row sort
+        for i, t in enumerate(batch.tensors):
+            ti, tv = _encode_topk(t, t.shape[0], t.shape[1], t.stride(0), k, use_dct)
+            si, sv = batch.payload_slice(i, idx12, val, k)
+            si.copy_(ti.reshape(si.shape))
+            sv.copy_(tv.reshape(sv.shape))
+        return idx12, val
     with _on(batch.device):
         st = lib.tplr_encode_topk_pack_batch(_ptr(batch.table), len(batch), n, k, int(use_dct), _ptr(idx12), _ptr(val),
                                              _stream(batch.device))

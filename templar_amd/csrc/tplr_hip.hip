@@ -413,6 +413,56 @@ __global__ __launch_bounds__(64) void k_topk_rows(const float* __restrict__ coef
     emit_selected<kTwo>(s, lane, k, row, idx12, val);
 }
 
+// Any k up to the row length: the whole row sorted.  One workgroup of 256 threads per row, the row as
+// 4096 keys (magnitude, 4095 - index, sign: the canonical order of select_topk, elements past the row
+// as zeros at their own indices, which no real element ranks below) in LDS, a bitonic network of 78
+// steps in descending order, then the k leading keys unpacked as select_topk unpacks its candidates.
+// Not a fast path: it serves selections larger than the register-resident select holds (k > 128).
+__global__ __launch_bounds__(256) void k_topk_rows_sorted(const float* __restrict__ coef, int64_t n_rows, int row_len,
+                                                          int k, uint8_t* __restrict__ idx12, float* __restrict__ val) {
+    __shared__ uint64_t keys[4096];
+    const int tid = threadIdx.x;
+    const int64_t row = xcd_contiguous(blockIdx.x, gridDim.x);
+    if (row >= n_rows) return;  // (the whole workgroup)
+    const float* src = coef + row * row_len;
+    for (int e = tid; e < 4096; e += 256) {
+        const uint32_t bits = e < row_len ? __float_as_uint(src[e]) : 0u;
+        keys[e] = (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - static_cast<uint32_t>(e)) << 1) | (bits >> 31);
+    }
+    __syncthreads();
+    for (int size = 2; size <= 4096; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            for (int i = tid; i < 2048; i += 256) {
+                const int pos = 2 * i - (i & (stride - 1));
+                const uint64_t a = keys[pos], b = keys[pos + stride];
+                const bool down = (pos & size) == 0;  // this run is sorted in descending order
+                if ((a < b) == down) {
+                    keys[pos] = b;
+                    keys[pos + stride] = a;
+                }
+            }
+            __syncthreads();
+        }
+    }
+    float* vrow = val + row * k;
+    uint8_t* irow = idx12 + row * (k + (k >> 1));
+    for (int j = tid; j < (k >> 1); j += 256) {
+        uint32_t ix[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint64_t e = keys[2 * j + h];
+            const uint32_t lo = static_cast<uint32_t>(e), key = static_cast<uint32_t>(e >> 32);
+            ix[h] = 4095u - ((lo >> 1) & 4095u);
+            const uint32_t mag = key == 0x7fffffffu ? 0x7fc00000u : key;
+            vrow[2 * j + h] = __uint_as_float(mag | (lo << 31));
+        }
+        const uint32_t w = ix[0] | (ix[1] << 12);
+        irow[3 * j] = static_cast<uint8_t>(w);
+        irow[3 * j + 1] = static_cast<uint8_t>(w >> 8);
+        irow[3 * j + 2] = static_cast<uint8_t>(w >> 16);
+    }
+}
+
 // The 1-D parameters of a set (norm vectors), every tensor a run of rows of 64 elements: transform,
 // top-k and pack of all of them in one launch, each tensor read where it lies.  One wave takes up to 64
 // rows of one tensor: staged through the tile, a row per lane in registers, the 64-point transform and
@@ -2585,12 +2635,15 @@ int tplr_dct2d_dense(const float* d_in, int64_t R, int64_t C, int h, int w, cons
 
 int tplr_topk_pack(const float* d_coef, int64_t n_rows, int64_t row_len, int k, uint8_t* d_idx12,
                    float* d_val, void* stream) {
-    if (n_rows < 0 || row_len < 1 || k < 2 || (k & 1) || k > row_len || k > kCandCap) return TPLR_E_BADARG;
+    if (n_rows < 0 || row_len < 1 || k < 2 || (k & 1) || k > row_len) return TPLR_E_BADARG;
     if (row_len > TPLR_MAX_ROW) return TPLR_E_TOOMANY;
     if (n_rows == 0) return 0;
     if (!d_coef || !d_idx12 || !d_val) return TPLR_E_BADARG;
     const int rl = static_cast<int>(row_len);
-    if (k > 32)
+    if (k > kCandCap)
+        hipLaunchKernelGGL(k_topk_rows_sorted, dim3(grid8(n_rows)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           d_coef, n_rows, rl, k, d_idx12, d_val);
+    else if (k > 32)
         hipLaunchKernelGGL(k_topk_rows<true>, dim3(grid8(n_rows)), dim3(64), 0,
                            static_cast<hipStream_t>(stream), d_coef, n_rows, rl, k, d_idx12, d_val);
     else

@@ -173,7 +173,7 @@ def test_topk_fixture_bit_exact(dev):
     assert np.array_equal(val.cpu().numpy().reshape(z["val"].shape), z["val"])
 
 
-@pytest.mark.parametrize("k", [2, 16, 32, 34, 64, 100, 128])
+@pytest.mark.parametrize("k", [2, 16, 32, 34, 64, 100, 128, 130, 256, 1000, 4096])
 def test_topk_chunks_bit_exact(dev, k):
     rows = t3((48, 4096), 1000 + k).numpy()
     check_topk(rows, k, dev)
@@ -227,7 +227,7 @@ def test_topk_special_values(dev):
     rows[4, ::2] = 1.0
     rows[4, 1::2] = -1.0
     rows[5] = np.linspace(-1, 1, 4096, dtype=np.float32)
-    for k in (2, 32, 64):
+    for k in (2, 32, 64, 200, 4096):
         rows_d = torch.from_numpy(rows).to(dev)
         idx12, val = tc._topk_rows(rows_d, k)
         want_i, want_v = orc.topk_rows(rows, k)
@@ -236,7 +236,8 @@ def test_topk_special_values(dev):
         assert np.array_equal(val.cpu().numpy().view(np.uint32), want_v.view(np.uint32))
 
 
-@pytest.mark.parametrize("n,k", [(64, 32), (64, 64), (100, 10), (37, 6), (4095, 32), (2048, 128), (2, 2)])
+@pytest.mark.parametrize("n,k", [(64, 32), (64, 64), (100, 10), (37, 6), (4095, 32), (2048, 128), (2, 2), (2048, 512),
+                                 (300, 300), (4095, 4094)])
 def test_topk_generic_rows(dev, n, k):
     rows = t3((9, n), n * 7 + k).numpy()
     rows[3] = 0.0
@@ -257,6 +258,30 @@ def test_fused_encode_equals_unfused(dev, shape, k):
     want_i, want_v = orc.topk_rows(coef.cpu().numpy().reshape(-1, 4096), k)
     assert np.array_equal(idx_f.cpu().numpy(), orc.pack12(want_i))
     assert np.array_equal(val_f.cpu().numpy().reshape(-1, k), want_v)
+
+
+@pytest.mark.parametrize("use_dct", [True, False])
+def test_selections_larger_than_the_fused_select_holds(dev, use_dct):
+    # k > 128: the chunked (transformed) tensor is written out and every chunk sorted whole.  Same canonical
+    # payload as the oracle's selection on the device's coefficients, through the per-tensor and the whole-set
+    # entry points; with every coefficient kept (k = 4096) decode(decompress(...)) gives the tensor back
+    shapes = [(128, 192), (64, 64)]
+    xs = [t3(s, 400 + i, row_scale=True).to(dev) for i, s in enumerate(shapes)]
+    tr = tc.ChunkingTransformer(_Stub(xs), 64)
+    for k in (130, 512, 4096):
+        batch = tc.TensorBatch(xs)
+        bi, bv = tc.encode_compress_batch(batch, k, use_dct=use_dct)
+        for i, x in enumerate(xs):
+            idx, val, xshape, totalk = tc.encode_compress(x, k, use_dct=use_dct)
+            coef = tr.encode(x, use_dct=use_dct)
+            want_i, want_v = orc.topk_rows(coef.cpu().numpy().reshape(-1, 4096), k)
+            assert np.array_equal(idx.cpu().numpy(), orc.pack12(want_i)), (k, i)
+            assert np.array_equal(val.cpu().numpy().reshape(-1, k).view(np.uint32), want_v.view(np.uint32)), (k, i)
+            si, sv = batch.payload_slice(i, bi, bv, k)
+            assert torch.equal(si, idx) and torch.equal(sv.reshape(val.shape), val)
+            if k == 4096:
+                back = tc.batch_decompress_decode([idx], [val], xshape, clip_norm=False, use_dct=use_dct)
+                assert relerr(back.cpu().numpy(), x.cpu().numpy()) <= TOL
 
 
 def near_tie_audit(x_np, idx12, val, k, tol=TOL):
