@@ -423,6 +423,18 @@ def main():
     aggn_ms, _ = event_ms(lambda: tc.aggregate_mean_normalised_batch(out_batch, idxs, vals, k), agg_steps, 1)
     aggn2_ms, _ = event_ms(lambda: tc.aggregate_mean_normalised_batch(out_batch, idxs, vals, k, two_pass=True),
                            agg_steps, 1)
+    # the aggregate together with what outer_step looks at next per parameter (L2 norm, mean, all-finite):
+    # from two floats per chunk left by the same launch, against the three torch reductions per dense tensor
+    aggs_ms, _ = event_ms(lambda: tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, scale=scale, use_dct=DCT,
+                                                                   stats=True), agg_steps, 1)
+
+    def stats_by_torch():
+        for o in outs:
+            torch.linalg.vector_norm(o)
+            o.mean()
+            torch.isfinite(o).all()
+
+    stats_torch_ms, _ = event_ms(stats_by_torch, 3, 1)
     agg_pt_ms, _ = event_ms(aggregate_per_tensor, 3, 1)
     agg_rc_ms, _ = event_ms(aggregate_reference_calls, 3, 1)
     # the same per-parameter loop recorded once into a HIP graph and replayed: what is left is device time
@@ -493,6 +505,12 @@ def main():
                                               "of the dense result, one scaling pass); aggregate_ms is the "
                                               "reference's batch_decompress semantics",
         "aggregate_sum_mean_normalised_two_pass_ms": round(aggn2_ms, 4),
+        "aggregate_with_result_stats": {"kernel_with_stats_ms": round(aggs_ms, 4), "kernel_ms": round(aggk_ms, 4),
+                                        "same_stats_by_torch_ms": round(stats_torch_ms, 4),
+                                        "what": "per-parameter L2 norm, mean and all-finite flag of the decoded "
+                                                "gradients from two floats per chunk left by the aggregate launch "
+                                                "(+ one small launch), against norm, mean and isfinite().all() of "
+                                                "every dense tensor by torch afterwards"},
         "ms_per_step_spread": {"median": enc_spread[0], "min": enc_spread[1], "max": enc_spread[2],
                                "what": "per-call durations of a further `steps` calls of the step, each between its own events"},
         "per_tensor_launches": {"encode_ms": round(enc_pt_ms, 4), "aggregate_ms": round(agg_pt_ms, 4),

@@ -304,6 +304,21 @@ int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_des
                         float range_in_sigmas, int n_slices, double* d_work, uint8_t* d_codes, float* d_shift,
                         float* d_scale, float* d_lookup, void* stream);
 
+/* tplr_decode_aggregate_batch together with what its caller looks at next, per parameter
+ * (src/tplr/neurons.py:380-385: L2 norm and mean of the decoded gradient for the fingerprint; :411 and
+ * :438: the parameter is skipped unless every element is finite), without another pass over the dense
+ * tensors: the aggregate leaves two floats per chunk in d_chunk_stats (2 * total_chunks floats: sum of
+ * squares and sum of the chunk's 4096 results) and one small launch turns them into
+ * d_tensor_stats[4 t .. 4 t + 3] = {L2 norm, mean, 1.0 if every element is finite else 0.0, sum of squares}.
+ * The flag is exact: a chunk whose figures are not finite is read back and examined element by element
+ * (and, when its elements are all finite, summed again in double).  Norm and mean are sums in another
+ * order than torch's: equal within fp32 rounding of the accumulation (1e-6 relative), non-finite when
+ * the flag is 0.  Other arguments as tplr_decode_aggregate_batch. */
+int tplr_decode_aggregate_stats_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale,
+                                      int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
+                                      int64_t total_chunks, int reduce_mode, int normalise, int use_dct,
+                                      float* d_chunk_stats, float* d_tensor_stats, void* stream);
+
 /* ---- per-tensor L2 normalisation of an aggregate ----------------------------------------------
  * The reference has no such step inside tplr.compress; the benchmark's aggregation workload words it
  * ("scatter-summed, inverse DCT, mean over peers, then L2-normalised per tensor"), and the per-chunk

@@ -1001,9 +1001,14 @@ def peer_clip_scales_batch(batch: TensorBatch, vals: Sequence[torch.Tensor], k: 
 @torch.no_grad()
 def batch_decompress_decode_batch(out: TensorBatch, idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], k: int,
                                   *, clip_norm: bool = True, scale: torch.Tensor | None = None, normalise: bool = False,
-                                  use_dct: bool = True, mean: bool = True, sumsq: torch.Tensor | None = None) -> None:
+                                  use_dct: bool = True, mean: bool = True, sumsq: torch.Tensor | None = None,
+                                  stats: bool = False) -> "torch.Tensor | None":
     """batch_decompress + decode of every parameter in one launch (src/tplr/neurons.py:309-367):
-    peer p's flat payload is (idxs[p], vals[p]); results are written into the tensors of `out`."""
+    peer p's flat payload is (idxs[p], vals[p]); results are written into the tensors of `out`.
+    stats=True also returns a (T, 4) tensor {L2 norm, mean, all-finite flag (1.0 / 0.0), sum of squares}
+    of every decoded parameter - what outer_step computes next with three more passes over each dense
+    gradient (fingerprint norm and mean :380-385, the isfinite test :411/:438) - from two floats per chunk that
+    the aggregate kernel leaves on its way."""
     lib = _lib.load()
     P = len(vals)
     if P > _lib.TPLR_MAX_PEERS:
@@ -1018,11 +1023,23 @@ def batch_decompress_decode_batch(out: TensorBatch, idxs: Sequence[torch.Tensor]
         scale = peer_clip_scales_batch(out, vals, k)
     ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
     vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
+    if stats:
+        if sumsq is not None:
+            raise ValueError("stats=True keeps its own per-chunk figures: pass either `sumsq` or `stats`")
+        per_chunk = torch.empty((max(n, 1), 2), dtype=torch.float32, device=out.device)
+        per_tensor = torch.empty((len(out), 4), dtype=torch.float32, device=out.device)
+        with _on(out.device):
+            st = lib.tplr_decode_aggregate_stats_batch(ip, vp, _ptr(scale), P, k, _ptr(out.table), len(out), n,
+                                                       _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM, int(normalise),
+                                                       int(use_dct), _ptr(per_chunk), _ptr(per_tensor), _stream(out.device))
+        _lib.check(st, "tplr_decode_aggregate_stats_batch")
+        return per_tensor
     with _on(out.device):
         st = lib.tplr_decode_aggregate_batch(ip, vp, _ptr(scale), P, k, _ptr(out.table), len(out), n,
                                              _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM, int(normalise), int(use_dct),
                                              _ptr(sumsq), _stream(out.device))
     _lib.check(st, "tplr_decode_aggregate_batch")
+    return None
 
 
 @torch.no_grad()

@@ -691,9 +691,35 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
                                                             int64_t first, int64_t total, int reduce_mode,
-                                                            int normalise, float* __restrict__ sumsq,
+                                                            int options, float* __restrict__ sumsq,
                                                             int64_t stride_idx, int64_t stride_val) {
     // this launch covers the chunks first .. first + total - 1 of the batch
+    // options: bit 0 = per-peer, per-chunk normalisation (generic instantiation); bit 1 = `sumsq` takes two
+    // floats per chunk, the sum of squares of the result and the sum of its elements
+    const bool normalise = (options & 1) != 0;
+    const bool with_sum = (options & 2) != 0;
+    // per-chunk statistics of the result in registers (v: a column per lane); a chunk that is to be done
+    // again on the exact path writes them there
+    auto chunk_stats = [&](const float (&v)[64], int64_t g, bool skip) {
+        if (!sumsq) return;  // wave-uniform
+        const int lane_ = threadIdx.x;
+        float ss = 0.f;
+#pragma unroll
+        for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
+        ss = wave_sum_f32(ss);
+        if (with_sum) {
+            float sm = 0.f;
+#pragma unroll
+            for (int r = 0; r < 64; ++r) sm += v[r];
+            sm = wave_sum_f32(sm);
+            if (lane_ == 0 && !skip) {
+                sumsq[2 * g] = ss;
+                sumsq[2 * g + 1] = sm;
+            }
+        } else if (lane_ == 0 && !skip) {
+            sumsq[g] = ss;
+        }
+    };
     using Cnt = Counters<kCntBits>;
     // kPark: lanes and units without an entry scatter "coefficient 4096 + lane", which the address
     // arithmetic of real coefficients maps to 64 tile slots and 8 counter words past the chunk's own
@@ -1009,13 +1035,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             for (int r = 0; r < 64; ++r)
                 v[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4, r * ld4, 0)) - v[r];
         }
-        if (sumsq) {
-            float ss = 0.f;
-#pragma unroll
-            for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
-            ss = wave_sum_f32(ss);
-            if (lane == 0) sumsq[g] = ss;
-        }
+        chunk_stats(v, g, false);
         if (rows) {
             store_chunk_rows(v, (void*)dst, ld, lane);
         } else {
@@ -1316,12 +1336,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
 #pragma unroll
                 for (int r = 0; r < 64; ++r) v[r] = before[r] - v[r];
             }
-            float ss = 0.f;
-            if (sumsq) {
-#pragma unroll
-                for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
-                ss = wave_sum_f32(ss);
-            }
+            chunk_stats(v, g, skip0);
             // (the loop-carried destination may have been parked in vector registers: make it
             // scalar again, or every store becomes a loop over distinct descriptors)
             const bool skip1 = g + 1 < g1 && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
@@ -1330,7 +1345,6 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             mean_pass();
             // a chunk that is to be done again is not stored: its descriptor gets a range of zero bytes
             store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane, skip0);
-            if (sumsq && lane == 0 && !skip0) sumsq[g] = ss;
             skip0 = skip1;
             o0 = o1;
             o1 = o2;
@@ -1402,12 +1416,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
         // ---- second half of chunk g, in registers
         if (kUseDct) dct64_inv(v);  // along b: v[k] = sum_b Z[b][lane] F[k][b]
-        float ss = 0.f;
-        if (sumsq) {
-#pragma unroll
-            for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
-            ss = wave_sum_f32(ss);
-        }
+        chunk_stats(v, g, skip_cur);
         const bool skip_next = more && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
         if (skip_next) mark_redo(g + 1);
         repeat = 0;
@@ -1424,7 +1433,6 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 reinterpret_cast<float4*>((float*)dst)[q0 * 64 + lane] =
                     make_float4(v[4 * q0], v[4 * q0 + 1], v[4 * q0 + 2], v[4 * q0 + 3]);
         }
-        if (sumsq && lane == 0 && !skip_cur) sumsq[g] = ss;
         skip_cur = skip_next;
         out_cur = out_next;
         out_next = out_after;
@@ -2333,6 +2341,60 @@ __global__ __launch_bounds__(256) void k_tensor_rnorm_scales(const float* __rest
     for (int p = threadIdx.x; p < P; p += 256) scale[static_cast<int64_t>(blockIdx.x) * P + p] = f_all;
 }
 
+// What the caller of the aggregate looks at next, per tensor (src/tplr/neurons.py:380-385: L2 norm and mean of
+// the decoded gradient; :411 and :438: is every element finite), from the two floats per chunk the aggregate
+// kernel leaves when asked - no further pass over the dense tensors.  One workgroup per tensor; the chunks'
+// figures are added in double, in a fixed order.  out[t]: {norm, mean, 1.0 if all finite else 0.0, sum of squares}.
+// A chunk whose sum of squares (or sum) is not finite either holds a non-finite element or overflowed in
+// fp32: its 4096 elements are read back and examined one by one, and where they are all finite their figures
+// are formed again in double, so the flag is exact and the norm survives values near the top of the range.
+__global__ __launch_bounds__(256) void k_tensor_stats(const float* __restrict__ chunk_stats,
+                                                      const tplr_tensor_desc* __restrict__ table, int use_dct,
+                                                      float* __restrict__ out) {
+    __shared__ double part[4];
+    __shared__ int bad_any;
+    const tplr_tensor_desc d = table[blockIdx.x];
+    const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
+    if (threadIdx.x == 0) bad_any = 0;
+    __syncthreads();
+    double acc_ss = 0.0, acc_sm = 0.0;
+    int bad = 0;
+    for (int64_t i = threadIdx.x; i < n; i += 256) {
+        double ss = static_cast<double>(chunk_stats[2 * (d.chunk_begin + i)]);
+        double sm = static_cast<double>(chunk_stats[2 * (d.chunk_begin + i) + 1]);
+        if (!isfinite(ss) || !isfinite(sm)) {
+            const bool rows = use_dct || d.ld > 0;  // the (R, C) tensor itself, or chunk after chunk
+            const int64_t y = i / d.x_chunks, x = i - y * d.x_chunks;
+            const float* c0 = rows ? static_cast<const float*>(d.dense) + (y * 64) * d.ld + x * 64
+                                   : static_cast<const float*>(d.dense) + i * 4096;
+            const int64_t ld = rows ? d.ld : 64;
+            ss = 0.0;
+            sm = 0.0;
+            for (int r = 0; r < 64; ++r)
+                for (int c = 0; c < 64; ++c) {
+                    const float v = c0[r * ld + c];
+                    if (!isfinite(v)) bad = 1;
+                    ss += static_cast<double>(v) * static_cast<double>(v);
+                    sm += static_cast<double>(v);
+                }
+        }
+        acc_ss += ss;
+        acc_sm += sm;
+    }
+    if (bad) bad_any = 1;  // (every writer writes the same value)
+    acc_ss = block256_sum_f64(acc_ss, part, threadIdx.x);
+    __syncthreads();
+    acc_sm = block256_sum_f64(acc_sm, part, threadIdx.x);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float* o = out + 4 * static_cast<int64_t>(blockIdx.x);
+        o[0] = static_cast<float>(sqrt(acc_ss));
+        o[1] = n > 0 ? static_cast<float>(acc_sm / (static_cast<double>(n) * 4096.0)) : 0.0f;
+        o[2] = bad_any ? 0.0f : 1.0f;
+        o[3] = static_cast<float>(acc_ss);
+    }
+}
+
 // Plain streaming copy (16 bytes per lane per step, grid-stride).  It exists so that hardware
 // traffic counters can be calibrated: it moves exactly n16 * 16 bytes each way.
 __global__ __launch_bounds__(256) void k_calib_copy(const v4f* __restrict__ src, v4f* __restrict__ dst, int64_t n16) {
@@ -2760,7 +2822,7 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
         if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
     }
     // register-resident fast path: k <= 64 and at most 24 peers; 4-bit counters up to 15 peers, 5-bit beyond
-    const int units = (k > 64 || normalise) ? 0 : n_peers <= 8 ? 8 : n_peers <= 15 ? 16 : n_peers <= 24 ? 24 : 0;
+    const int units = (k > 64 || (normalise & 1)) ? 0 : n_peers <= 8 ? 8 : n_peers <= 15 ? 16 : n_peers <= 24 ? 24 : 0;
     // equally spaced payloads (one staged buffer per window): scalar addressing
     auto apart = [](const void* a, const void* b) {
         return static_cast<int64_t>(reinterpret_cast<intptr_t>(a) - reinterpret_cast<intptr_t>(b));
@@ -2822,7 +2884,7 @@ int tplr_decode_aggregate(const uint8_t* const* h_idx12, const float* const* h_v
     single.chunk_begin = 0;
     single.x_chunks = static_cast<int32_t>(C / 64);
     single.y_chunks = static_cast<int32_t>(R / 64);
-    return launch_decode(h_idx12, h_val, d_peer_scale, n_peers, k, nullptr, single, 1, n, reduce_mode, normalise,
+    return launch_decode(h_idx12, h_val, d_peer_scale, n_peers, k, nullptr, single, 1, n, reduce_mode, normalise ? 1 : 0,
                          use_dct, d_sumsq, stream);
 }
 
@@ -2835,7 +2897,24 @@ int tplr_decode_aggregate_batch(const uint8_t* const* h_idx12, const float* cons
     if (total_chunks == 0) return 0;
     tplr_tensor_desc none = {};
     return launch_decode(h_idx12, h_val, d_scale, n_peers, k, d_desc, none, n_tensors, total_chunks, reduce_mode,
-                         normalise, use_dct, d_sumsq, stream);
+                         normalise ? 1 : 0, use_dct, d_sumsq, stream);
+}
+
+int tplr_decode_aggregate_stats_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale,
+                                      int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
+                                      int64_t total_chunks, int reduce_mode, int normalise, int use_dct,
+                                      float* d_chunk_stats, float* d_tensor_stats, void* stream) {
+    if (int s = check_decode(h_idx12, h_val, n_peers, k, reduce_mode)) return s;
+    if (!d_desc || !d_chunk_stats || !d_tensor_stats || n_tensors < 1 || total_chunks < 0) return TPLR_E_BADARG;
+    if (total_chunks > 0) {
+        tplr_tensor_desc none = {};
+        if (int s = launch_decode(h_idx12, h_val, d_scale, n_peers, k, d_desc, none, n_tensors, total_chunks, reduce_mode,
+                                  (normalise ? 1 : 0) | 2, use_dct, d_chunk_stats, stream))
+            return s;
+    }
+    hipLaunchKernelGGL(k_tensor_stats, dim3(static_cast<unsigned>(n_tensors)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), d_chunk_stats, d_desc, use_dct, d_tensor_stats);
+    return launch_status();
 }
 
 // Rows of any length up to TPLR_MAX_ROW from P peers' flat payloads: row g of the result takes, element

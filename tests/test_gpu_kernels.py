@@ -1152,6 +1152,44 @@ def test_sums_of_squares_of_the_summed_coefficients_from_the_payloads(dev, P, k,
             b0 += cnt
 
 
+@pytest.mark.parametrize("P,k,use_dct", [(15, 32, True), (20, 64, True), (3, 128, True), (15, 32, False), (40, 16, False)])
+def test_aggregate_returns_norm_mean_and_finiteness_of_every_parameter(dev, P, k, use_dct):
+    # what outer_step computes after decode with three passes over each dense gradient
+    # (src/tplr/neurons.py:380-385 norm and mean, :411/:438 isfinite), here from two floats per chunk: against
+    # numpy on the very tensors the launch wrote; every fast and generic instantiation
+    shapes = [(128, 192), (64, 64), (256, 128), (64, 320)]
+    counts = [(a // 64) * (b // 64) for a, b in shapes]
+    n = sum(counts)
+    idxs, vals = make_peers(P, 1, n, k, 6000 + 10 * P + k)
+    # tensor 1: one peer sends a NaN; tensor 2: values near the top of the range (squares overflow, elements and
+    # their sum stay finite); tensor 3: an infinity
+    b = np.cumsum([0] + counts)
+    vals[0].reshape(n, k)[b[1], 3] = np.nan
+    for p in range(P):
+        vals[p].reshape(n, k)[b[2]:b[3]] *= np.float32(1e36) / np.abs(vals[p].reshape(n, k)[b[2]:b[3]]).max()
+    vals[P - 1].reshape(n, k)[b[3] + 2, 0] = np.inf
+    outs = [torch.full(s, 3.0, device=dev) for s in shapes]
+    batch = tc.TensorBatch(outs)
+    di = [torch.from_numpy(i).to(dev) for i in idxs]
+    dv = [torch.from_numpy(v.reshape(n, k)).to(dev) for v in vals]
+    scale = torch.full((len(shapes), P), 0.5, device=dev)
+    st = tc.batch_decompress_decode_batch(batch, di, dv, k, scale=scale, use_dct=use_dct, stats=True).cpu().numpy()
+    plain = [torch.full(s, 3.0, device=dev) for s in shapes]
+    assert tc.batch_decompress_decode_batch(tc.TensorBatch(plain), di, dv, k, scale=scale, use_dct=use_dct) is None
+    for t, o in enumerate(outs):
+        got = o.cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), plain[t].cpu().numpy().view(np.uint32)), t  # the same launch otherwise
+        finite = bool(np.isfinite(got).all())
+        assert st[t, 2] == (1.0 if finite else 0.0), (t, st[t])
+        assert finite == (t in (0, 2)), t
+        if finite:
+            g = got.astype(np.float64)
+            assert abs(st[t, 0] - np.sqrt((g * g).sum())) <= 1e-5 * np.sqrt((g * g).sum()), (t, st[t])
+            assert abs(st[t, 1] - g.mean()) <= 1e-5 * np.abs(g).mean(), (t, st[t])
+        else:
+            assert not np.isfinite(st[t, 0])
+
+
 @pytest.mark.parametrize("two_pass", [False, True])
 @pytest.mark.parametrize("use_dct", [True, False])
 def test_aggregate_mean_over_peers_then_normalised_per_tensor(dev, use_dct, two_pass):
