@@ -204,6 +204,15 @@ int tplr_aggregate_rows(const uint8_t* const* h_idx12, const float* const* h_val
                         int k, const tplr_tensor_desc* d_desc, int n_tensors, int64_t n_rows, int64_t row_len,
                         int reduce_mode, float* d_out, int32_t* d_err, void* stream);
 
+/* tplr_aggregate_rows for rows of 64 (the 1-D parameters) followed by decode (tplr_dct1d, inverse, when use_dct
+ * != 0; src/tplr/compress.py:283-290) in ONE launch, every row written into its tensor where that lies:
+ * d_desc as for tplr_encode_rows_batch (`dense` = the tensor, x_chunks = its rows, chunk_begin = the id of
+ * its first row), total_rows the sum of the tensors' rows.  Same bits as the two calls it replaces.
+ * k even, 2 <= k <= 64; d_err as for tplr_scatter_rows (indices >= 64 are skipped and reported). */
+int tplr_decode_rows_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale, int n_peers,
+                           int k, const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_rows, int reduce_mode,
+                           int use_dct, int32_t* d_err, void* stream);
+
 /* The elementwise steps of the miner's loop body on a flat run of n values (the 1-D parameters):
  * subtract == 0: d_a <- d_a * decay + d_b, two roundings, as mul_ then add_
  * (src/tplr/neurons.py:151-152); subtract != 0: d_a <- d_a - d_b (:171). */

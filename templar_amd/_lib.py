@@ -45,6 +45,7 @@ SIGNATURES = {
     "tplr_scatter_rows": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp]),
     "tplr_flat_update": (_i32, [_vp, _vp, _i64, C.c_float, _i32, _vp]),
     "tplr_aggregate_rows": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _i64, _i32, _vp, _vp, _vp]),
+    "tplr_decode_rows_batch": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _i32, _i32, _vp, _vp]),
     "tplr_peer_sumsq": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp]),
     "tplr_clip_scales": (_i32, [_vp, _i32, _i32, _vp, _vp, _vp]),
     "tplr_calib_copy": (_i32, [_vp, _vp, _i64, _vp]),

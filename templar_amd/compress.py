@@ -1238,14 +1238,16 @@ def encode_compress_rows_batch(batch: RowBatch, topk: int, *, use_dct: bool = Tr
 
 @torch.no_grad()
 def batch_decompress_decode_rows_batch(out: RowBatch, idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], k: int,
-                                       *, clip_norm: bool = True, use_dct: bool = True, validate: bool = True) -> None:
+                                       *, clip_norm: bool = True, use_dct: bool = True, validate: bool = True,
+                                       two_step: bool = False) -> None:
     """batch_decompress + decode (src/tplr/neurons.py:341-367) of every 1-D parameter at once: peer p's
     flat payload is (idxs[p], vals[p]).  Per parameter and peer the values are clipped to the median
     norm over the peers (reference :526-556), every row takes the mean over the peers that sent each
     element (:574-580), the rows go back through the 64-point transform and into the tensors of `out`.
     The payloads are a few hundred KB: a fixed, small number of launches whatever the number of
     parameters.  `validate` (default) raises on an index of 64 or more, as torch's scatter does, which
-    costs a synchronisation; without it such entries are dropped."""
+    costs a synchronisation; without it such entries are dropped.  `two_step` keeps the aggregate and the
+    transform as two launches with the rows in a buffer between them (the same bits)."""
     lib = _lib.load()
     P, R, T, dev = len(vals), out.total_rows, len(out), out.device
     for i, v in zip(idxs, vals):
@@ -1256,10 +1258,21 @@ def batch_decompress_decode_rows_batch(out: RowBatch, idxs: Sequence[torch.Tenso
     vals = [_val_on(x, dev) for x in vals]
     idxs = [_idx_on(i, dev) for i in idxs]
     scale = peer_clip_scales_batch(out, vals, k) if clip_norm else None               # (T, P), two launches
-    rows = torch.empty((R, _CH), dtype=torch.float32, device=dev)
     err = torch.zeros(1, dtype=torch.int32, device=dev) if validate else None
     ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
     vp = (C.c_void_p * P)(*[x.data_ptr() for x in vals])
+    if k <= _CH and not two_step:
+        # one launch: scatter-mean of every row, its inverse transform, written into its tensor
+        with _on(dev):
+            st = lib.tplr_decode_rows_batch(ip, vp, _ptr(scale), P, k, _ptr(out.table), T, R, _lib.REDUCE_MEAN,
+                                            int(use_dct), _ptr(err), _stream(dev))
+        _lib.check(st, "tplr_decode_rows_batch")
+        if validate:
+            bad = int(err.item())  # torch's scatter raises on an out-of-range index as well
+            if bad:
+                raise RuntimeError(f"index {bad} is out of bounds for dimension -1 with size {_CH}")
+        return
+    rows = torch.empty((R, _CH), dtype=torch.float32, device=dev)
     with _on(dev):
         st = lib.tplr_aggregate_rows(ip, vp, _ptr(scale), P, k, _ptr(out.table), T, R, _CH, _lib.REDUCE_MEAN, _ptr(rows),
                                      _ptr(err), _stream(dev))

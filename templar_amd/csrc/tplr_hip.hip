@@ -2395,6 +2395,111 @@ __global__ __launch_bounds__(256) void k_tensor_stats(const float* __restrict__ 
     }
 }
 
+// The 1-D parameters of a set (rows of 64 elements) decoded where they lie: what k_aggregate_rows leaves for a
+// row, then the 64-point inverse transform and its scale exactly as k_dct1d applies them, written into the
+// row's tensor.  One wave per row, a handful of rows per parameter: every peer's entries of the row are
+// requested at once (32 peers to a round), so a row waits for one memory round trip instead of one per peer,
+// and the row's transform runs on one lane (the same instruction sequence as on any lane of k_dct1d).
+template <bool kUseDct>
+__global__ __launch_bounds__(64) void k_decode_rows64(const PeerPtrs pp, const float* __restrict__ scale, int P, int k,
+                                                      const tplr_tensor_desc* __restrict__ table, int n_tensors,
+                                                      int reduce_mode, int32_t* __restrict__ err) {
+    __shared__ float acc[64];
+    __shared__ uint32_t cnt[64];
+    __shared__ uint32_t tag[64];
+    const int lane = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    acc[lane] = 0.f;
+    cnt[lane] = 0;
+    int t = 0;
+    {  // the tensor this row belongs to: the last one that begins at or before it
+        int lo = 0, hi = n_tensors;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (table[mid].chunk_begin <= row)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        t = lo;
+    }
+    const tplr_tensor_desc d = table[t];
+    wave_lds_fence();
+    const int64_t idx_stride = k + (k >> 1);
+    constexpr int kRound = 32;
+    for (int p0 = 0; p0 < P; p0 += kRound) {
+        int me[kRound];
+        float a[kRound];
+#pragma unroll
+        for (int i = 0; i < kRound; ++i) {
+            me[i] = -1;
+            a[i] = 0.f;
+            if (p0 + i < P && lane < k) {
+                const int p = p0 + i;
+                const gbyte* irow = (const gbyte*)pp.idx[p] + row * idx_stride;
+                const gfloat* vrow = (const gfloat*)pp.val[p] + row * k;
+                const float s = scale ? scale[static_cast<int64_t>(t) * P + p] : 1.0f;
+                me[i] = static_cast<int>(load_idx12(irow, lane));
+                a[i] = vrow[lane] * s;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kRound; ++i) {
+            if (p0 + i >= P) break;  // wave-uniform
+            int m = me[i];
+            if (m >= 64) {
+                if (err) atomicMax(err, m);
+                m = -1;
+            }
+            // the usual case: the entries name distinct elements
+            if (m >= 0) tag[m] = static_cast<uint32_t>(lane);
+            wave_lds_fence();
+            const bool clash = m >= 0 && tag[m] != static_cast<uint32_t>(lane);
+            if (__ballot(clash) == 0) {
+                if (m >= 0) {
+                    acc[m] += a[i];
+                    cnt[m] += 1;
+                }
+            } else {
+                // rank among the earlier lanes that name the same element; one rank per turn
+                int rank = 0;
+                for (int l = 0; l < 63; ++l) {
+                    const int other = __shfl(m, l);
+                    rank += (l < lane && other == m && m >= 0) ? 1 : 0;
+                }
+                const int maxrank = static_cast<int>(wave_max_u32(static_cast<uint32_t>(rank)));
+                for (int r = 0; r <= maxrank; ++r) {
+                    if (m >= 0 && rank == r) {
+                        acc[m] += a[i];
+                        cnt[m] += 1;
+                    }
+                    wave_lds_fence();
+                }
+            }
+            wave_lds_fence();
+        }
+    }
+    const uint32_t c = cnt[lane];
+    float v = acc[lane];
+    v = (reduce_mode == TPLR_REDUCE_MEAN && c > 1) ? v / static_cast<float>(c) : v;
+    if (kUseDct) {
+        wave_lds_fence();
+        acc[lane] = v;
+        wave_lds_fence();
+        if (lane == 0) {
+            float w[64];
+#pragma unroll
+            for (int e = 0; e < 64; ++e) w[e] = acc[e];
+            dct64_inv(w);
+#pragma unroll
+            for (int e = 0; e < 64; ++e) acc[e] = w[e] * 0.17677669529663687f;  // one pass is sqrt(32) times the orthonormal transform
+        }
+        wave_lds_fence();
+        v = acc[lane];
+    }
+    static_cast<float*>(d.dense)[(row - d.chunk_begin) * 64 + lane] = v;
+}
+
 // Plain streaming copy (16 bytes per lane per step, grid-stride).  It exists so that hardware
 // traffic counters can be calibrated: it moves exactly n16 * 16 bytes each way.
 __global__ __launch_bounds__(256) void k_calib_copy(const v4f* __restrict__ src, v4f* __restrict__ dst, int64_t n16) {
@@ -3034,6 +3139,30 @@ int tplr_aggregate_rows(const uint8_t* const* h_idx12, const float* const* h_val
     hipLaunchKernelGGL(k_aggregate_rows, dim3(static_cast<unsigned>(n_rows)), dim3(64), 0,
                        static_cast<hipStream_t>(stream), pp, d_scale, n_peers, k, d_desc, n_tensors,
                        static_cast<int>(row_len), reduce_mode, d_out, d_err);
+    return launch_status();
+}
+
+int tplr_decode_rows_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale, int n_peers,
+                           int k, const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_rows, int reduce_mode,
+                           int use_dct, int32_t* d_err, void* stream) {
+    if (!h_idx12 || !h_val || !d_desc || n_tensors < 1 || n_peers < 1 || total_rows < 0 || k < 2 || (k & 1) || k > 64 ||
+        (reduce_mode != TPLR_REDUCE_MEAN && reduce_mode != TPLR_REDUCE_SUM))
+        return TPLR_E_BADARG;
+    if (n_peers > TPLR_MAX_PEERS || total_rows > 0x7fffffff) return TPLR_E_TOOMANY;
+    if (total_rows == 0) return 0;
+    PeerPtrs pp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        pp.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
+        pp.val[p] = p < n_peers ? h_val[p] : nullptr;
+        if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
+    }
+    const dim3 grid(static_cast<unsigned>(total_rows)), block(64);
+    if (use_dct)
+        hipLaunchKernelGGL(k_decode_rows64<true>, grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale, n_peers,
+                           k, d_desc, n_tensors, reduce_mode, d_err);
+    else
+        hipLaunchKernelGGL(k_decode_rows64<false>, grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale, n_peers,
+                           k, d_desc, n_tensors, reduce_mode, d_err);
     return launch_status();
 }
 

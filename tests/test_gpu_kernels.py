@@ -1001,6 +1001,40 @@ def test_row_batch_matches_per_parameter_calls_and_oracle(dev, use_dct):
         tc.batch_decompress_decode_rows_batch(tc.RowBatch(outs), [bad] + idxs[1:], vals, k, use_dct=use_dct)
 
 
+@pytest.mark.parametrize("use_dct", [True, False])
+@pytest.mark.parametrize("P,k", [(1, 2), (15, 32), (20, 64), (40, 16)])
+def test_rows_decode_in_one_launch_equals_aggregate_then_transform(dev, P, k, use_dct):
+    # tplr_decode_rows_batch (scatter-mean of every row, inverse transform, written into its tensor) against
+    # tplr_aggregate_rows followed by tplr_dct1d: the same bits, for separately allocated vectors of ragged
+    # lengths, more peers than one round of loads holds, and rows with repeated indices (added in entry order)
+    rng = np.random.default_rng(7000 + 10 * P + k)
+    lengths = [64, 2048, 128, 768, 64 * 65]
+    R = sum(n // 64 for n in lengths)
+    idxs, vals = [], []
+    for p in range(P):
+        sel = np.argsort(rng.random((R, 64)), axis=1)[:, :k].astype(np.int64)
+        for r in range(p % 3, R, 5):
+            sel[r, k - 1] = sel[r, 0]                      # a repeat inside the row
+        idxs.append(tc.pack_12bit_indices(torch.from_numpy(sel).to(dev).reshape(-1)))
+        vals.append(torch.from_numpy((rng.standard_t(3, size=(R, k)) * (1 + p)).astype(np.float32)).to(dev))
+    one = [torch.full((n,), float("nan"), device=dev) for n in lengths]
+    two = [torch.full((n,), float("nan"), device=dev) for n in lengths]
+    tc.batch_decompress_decode_rows_batch(tc.RowBatch(one), idxs, vals, k, use_dct=use_dct)
+    tc.batch_decompress_decode_rows_batch(tc.RowBatch(two), idxs, vals, k, use_dct=use_dct, two_step=True)
+    for a, b in zip(one, two):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    # and against the oracle's scatter on the concatenation, tensor by tensor
+    r0 = 0
+    for i, n in enumerate(lengths):
+        rows = n // 64
+        pi = [orc.pack12(orc.unpack12(a.cpu().numpy(), (R, k)).reshape(R, k)[r0:r0 + rows]) for a in idxs]
+        pv = [v.cpu().numpy()[r0:r0 + rows] for v in vals]
+        ref = orc.batch_decompress(pi, pv, (rows, 64), 64)
+        ref = orc.dct1d(ref, inverse=True) if use_dct else ref
+        assert np.abs(one[i].cpu().numpy() - ref.reshape(-1)).max() <= 1e-5 * np.abs(ref).max(), i
+        r0 += rows
+
+
 @pytest.mark.parametrize("use_dct,bins,flat", [(True, 0, False), (True, 4, True), (False, 256, False), (False, 0, True)])
 def test_error_feedback_step_for_the_1d_parameters(dev, use_dct, bins, flat):
     # src/tplr/neurons.py:147-171 per parameter, restated with the oracle's pieces on rows of 64
