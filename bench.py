@@ -457,6 +457,46 @@ def main():
         stats = {"what": f"pairwise index overlap + repeats + bounds of {P} peers' packed indices, one launch",
                  "ms": round(st_ms, 4), "GBps": round(st_bytes / (st_ms * 1e-3) / 1e9, 2), "bytes": st_bytes}
 
+    # templar's own settings carry the values as the codes of a four-bin quantiser: the aggregate straight from
+    # the codes against de-quantising every peer first (what outer_step does, src/tplr/neurons.py:325-364)
+    codes_path = None
+    if not DCT and k <= 64 and P <= 24 and args.profile is None:
+        T = len(out_batch)
+        cbuf = torch.empty((P, n_chunks, k), dtype=torch.uint8, device=dev)
+        qps = [[None] * P for _ in range(T)]
+        peer_tables = []
+        for p in range(P):
+            c, q_shift, q_scale, q_lookup = tc.quantize_batch(out_batch, vals[p], k, 4, 6.0)
+            cbuf[p].copy_(c)
+            peer_tables.append((q_lookup, q_shift))
+            for i in range(T):
+                qps[i][p] = (q_shift[i], 1.0, 2, q_lookup[i], torch.float32)
+        codes = [cbuf[p] for p in range(P)]
+        fp32_buf = torch.empty((P, n_chunks, k), dtype=torch.float32, device=dev)
+
+        q_tables = tc.dequantised_tables(qps, dev)   # once per window, like the stage's own tables
+
+        def from_codes():
+            tc.batch_decompress_decode_codes_batch(out_batch, idxs, codes, qps, k, validate=False, tables=q_tables)
+
+        def dequantise_first():
+            fp = [tc.dequantize_batch(out_batch, codes[p].reshape(-1), None, k, out=fp32_buf[p], tables=peer_tables[p])
+                  for p in range(P)]
+            tc.batch_decompress_decode_batch(out_batch, idxs, fp, k, clip_norm=True, use_dct=False)
+
+        c_ms, c_wall = event_ms(from_codes, agg_steps, 2)
+        d_ms, d_wall = event_ms(dequantise_first, agg_steps, 2)
+        code_bytes = n_chunks * (P * (k + k // 2 + k) + 16384)
+        codes_path = {"what": "aggregate of the 2-D set from 4-bin codes (index bytes + one byte per value read, dense "
+                              "written; norms from counts; no fp32 copy of the payload) against de-quantise every peer, "
+                              "norms, fp32 aggregate",
+                      "from_codes_ms": round(c_ms, 4), "from_codes_wall_ms": round(c_wall, 4),
+                      "dequantise_first_ms": round(d_ms, 4), "dequantise_first_wall_ms": round(d_wall, 4),
+                      "from_codes_bytes": code_bytes,
+                      "from_codes_GBps": round(code_bytes / (c_ms * 1e-3) / 1e9, 2),
+                      "from_codes_frac_of_hbm_peak": round(code_bytes / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+        del cbuf, fp32_buf, codes
+
     # a gathered window arriving as the reference's per-parameter host lists (torch.load output):
     # flat staging through one pinned buffer, against one transfer per tensor
     staging = None
@@ -505,6 +545,7 @@ def main():
                                               "of the dense result, one scaling pass); aggregate_ms is the "
                                               "reference's batch_decompress semantics",
         "aggregate_sum_mean_normalised_two_pass_ms": round(aggn2_ms, 4),
+        "aggregate_from_quantised_codes": codes_path,
         "aggregate_with_result_stats": {"kernel_with_stats_ms": round(aggs_ms, 4), "kernel_ms": round(aggk_ms, 4),
                                         "same_stats_by_torch_ms": round(stats_torch_ms, 4),
                                         "what": "per-parameter L2 norm, mean and all-finite flag of the decoded "

@@ -313,6 +313,27 @@ int tplr_quantize_batch(const float* d_val, int k, const tplr_tensor_desc* d_des
                         float range_in_sigmas, int n_slices, double* d_work, uint8_t* d_codes, float* d_shift,
                         float* d_scale, float* d_lookup, void* stream);
 
+/* The aggregate straight from quantised payloads, for a quantiser of at most four bins (templar runs
+ * quantization_bins = 4, hparams/hparams.json) and chunks that are not transformed (use_dct = false): the
+ * loop of maybe_dequantize_values over peers and parameters (src/tplr/compress.py:646-696,
+ * src/tplr/neurons.py:325), the block norms (:346) and batch_decompress (:355-364) without ever writing the
+ * fp32 values.  h_codes[p]: peer p's flat payload of one-byte codes (total_chunks * k bytes, chunk g's at g * k);
+ * d_deq: (n_tensors, n_peers, 4) floats, d_deq[(t * n_peers + p) * 4 + c] = lookup[c] + shift of tensor t as
+ * peer p sent them (:641-643; entries past the quantiser's bins are not read for valid codes).
+ * tplr_code_sumsq: the sums of squares of the de-quantised values per (tensor, peer, slice), in the layout of
+ * tplr_segment_sumsq and for the same consumer (tplr_clip_scales_batch), from four counts per slice;
+ * *d_bad (caller-zeroed, nullable) receives by atomic maximum a code >= n_bins that was met (255 for any
+ * byte above 3): the reference's lookup raises on such a code.
+ * tplr_decode_aggregate_codes_batch: tplr_decode_aggregate_batch with use_dct = 0 and normalise = 0 whose
+ * values are d_deq[..][code & 3] - the same bits as de-quantising first.  k <= 64, n_peers <= 24
+ * (TPLR_E_TOOMANY beyond: de-quantise and call tplr_decode_aggregate_batch). */
+int tplr_code_sumsq(const uint8_t* const* h_codes, int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
+                    int n_slices, int n_bins, const float* d_deq, float* d_sumsq, int32_t* d_bad, void* stream);
+int tplr_decode_aggregate_codes_batch(const uint8_t* const* h_idx12, const uint8_t* const* h_codes, const float* d_deq,
+                                      const float* d_scale, int n_peers, int k, const tplr_tensor_desc* d_desc,
+                                      int n_tensors, int64_t total_chunks, int reduce_mode, float* d_sumsq,
+                                      void* stream);
+
 /* tplr_decode_aggregate_batch together with what its caller looks at next, per parameter
  * (src/tplr/neurons.py:380-385: L2 norm and mean of the decoded gradient for the fingerprint; :411 and
  * :438: the parameter is skipped unless every element is finite), without another pass over the dense

@@ -1442,6 +1442,76 @@ def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[
     return out
 
 
+def dequantised_tables(quant_params: Sequence[Sequence[QuantParamsT]], dev: torch.device) -> tuple[torch.Tensor, int]:
+    """quant_params[i][p] (parameter i, peer p, the reference's 5-tuples) -> ((T, P, max(n_bins, 4)) fp32 table
+    of lookup + shift, n_bins): the value behind every code of every parameter and peer
+    (src/tplr/compress.py:641-643), formed by the same fp32 addition as the element-wise form."""
+    T, P = len(quant_params), len(quant_params[0])
+    lookup, shift, n_bins = _qparam_tables([quant_params[i][p] for i in range(T) for p in range(P)], dev)
+    deq = (lookup + shift[:, None]).view(T, P, n_bins)
+    if n_bins < 4:
+        deq = torch.cat([deq, torch.zeros((T, P, 4 - n_bins), dtype=torch.float32, device=dev)], dim=2)
+    return deq.contiguous(), n_bins
+
+
+@torch.no_grad()
+def batch_decompress_decode_codes_batch(out: TensorBatch, idxs: Sequence[torch.Tensor], codes: Sequence[torch.Tensor],
+                                        quant_params: Sequence[Sequence[QuantParamsT]], k: int, *,
+                                        clip_norm: bool = True, use_dct: bool = False, mean: bool = True,
+                                        validate: bool = True,
+                                        tables: "tuple[torch.Tensor, int] | None" = None) -> None:
+    """maybe_dequantize_values + block norms + batch_decompress + decode of every parameter
+    (src/tplr/neurons.py:325-367) from the peers' QUANTISED flat payloads: codes[p] holds peer p's one-byte
+    codes (total_chunks * k), quant_params[i][p] parameter i's 5-tuple from peer p.  With templar's settings - a
+    quantiser of at most four bins, chunks not transformed, k <= 64, at most 24 peers - the fp32 values are
+    never written: the norms come from four counts per (parameter, peer), and the aggregate kernel picks every
+    entry's value among its peer's four.  Other settings de-quantise first (one launch per peer) and take the
+    fp32 path: the same results either way.  `validate` raises on a code the quantiser cannot have produced,
+    as the reference's table lookup does, at the cost of a synchronisation.  `tables` = what
+    dequantised_tables(quant_params, device) returns, for callers that build it once per window (a few thousand
+    small tensors are stacked to make it)."""
+    lib = _lib.load()
+    P, T, n, dev = len(codes), len(out), out.total_chunks, out.device
+    if tables is None and (len(quant_params) != T or any(len(q) != P for q in quant_params)):
+        raise IndexError("quant_params must hold one entry per parameter and peer")
+    for i, c in zip(idxs, codes):
+        if i.dtype != torch.uint8:
+            raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
+        if c.dtype != torch.uint8 or c.numel() != n * k or i.numel() * 2 != n * k * 3 or not c.is_contiguous():
+            raise RuntimeError(f"flat payload mismatch: {i.numel()} index bytes / {c.numel()} codes for {n} chunks, k={k}")
+    n_bins = int(tables[1]) if tables is not None else int(quant_params[0][0][3].numel())
+    if n_bins > 4 or use_dct or k > _CH or P > 24:
+        vals = []
+        for p in range(P):
+            vals.append(dequantize_batch(out, codes[p].reshape(-1), [quant_params[i][p] for i in range(T)], k))
+        batch_decompress_decode_batch(out, idxs, vals, k, clip_norm=clip_norm, use_dct=use_dct, mean=mean)
+        return
+    deq, n_bins = tables if tables is not None else dequantised_tables(quant_params, dev)
+    if deq.shape != (T, P, 4) or deq.dtype != torch.float32 or not deq.is_contiguous():
+        raise ValueError(f"tables: expected a contiguous fp32 ({T}, {P}, 4) tensor, got {tuple(deq.shape)}")
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+    cp = (C.c_void_p * P)(*[c.data_ptr() for c in codes])
+    scale = None
+    bad = torch.zeros(1, dtype=torch.int32, device=dev) if validate else None
+    with _on(dev):
+        if clip_norm or validate:
+            slices = max(1, min(64, 8192 // (T * P)))
+            ss = torch.empty((T, P, slices), dtype=torch.float32, device=dev)
+            _lib.check(lib.tplr_code_sumsq(cp, P, k, _ptr(out.table), T, slices, n_bins, _ptr(deq), _ptr(ss), _ptr(bad),
+                                           _stream(dev)), "tplr_code_sumsq")
+            if clip_norm:
+                scale = torch.empty((T, P), dtype=torch.float32, device=dev)
+                _lib.check(lib.tplr_clip_scales_batch(_ptr(ss), T, P, slices, _ptr(scale), None, _stream(dev)),
+                           "tplr_clip_scales_batch")
+        if validate:
+            worst = int(bad.item())
+            if worst:
+                raise IndexError(f"index {worst} is out of bounds for dimension 0 with size {n_bins}")
+        st = lib.tplr_decode_aggregate_codes_batch(ip, cp, _ptr(deq), _ptr(scale), P, k, _ptr(out.table), T, n,
+                                                   _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM, None, _stream(dev))
+    _lib.check(st, "tplr_decode_aggregate_codes_batch")
+
+
 class PayloadStage:
     """One window's payloads of all peers as flat buffers in the layout the batch kernels read.
 
@@ -1670,6 +1740,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

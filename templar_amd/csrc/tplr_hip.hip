@@ -686,13 +686,20 @@ struct Counters {
 // pp.idx[0] + p * stride_idx, its values at pp.val[0] + p * stride_val floats, as a staged window lays
 // them out - so every payload address is scalar arithmetic on two base pointers instead of a pair of
 // lane broadcasts per peer and chunk.
-template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false, bool kStrided = false>
+// kCodes (fast path without the transform): the peers' values arrive as the quantiser's codes, one byte
+// each, for a quantiser of at most four bins (templar runs four): pp.val[p] points at bytes, `deq` holds the
+// de-quantised value of every code, deq[(t * P + p) * 4 + c] = lookup + shift of tensor t as peer p sent them
+// (src/tplr/compress.py:637-643), and a lane picks its entry's value among the four its peer's lane holds.
+// A quarter of the value bytes, and the fp32 copy of the payload is never made.
+template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false, bool kStrided = false, bool kCodes = false>
 __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
                                                             int64_t first, int64_t total, int reduce_mode,
                                                             int options, float* __restrict__ sumsq,
-                                                            int64_t stride_idx, int64_t stride_val) {
+                                                            int64_t stride_idx, int64_t stride_val,
+                                                            const float* __restrict__ deq) {
+    static_assert(!kCodes || (kUnits > 0 && !kUseDct && !kSubtract), "codes are served by the fast path without the transform");
     // this launch covers the chunks first .. first + total - 1 of the batch
     // options: bit 0 = per-peer, per-chunk normalisation (generic instantiation); bit 1 = `sumsq` takes two
     // floats per chunk, the sum of squares of the result and the sum of its elements
@@ -768,11 +775,28 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     float a[kRegs];
 
     // clip factors of tensor t into my_scale (wave-uniform branch, taken once per tensor)
+    float my_tab[kCodes ? 4 : 1] = {};  // (kCodes) lane p: peer p's four de-quantised values for that tensor, times my_scale
     auto load_scale = [&](int t) {
-        if (scale && t != t_scale) {
+        if constexpr (kCodes) {
+            if (t != t_scale) {
+                my_scale = (scale ? scale[static_cast<int64_t>(t) * P + pl] : 1.0f) * out_scale;
+                const float4 d4 = *reinterpret_cast<const float4*>(deq + (static_cast<int64_t>(t) * P + pl) * 4);
+                my_tab[0] = d4.x * my_scale, my_tab[1] = d4.y * my_scale, my_tab[2] = d4.z * my_scale, my_tab[3] = d4.w * my_scale;
+                t_scale = t;
+            }
+        } else if (scale && t != t_scale) {
             my_scale = scale[static_cast<int64_t>(t) * P + pl] * out_scale;
             t_scale = t;
         }
+    };
+    // (kCodes) the value of code c as unit i's peer sent it, times its clip factor
+    auto code_value = [&](uint32_t c, int i) -> float {
+        const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_tab[0]), i));
+        const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_tab[kCodes ? 1 : 0]), i));
+        const float s2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_tab[kCodes ? 2 : 0]), i));
+        const float s3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_tab[kCodes ? 3 : 0]), i));
+        const float r0 = (c & 1u) ? s1 : s0, r1 = (c & 1u) ? s3 : s2;
+        return (c & 2u) ? r1 : r0;
     };
     // unit i's entries of chunk g into its two registers
     auto load_payload = [&](int64_t g, int t) {  // fast path only
@@ -780,18 +804,24 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         // kStrided: peer after peer by scalar additions from chunk g's place in peer 0's payload
         const gbyte* irow = (const gbyte*)pp.idx[0] + uniform64(g * idx_stride);
         const gfloat* vrow = (const gfloat*)pp.val[0] + uniform64(g * k);
+        const gbyte* crow = (const gbyte*)pp.val[0] + uniform64(g * k);  // (kCodes)
 #pragma unroll
         for (int i = 0; i < kRegs; ++i) {
             if constexpr (!kStrided) {
                 const int u = i < P ? i : P - 1;  // unused units reload the last peer and stay out of the scatter
                 irow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + g * idx_stride;
                 vrow = reinterpret_cast<const gfloat*>(lane_bcast64(my_val, u)) + g * k;
+                crow = reinterpret_cast<const gbyte*>(lane_bcast64(my_val, u)) + g * k;
             }
             ix[i] = *(const gu16*)(irow + lane_ioff);
-            a[i] = vrow[le];
+            if constexpr (kCodes)
+                a[i] = __builtin_bit_cast(float, static_cast<uint32_t>(crow[le]));
+            else
+                a[i] = vrow[le];
             if (kStrided && i + 1 < P) {  // (unused units reload the last peer)
                 irow += stride_idx;
                 vrow += stride_val;
+                crow += stride_val;  // (kCodes: the stride counts bytes)
             }
         }
     };
@@ -800,7 +830,10 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         const gbyte* irow = (const gbyte*)pp.idx[p] + g * idx_stride;
         const uint32_t w = *(const gu16*)(irow + (3 * (j >> 1) + (j & 1)));
         ixo = (j & 1) ? (w >> 4) : (w & 0xfffu);
-        ao = ((const gfloat*)pp.val[p] + g * k)[j];
+        if constexpr (kCodes)  // (the caller turns the code into its value)
+            ao = __builtin_bit_cast(float, static_cast<uint32_t>(((const gbyte*)pp.val[p] + g * k)[j]));
+        else
+            ao = ((const gfloat*)pp.val[p] + g * k)[j];
     };
 
     const bool fast = kFast;  // (normalise is served by the generic instantiation only)
@@ -852,8 +885,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 for (int i = 0; i < kRegs; ++i) {
                     if (i < P) {  // wave-uniform
                         const uint32_t e = (lane & 1) ? (ix[i] >> 4) : (ix[i] & 0xfffu);
-                        const float x = a[i] * __builtin_bit_cast(float, __builtin_amdgcn_readlane(
-                                                   __builtin_bit_cast(int, my_scale), i));
+                        const float x = kCodes ? code_value(__builtin_bit_cast(uint32_t, a[i]), i)
+                                               : a[i] * __builtin_bit_cast(float, __builtin_amdgcn_readlane(
+                                                            __builtin_bit_cast(int, my_scale), i));
                         // claim, add, write back: the floating-point LDS atomic costs about 3 cycles
                         // per lane, six times this sequence
                         float* t = &tile[tile_pos(e)];
@@ -957,6 +991,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                         float ae;
                         load_entry(p, j, g, ixe, ae);
                         me = static_cast<int>(ixe);
+                        if constexpr (kCodes)
+                            ae = deq[(static_cast<int64_t>(t_now) * P + p) * 4 + (__builtin_bit_cast(uint32_t, ae) & 3u)];
                         // the value as the path this kernel was built for forms it
                         x = normalise ? (ae / nrm) * out_scale : fast ? ae * (sc * out_scale) : (ae * sc) * out_scale;
                         if (phase) x = 1.0f;
@@ -2445,7 +2481,7 @@ __global__ __launch_bounds__(64) void k_decode_rows64(const PeerPtrs pp, const f
         }
 #pragma unroll
         for (int i = 0; i < kRound; ++i) {
-            if (p0 + i >= P) break;  // wave-uniform
+            if (p0 + i >= P) continue;  // wave-uniform
             int m = me[i];
             if (m >= 64) {
                 if (err) atomicMax(err, m);
@@ -2498,6 +2534,81 @@ __global__ __launch_bounds__(64) void k_decode_rows64(const PeerPtrs pp, const f
         v = acc[lane];
     }
     static_cast<float*>(d.dense)[(row - d.chunk_begin) * 64 + lane] = v;
+}
+
+// Per-peer, per-tensor sums of squares of the values behind a payload of codes (quantiser of at most four
+// bins), from the codes alone: a value is one of four, so the sum is four counts times four squares.  Block
+// = (tensor, peer, slice) as in k_segment_sumsq, whose output layout this has; a code is two bits in a byte, and
+// a 32-bit word's four codes are counted with three byte-sum instructions (bit 0 set, bit 1 set, both set).
+// A code that the quantiser cannot have produced (>= n_bins) is reported through `bad` (atomic maximum of
+// the offending byte): the reference's table lookup raises on it (src/tplr/compress.py:641).
+struct CodePtrs {
+    const uint8_t* code[TPLR_MAX_PEERS];
+};
+__global__ __launch_bounds__(256) void k_code_sumsq4(const CodePtrs cp, int P, int k, int S,
+                                                     const tplr_tensor_desc* __restrict__ table, int n_bins,
+                                                     const float* __restrict__ deq, float* __restrict__ sumsq,
+                                                     int32_t* __restrict__ bad) {
+    __shared__ uint32_t part[4][4];
+    const int tp = blockIdx.x / S, sl = blockIdx.x - tp * S;
+    const int t = tp / P, p = tp - t * P;
+    const tplr_tensor_desc d = table[t];
+    const int64_t n_chunks = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
+    const int64_t c0 = n_chunks * sl / S, c1 = n_chunks * (sl + 1) / S;
+    const uint8_t* base = cp.code[p] + (d.chunk_begin + c0) * k;
+    const int64_t n = (c1 - c0) * k;
+    uint32_t n0 = 0, n1 = 0, n11 = 0, over = 0;
+    auto word = [&](uint32_t w) {
+        const uint32_t b0 = w & 0x01010101u, b1 = (w >> 1) & 0x01010101u;
+        n0 = __builtin_amdgcn_sad_u8(b0, 0u, n0);
+        n1 = __builtin_amdgcn_sad_u8(b1, 0u, n1);
+        n11 = __builtin_amdgcn_sad_u8(b0 & b1, 0u, n11);
+        over |= w & 0xfcfcfcfcu;
+    };
+    // bytes up to the first 16-byte boundary and after the last one go one at a time (a byte alone is a word
+    // whose other codes are zero: they add to no count)
+    const int64_t head = n < 16 ? n : ((16 - (reinterpret_cast<uintptr_t>(base) & 15)) & 15);
+    const int64_t body = (n - head) >> 4;
+    const int64_t tail0 = head + (body << 4);
+    for (int64_t i = threadIdx.x; i < head; i += 256) word(base[i]);
+    for (int64_t i = tail0 + threadIdx.x; i < n; i += 256) word(base[i]);
+    typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+    const v4u* v = reinterpret_cast<const v4u*>(base + head);
+    int64_t i = threadIdx.x;
+    for (; i + 7 * 256 < body; i += 8 * 256) {  // eight independent loads in flight per lane
+        v4u x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = __builtin_nontemporal_load(v + i + u * 256);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) word(x[u].x), word(x[u].y), word(x[u].z), word(x[u].w);
+    }
+    for (; i < body; i += 256) {
+        const v4u x = __builtin_nontemporal_load(v + i);
+        word(x.x), word(x.y), word(x.z), word(x.w);
+    }
+    n0 = wave_sum_u32(n0), n1 = wave_sum_u32(n1), n11 = wave_sum_u32(n11);
+    over = wave_max_u32(over);
+    if ((threadIdx.x & 63) == 0) {
+        uint32_t* o = part[threadIdx.x >> 6];
+        o[0] = n0, o[1] = n1, o[2] = n11, o[3] = over;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint64_t a0 = 0, a1 = 0, a11 = 0;
+        uint32_t ov = 0;
+        for (int w = 0; w < 4; ++w) a0 += part[w][0], a1 += part[w][1], a11 += part[w][2], ov |= part[w][3];
+        const uint64_t cnt[4] = {static_cast<uint64_t>(n) - a0 - a1 + a11, a0 - a11, a1 - a11, a11};
+        const float* dq = deq + (static_cast<int64_t>(t) * P + p) * 4;
+        double ss = 0.0;
+        for (int b = 0; b < 4; ++b)
+            if (cnt[b]) ss += static_cast<double>(cnt[b]) * static_cast<double>(dq[b]) * static_cast<double>(dq[b]);
+        sumsq[blockIdx.x] = static_cast<float>(ss);
+        int worst = 0;
+        if (ov) worst = 255;  // (some byte of the slice has a bit beyond the two a code may use)
+        for (int b = n_bins; b < 4; ++b)
+            if (cnt[b]) worst = worst > b ? worst : b;
+        if (worst && bad) atomicMax(bad, worst);
+    }
 }
 
 // Plain streaming copy (16 bytes per lane per step, grid-stride).  It exists so that hardware
@@ -2627,7 +2738,7 @@ template <typename Kernel>
 static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_scale, int n_peers, int k,
                             const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single, int n_tensors,
                             int64_t total, int reduce_mode, int normalise, float* d_sumsq, void* stream,
-                            int64_t stride_idx = 0, int64_t stride_val = 0) {
+                            int64_t stride_idx = 0, int64_t stride_val = 0, const float* d_deq = nullptr) {
     static int resident = 0;  // per kernel variant
     if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
     // a wave keeps one mark per chunk of its range (chunks to be done again on the exact path), so
@@ -2639,7 +2750,7 @@ static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_sc
         const int64_t need = ((count + 7) / 8) * 8;
         const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
         hipLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale, n_peers, k, d_desc,
-                           single, n_tensors, first, count, reduce_mode, normalise, d_sumsq, stride_idx, stride_val);
+                           single, n_tensors, first, count, reduce_mode, normalise, d_sumsq, stride_idx, stride_val, d_deq);
     }
     return launch_status();
 }
@@ -2919,7 +3030,9 @@ int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, co
 
 static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale, int n_peers,
                          int k, const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single, int n_tensors,
-                         int64_t total, int reduce_mode, int normalise, int use_dct, float* d_sumsq, void* stream) {
+                         int64_t total, int reduce_mode, int normalise, int use_dct, float* d_sumsq, void* stream,
+                         const float* d_deq = nullptr) {
+    // d_deq: h_val points at one-byte codes of a quantiser of at most four bins (see kCodes)
     PeerPtrs pp;
     for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
         pp.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
@@ -2938,6 +3051,25 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
     bool strided = true;
     for (int p = 1; p < n_peers; ++p)
         strided = strided && apart(pp.idx[p], pp.idx[0]) == p * si && apart(pp.val[p], pp.val[0]) == p * sv4;
+    if (d_deq) {
+        if (use_dct || units == 0) return TPLR_E_TOOMANY;
+#define TPLR_CODES_CASE(U, BITS)                                                                                    \
+    case U:                                                                                                         \
+        if (strided)                                                                                                \
+            return launch_decode_as(k_decode_aggregate<false, U, BITS, false, true, true>, pp, d_scale, n_peers, k,   \
+                                    d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream, si,    \
+                                    sv4, d_deq);                                                                    \
+        return launch_decode_as(k_decode_aggregate<false, U, BITS, false, false, true>, pp, d_scale, n_peers, k,      \
+                                d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream, 0, 0, d_deq);
+        switch (units) {
+            TPLR_CODES_CASE(8, 4)
+            TPLR_CODES_CASE(16, 4)
+            TPLR_CODES_CASE(24, 5)
+            default:
+                return TPLR_E_TOOMANY;
+        }
+#undef TPLR_CODES_CASE
+    }
 #define TPLR_DECODE_CASE(U, BITS)                                                                                   \
     case U:                                                                                                         \
         if (strided)                                                                                                \
@@ -3003,6 +3135,35 @@ int tplr_decode_aggregate_batch(const uint8_t* const* h_idx12, const float* cons
     tplr_tensor_desc none = {};
     return launch_decode(h_idx12, h_val, d_scale, n_peers, k, d_desc, none, n_tensors, total_chunks, reduce_mode,
                          normalise ? 1 : 0, use_dct, d_sumsq, stream);
+}
+
+int tplr_decode_aggregate_codes_batch(const uint8_t* const* h_idx12, const uint8_t* const* h_codes, const float* d_deq,
+                                      const float* d_scale, int n_peers, int k, const tplr_tensor_desc* d_desc,
+                                      int n_tensors, int64_t total_chunks, int reduce_mode, float* d_sumsq,
+                                      void* stream) {
+    if (int s = check_decode(h_idx12, h_codes, n_peers, k, reduce_mode)) return s;
+    if (!d_desc || !d_deq || n_tensors < 1 || total_chunks < 0) return TPLR_E_BADARG;
+    if (k > 64 || n_peers > 24) return TPLR_E_TOOMANY;
+    if (total_chunks == 0) return 0;
+    tplr_tensor_desc none = {};
+    return launch_decode(h_idx12, reinterpret_cast<const float* const*>(h_codes), d_scale, n_peers, k, d_desc, none,
+                         n_tensors, total_chunks, reduce_mode, 0, 0, d_sumsq, stream, d_deq);
+}
+
+int tplr_code_sumsq(const uint8_t* const* h_codes, int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
+                    int n_slices, int n_bins, const float* d_deq, float* d_sumsq, int32_t* d_bad, void* stream) {
+    if (!h_codes || !d_desc || !d_deq || !d_sumsq || n_peers < 1 || n_tensors < 1 || k < 2 || (k & 1) || n_slices < 1 ||
+        n_bins < 1 || n_bins > 4)
+        return TPLR_E_BADARG;
+    if (n_peers > TPLR_MAX_PEERS || n_slices > 4096) return TPLR_E_TOOMANY;
+    CodePtrs cp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        cp.code[p] = p < n_peers ? h_codes[p] : nullptr;
+        if (p < n_peers && !cp.code[p]) return TPLR_E_BADARG;
+    }
+    hipLaunchKernelGGL(k_code_sumsq4, dim3(static_cast<unsigned>(n_tensors) * n_peers * n_slices), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), cp, n_peers, k, n_slices, d_desc, n_bins, d_deq, d_sumsq, d_bad);
+    return launch_status();
 }
 
 int tplr_decode_aggregate_stats_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale,

@@ -1186,6 +1186,78 @@ def test_sums_of_squares_of_the_summed_coefficients_from_the_payloads(dev, P, k,
             b0 += cnt
 
 
+@pytest.mark.parametrize("P,k,bins,staged", [(20, 64, 4, True), (15, 32, 4, False), (5, 64, 2, False), (8, 16, 3, True),
+                                             (24, 4, 4, False)])
+def test_aggregate_straight_from_four_bin_codes_equals_dequantise_then_aggregate(dev, P, k, bins, staged):
+    # templar's own settings (hparams.json: quantization_bins 4, topk 64, use_dct false, 20 peers): the aggregate
+    # picks every entry's value among its peer's four and the norms come from four counts - against
+    # de-quantising every peer's payload first (src/tplr/neurons.py:325, :346) and the fp32 aggregate: the same
+    # bits (sum mode, fixed factors), and with the clip factors from the counts within rounding of the norms;
+    # against the oracle on the de-quantised values; rows with repeated indices; payloads equally spaced or not
+    shapes = [(128, 192), (64, 64), (192, 128)]
+    T = len(shapes)
+    counts = [(a // 64) * (b // 64) for a, b in shapes]
+    n = sum(counts)
+    idxs, vals = make_peers(P, 1, n, k, 8000 + 10 * P + k)
+    for p in range(0, P, 3):   # repeats inside a row
+        ii = orc.unpack12(idxs[p], (n, k)).reshape(n, k).copy()
+        ii[p % n, k - 1] = ii[p % n, 0]
+        idxs[p] = orc.pack12(ii)
+    batch = tc.TensorBatch([torch.empty(s, device=dev) for s in shapes])
+    di = [torch.from_numpy(i).to(dev) for i in idxs]
+    codes, qps = [], [[None] * P for _ in range(T)]
+    for p in range(P):
+        c, shift, scale, lookup = tc.quantize_batch(batch, torch.from_numpy(vals[p].reshape(n, k)).to(dev), k, bins, 6.0)
+        codes.append(c)
+        for i in range(T):
+            qps[i][p] = (shift[i].clone(), float(scale[i]), bins // 2, lookup[i].clone(), torch.float32)
+    if staged:  # one buffer, the peers' payloads equally spaced (scalar addressing in the kernel)
+        ib = torch.stack(di)
+        cb = torch.stack([c.reshape(-1) for c in codes])
+        di, codes = [ib[p] for p in range(P)], [cb[p].view(n, k) for p in range(P)]
+    fp32 = [tc.dequantize_batch(batch, codes[p].reshape(-1), [qps[i][p] for i in range(T)], k) for p in range(P)]
+    got = [torch.full(s, 7.0, device=dev) for s in shapes]
+    want = [torch.full(s, 7.0, device=dev) for s in shapes]
+    # fixed factors, both reduce modes: bit for bit
+    fixed = torch.from_numpy(np.random.default_rng(P).uniform(0.3, 1.0, (T, P)).astype(np.float32)).to(dev)
+    deq, nb = tc.dequantised_tables(qps, dev)
+    assert nb == bins and deq.shape == (T, P, 4)
+    lib = _lib.load()
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in di])
+    cp = (C.c_void_p * P)(*[c.data_ptr() for c in codes])
+    for mode in (_lib.REDUCE_MEAN, _lib.REDUCE_SUM):
+        for sc in (fixed, None):
+            st = lib.tplr_decode_aggregate_codes_batch(ip, cp, deq.data_ptr(), sc.data_ptr() if sc is not None else None, P, k,
+                                                       tc.TensorBatch(got).table.data_ptr(), T, n, mode, None, None)
+            assert st == 0
+            tc.batch_decompress_decode_batch(tc.TensorBatch(want), di, fp32, k, scale=sc, clip_norm=False, use_dct=False,
+                                             mean=mode == _lib.REDUCE_MEAN)
+            for a, b in zip(got, want):
+                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (mode, sc is None)
+    # the whole call with clip factors from the counts
+    tc.batch_decompress_decode_codes_batch(tc.TensorBatch(got), di, codes, qps, k)
+    tc.batch_decompress_decode_batch(tc.TensorBatch(want), di, fp32, k, use_dct=False)
+    b0 = 0
+    for t, cnt in enumerate(counts):
+        assert relerr(got[t].cpu().numpy(), want[t].cpu().numpy()) <= 1e-6, t
+        ti = [orc.pack12(orc.unpack12(i, (n, k)).reshape(n, k)[b0:b0 + cnt]) for i in idxs]
+        tv = [v.cpu().numpy()[b0:b0 + cnt].reshape(1, cnt, k) for v in fp32]
+        Y, X = shapes[t][0] // 64, shapes[t][1] // 64
+        ref = orc.batch_decompress(ti, tv, (1, cnt, 64, 64), 4096).reshape(Y, X, 64, 64).transpose(0, 2, 1, 3)
+        assert relerr(got[t].cpu().numpy(), ref.reshape(shapes[t])) <= TOL, t
+        b0 += cnt
+    # the settings the kernel does not take (here: the transform) de-quantise first: same call, same semantics
+    tc.batch_decompress_decode_codes_batch(tc.TensorBatch(got), di, codes, qps, k, use_dct=True)
+    tc.batch_decompress_decode_batch(tc.TensorBatch(want), di, fp32, k, use_dct=True)
+    for a, b in zip(got, want):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    # a code the quantiser cannot have produced: the reference's lookup raises
+    spoiled = [c.clone() for c in codes]
+    spoiled[P - 1].view(-1)[5] = bins if bins < 4 else 9
+    with pytest.raises(IndexError):
+        tc.batch_decompress_decode_codes_batch(tc.TensorBatch(got), di, spoiled, qps, k)
+
+
 @pytest.mark.parametrize("P,k,use_dct", [(15, 32, True), (20, 64, True), (3, 128, True), (15, 32, False), (40, 16, False)])
 def test_aggregate_returns_norm_mean_and_finiteness_of_every_parameter(dev, P, k, use_dct):
     # what outer_step computes after decode with three passes over each dense gradient
