@@ -691,7 +691,16 @@ struct Counters {
 // de-quantised value of every code, deq[(t * P + p) * 4 + c] = lookup + shift of tensor t as peer p sent them
 // (src/tplr/compress.py:637-643), and a lane picks its entry's value among the four its peer's lane holds.
 // A quarter of the value bytes, and the fp32 copy of the payload is never made.
-template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false, bool kStrided = false, bool kCodes = false>
+// kWideK (kCodes with equally spaced payloads, k = kWideK = 32 or 64): a load instruction costs this kernel
+// about as much as the bytes it brings (every load queues behind the stores of the compute unit's eight
+// waves), so one instruction serves several peers: every lane takes four bytes of codes - lane l the codes
+// 4 (l mod k/4) .. + 3 of the peer number l / (k/4) among the 256/k peers of that instruction - or the four
+// twelve bytes at 12 m of an index row (m = l mod k/8: entries 8 m .. 8 m + 7, peer l / (k/8) of 512/k), and a
+// lane fetches its own entry from the lane that holds it with lane permutes when the entry is scattered.
+// 8 load instructions per chunk instead of 40 for 20 peers at k = 64, and two register sets of 15
+// registers: the payload is requested two chunks ahead, as in the pipeline with the transform.
+template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false, bool kStrided = false, bool kCodes = false,
+          int kWideK = 0>
 __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
@@ -700,6 +709,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                                                             int64_t stride_idx, int64_t stride_val,
                                                             const float* __restrict__ deq) {
     static_assert(!kCodes || (kUnits > 0 && !kUseDct && !kSubtract), "codes are served by the fast path without the transform");
+    static_assert(kWideK == 0 || (kCodes && kStrided && (kWideK == 32 || kWideK == 64)), "wide loads: codes, equally spaced payloads");
     // this launch covers the chunks first .. first + total - 1 of the batch
     // options: bit 0 = per-peer, per-chunk normalisation (generic instantiation); bit 1 = `sumsq` takes two
     // floats per chunk, the sum of squares of the result and the sum of its elements
@@ -1389,6 +1399,210 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         for (int64_t g = g0; g < g1; g += 2) {
             step(g, s1, std::false_type{});
             if (g + 1 < g1) step(g + 1, s0, std::true_type{});
+        }
+        redo_marked();
+        return;
+    }
+
+    // =====================================================================================
+    // Codes through wide loads (kWideK): four chunks in flight.  Chunk g leaves the tile for registers
+    // and is stored; chunk g + 1 is scattered into the tile; chunk g + 2's payload sits in the other
+    // register set; chunk g + 3's is requested into the registers the scatter has just released.
+    // =====================================================================================
+    if constexpr (kWideK > 0) {
+        constexpr int kPc = 256 / kWideK;                     // peers per register of codes
+        constexpr int kPi = 512 / kWideK;                     // peers per load of packed indices (twelve bytes a lane)
+        constexpr int kCodeRegs = (kUnits + kPc - 1) / kPc;
+        constexpr int kIdxRegs = (kUnits + kPi - 1) / kPi;
+        constexpr int kLc = kWideK / 4, kLi = kWideK / 8;     // lanes per peer in either kind of load
+        struct WSet {  // one chunk's payload
+            uint32_t cw[kCodeRegs];
+            uint32_t iw[kIdxRegs][3];
+            float tab[4];  // lane p: peer p's four de-quantised values for tensor t, times its clip factor
+            int t;
+        };
+        WSet s0, s1;
+        s0.t = s1.t = -1;
+        s0.tab[0] = s0.tab[1] = s0.tab[2] = s0.tab[3] = 0.f;
+        s1.tab[0] = s1.tab[1] = s1.tab[2] = s1.tab[3] = 0.f;
+        // what this lane fetches: codes 4 mc .. 4 mc + 3 of peer (load * kPc + lane / kLc), the twelve bytes at
+        // 12 mi of peer (load * kPi + lane / kLi)'s index row: its entries 8 mi .. 8 mi + 7
+        const int pc_l = lane / kLc, mc = lane - pc_l * kLc;
+        const int pi_l = lane / kLi, mi = lane - pi_l * kLi;
+        const int ioff = 12 * mi;
+        // what this lane scatters: entry `lane` of every unit, found at lane (unit mod kPc) * kLc + lane / 4 of the
+        // unit's code register, byte lane mod 4, and in the three index registers of lane (unit mod kPi) * kLi +
+        // lane / 8, twelve bits from bit 12 (lane mod 8) of their 96
+        const gbyte* const idx0 = (const gbyte*)pp.idx[0];
+        const gbyte* const val0 = (const gbyte*)pp.val[0];
+        // where each register's four bytes lie from the chunk's place in peer 0's payload (the host has
+        // checked that the payloads of all peers span less than 4 GB)
+        uint32_t coff[kCodeRegs], ioff_r[kIdxRegs];
+#pragma unroll
+        for (int r = 0; r < kCodeRegs; ++r) {
+            int p = r * kPc + pc_l;
+            p = p < P ? p : P - 1;  // (lanes past the last peer reload it)
+            coff[r] = static_cast<uint32_t>(p) * static_cast<uint32_t>(stride_val) + 4u * mc;
+        }
+#pragma unroll
+        for (int r = 0; r < kIdxRegs; ++r) {
+            int p = r * kPi + pi_l;
+            p = p < P ? p : P - 1;
+            ioff_r[r] = static_cast<uint32_t>(p) * static_cast<uint32_t>(stride_idx) + static_cast<uint32_t>(ioff);
+        }
+        constexpr bool kAllOn = kWideK == 64;  // every lane owns an entry
+        const int dummy_pos = lane * kLd + kChunk;  // lanes without an entry work on a slot of their own in the tile's padding
+        if constexpr (!kAllOn) {
+            tile[dummy_pos] = 0.f;
+            wave_lds_fence();
+        }
+        typedef uint32_t v3u __attribute__((ext_vector_type(3), aligned(4)));
+        auto wset_load = [&](WSet& st, int64_t g, int t) {
+            if (t != st.t) {  // wave-uniform, once per tensor
+                const float sc = (scale ? scale[static_cast<int64_t>(t) * P + pl] : 1.0f) * out_scale;
+                const float4 d4 = *reinterpret_cast<const float4*>(deq + (static_cast<int64_t>(t) * P + pl) * 4);
+                st.tab[0] = d4.x * sc, st.tab[1] = d4.y * sc, st.tab[2] = d4.z * sc, st.tab[3] = d4.w * sc;
+                st.t = t;
+            }
+            const gbyte* crow = val0 + uniform64(g * kWideK);
+            const gbyte* irow = idx0 + uniform64(g * (kWideK + kWideK / 2));
+            // (the peer count as this call sees it: a copy the optimiser cannot see through, or it keeps one
+            // comparison per register and unit in scalar registers of their own across the chunk loop, and spills them)
+            int Pq = P;
+            asm volatile("" : "+s"(Pq));
+#pragma unroll
+            for (int r = 0; r < kCodeRegs; ++r)
+                if (r * kPc < Pq)  // wave-uniform
+                    st.cw[r] = *(const __attribute__((address_space(1))) uint32_t*)(crow + static_cast<uint64_t>(coff[r]));
+#pragma unroll
+            for (int r = 0; r < kIdxRegs; ++r)
+                if (r * kPi < Pq)  // wave-uniform
+                {
+                    const v3u w = *(const __attribute__((address_space(1))) v3u*)(irow + static_cast<uint64_t>(ioff_r[r]));
+                    st.iw[r][0] = w.x, st.iw[r][1] = w.y, st.iw[r][2] = w.z;
+                }
+        };
+        auto lane_of = [&](float mine, int i) {
+            return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), i));
+        };
+        auto from_lane = [&](uint32_t held, uint32_t from4) {
+            return static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(static_cast<int>(from4), static_cast<int>(held)));
+        };
+        auto wset_scatter = [&](const WSet& st) {
+            // (formed here from a copy of the lane id the optimiser cannot see through: hoisted out of the chunk loop,
+            // these and the per-unit permute addresses derived from them would take fifty registers)
+            int l2 = le;
+            asm volatile("" : "+v"(l2));
+            int Pq = P;
+            asm volatile("" : "+s"(Pq));
+            const uint32_t code_from4 = static_cast<uint32_t>(l2 >> 2) << 2, code_shift = (l2 & 3) * 8;
+            const uint32_t idx_from4 = static_cast<uint32_t>(l2 >> 3) << 2;
+            // the entry's twelve bits inside two of the three registers: (0, 1) for entries 0-2 of the eight,
+            // (1, 2) for 3-5, (2, 2) for 6-7, shifted by less than 32
+            const int e8 = l2 & 7;
+            const bool first3 = e8 < 3, last2 = e8 >= 6;
+            const uint32_t idx_shift = static_cast<uint32_t>(12 * e8 - (first3 ? 0 : last2 ? 64 : 32));
+#pragma unroll
+            for (int i = 0; i < kUnits; ++i) {
+                if (i < Pq) {  // wave-uniform
+                    // (every lane takes part in the permutes, also those without an entry)
+                    const uint32_t cbits = from_lane(st.cw[i / kPc], code_from4 + (i % kPc) * kLc * 4);
+                    const uint32_t w0 = from_lane(st.iw[i / kPi][0], idx_from4 + (i % kPi) * kLi * 4);
+                    const uint32_t w1 = from_lane(st.iw[i / kPi][1], idx_from4 + (i % kPi) * kLi * 4);
+                    const uint32_t w2 = from_lane(st.iw[i / kPi][2], idx_from4 + (i % kPi) * kLi * 4);
+                    const uint32_t ilo = first3 ? w0 : last2 ? w2 : w1, ihi = first3 ? w1 : w2;
+                    const float q0 = lane_of(st.tab[0], i), q1 = lane_of(st.tab[1], i);
+                    const float q2 = lane_of(st.tab[2], i), q3 = lane_of(st.tab[3], i);
+                    const uint32_t cde = cbits >> code_shift;
+                    const uint32_t e = __builtin_amdgcn_alignbit(ihi, ilo, idx_shift) & 0xfffu;
+                    const float r0 = (cde & 1u) ? q1 : q0, r1 = (cde & 1u) ? q3 : q2;
+                    const float xv = (cde & 2u) ? r1 : r0;
+                    // branch-free: a lane without an entry adds zero to its own slot and nothing to a counter
+                    const bool on = kAllOn || lane_on;
+                    const float x = on ? xv : 0.f;
+                    float* t = &tile[on ? tile_pos(e) : dummy_pos];
+                    const float cur = tile_claim(t);
+                    repeat = seen_mark(repeat, cur);
+                    *t = cur + x;
+                    atomicAdd(&cnt[on ? Cnt::word(e) : static_cast<uint32_t>(lane)], on ? 1u << Cnt::shift(e) : 0u);
+                }
+            }
+        };
+        Cursor c;
+        cursor_seek(c, table, single, n_tensors, g0);
+        Out out_cur = out_of(c, g0), out_next = out_cur, out_after = out_cur;
+        wset_load(s0, g0, c.t);
+        zero_tile();
+        wset_scatter(s0);
+        bool skip_cur = __ballot(repeat == kClaimMark) != 0;  // chunk g: found to hold a repeated index, not stored
+        if (skip_cur) mark_redo(g0);
+        repeat = 0;
+        mean_pass();
+        if (g0 + 1 < g1) {
+            cursor_next(c, g0 + 1);
+            out_next = out_of(c, g0 + 1);
+            wset_load(s1, g0 + 1, c.t);
+        }
+        if (g0 + 2 < g1) {
+            cursor_next(c, g0 + 2);
+            out_after = out_of(c, g0 + 2);
+            wset_load(s0, g0 + 2, c.t);
+        }
+        // one chunk: `st` holds chunk g + 1 and is refilled with chunk g + 3.  Chunk g is stored as soon as it has
+        // left the tile, so that its 64 registers are free while the next chunk is scattered
+        auto step = [&](int64_t g, WSet& st) {
+            {
+                // (tile and destination addresses are formed per chunk from an opaque copy of the lane id: hoisted
+                // out of the loop they take a hundred registers)
+                int lane = threadIdx.x;
+                asm volatile("" : "+v"(lane));
+                float v[64];
+                if (out_cur.ld > 0) {  // wave-uniform
+                    tile_cols_to_regs(v, tile, lane);
+                } else {
+#pragma unroll
+                    for (int q0 = 0; q0 < 16; ++q0) {
+                        const int q = q0 * 64 + lane;
+                        const float4 t = *reinterpret_cast<const float4*>(tile + (q >> 4) * kLd + ((q & 15) << 2));
+                        v[4 * q0] = t.x, v[4 * q0 + 1] = t.y, v[4 * q0 + 2] = t.z, v[4 * q0 + 3] = t.w;
+                    }
+                }
+                wave_lds_fence();
+                chunk_stats(v, g, skip_cur);
+                gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0));
+                if (out_cur.ld > 0) {
+                    store_chunk_rows(v, (void*)dst, uniform64(out_cur.ld), lane, skip_cur);
+                } else if (!skip_cur) {
+#pragma unroll
+                    for (int q0 = 0; q0 < 16; ++q0)
+                        reinterpret_cast<float4*>((float*)dst)[q0 * 64 + lane] =
+                            make_float4(v[4 * q0], v[4 * q0 + 1], v[4 * q0 + 2], v[4 * q0 + 3]);
+                }
+            }
+            const bool more = g + 1 < g1;
+            Out out3 = out_after;
+            bool skip_next = false;
+            if (more) {
+                zero_tile();
+                wset_scatter(st);
+                if (g + 3 < g1) {
+                    cursor_next(c, g + 3);
+                    out3 = out_of(c, g + 3);
+                    wset_load(st, g + 3, c.t);
+                }
+                skip_next = __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
+                if (skip_next) mark_redo(g + 1);
+                repeat = 0;
+                mean_pass();
+            }
+            skip_cur = skip_next;
+            out_cur = out_next;
+            out_next = out_after;
+            out_after = out3;
+        };
+        for (int64_t g = g0; g < g1; g += 2) {
+            step(g, s1);
+            if (g + 1 < g1) step(g + 1, s0);
         }
         redo_marked();
         return;
@@ -3053,8 +3267,20 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
         strided = strided && apart(pp.idx[p], pp.idx[0]) == p * si && apart(pp.val[p], pp.val[0]) == p * sv4;
     if (d_deq) {
         if (use_dct || units == 0) return TPLR_E_TOOMANY;
+        // wide loads take four aligned bytes of codes at a time, 32-bit lane offsets from peer 0's payload
+        const bool wide_ok = (reinterpret_cast<uintptr_t>(pp.val[0]) & 3) == 0 && (sv4 & 3) == 0 && sv4 >= 0 && si >= 0 &&
+                             (reinterpret_cast<uintptr_t>(pp.idx[0]) & 3) == 0 && (si & 3) == 0 &&
+                             sv4 * n_peers < (int64_t{1} << 32) && si * n_peers < (int64_t{1} << 32);
 #define TPLR_CODES_CASE(U, BITS)                                                                                    \
     case U:                                                                                                         \
+        if (strided && wide_ok && k == 64)                                                                          \
+            return launch_decode_as(k_decode_aggregate<false, U, BITS, false, true, true, 64>, pp, d_scale, n_peers,  \
+                                    k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream, si, \
+                                    sv4, d_deq);                                                                    \
+        if (strided && wide_ok && k == 32)                                                                          \
+            return launch_decode_as(k_decode_aggregate<false, U, BITS, false, true, true, 32>, pp, d_scale, n_peers,  \
+                                    k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream, si, \
+                                    sv4, d_deq);                                                                    \
         if (strided)                                                                                                \
             return launch_decode_as(k_decode_aggregate<false, U, BITS, false, true, true>, pp, d_scale, n_peers, k,   \
                                     d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream, si,    \
