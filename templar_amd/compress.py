@@ -1601,12 +1601,14 @@ class PayloadStage:
 
     @torch.no_grad()
     def load(self, idxs: Sequence[Sequence[torch.Tensor]], vals: Sequence[Sequence[torch.Tensor]],
-             quant_params: Sequence[Sequence[QuantParamsT]] | None = None):
+             quant_params: Sequence[Sequence[QuantParamsT]] | None = None, *, expand: bool = True):
         """`idxs[i][p]`, `vals[i][p]`, `quant_params[i][p]`: parameter i (TensorBatch order), peer p, as in
         the reference's lists.  Host tensors go through the pinned buffer and one copy; device tensors
         are concatenated on the device.  Returns (idx12, val): lists over peers of the flat packed
         indices and the fp32 values (total_chunks, k), ready for batch_decompress_decode_batch,
-        peer_clip_scales_batch and index_stats_batch."""
+        peer_clip_scales_batch and index_stats_batch.  expand=False (a stage that holds codes) leaves the
+        codes as they are: it returns them in place of the values and keeps `self.tables`, what
+        batch_decompress_decode_codes_batch takes as `tables` to aggregate straight from them."""
         T = len(self.batch)
         if len(idxs) != T or len(vals) != T:
             raise IndexError(f"{len(idxs)} index lists / {len(vals)} value lists for {T} parameters")
@@ -1666,6 +1668,9 @@ class PayloadStage:
             return out_i, out_v
         if quant_params is None or len(quant_params) != T or any(len(q) != P for q in quant_params):
             raise IndexError("quant_params must hold one entry per parameter and peer")
+        if not expand:
+            self.tables = dequantised_tables(quant_params, self.dev.device)
+            return out_i, out_v
         lookup, shift, n_bins = _qparam_tables([quant_params[i][p] for p in range(P) for i in range(T)], self.dev.device)
         lib = _lib.load()
         dev, n = self.dev.device, self.batch.total_chunks

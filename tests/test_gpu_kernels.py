@@ -1246,6 +1246,16 @@ def test_aggregate_straight_from_four_bin_codes_equals_dequantise_then_aggregate
         ref = orc.batch_decompress(ti, tv, (1, cnt, 64, 64), 4096).reshape(Y, X, 64, 64).transpose(0, 2, 1, 3)
         assert relerr(got[t].cpu().numpy(), ref.reshape(shapes[t])) <= TOL, t
         b0 += cnt
+    # a stage that keeps the codes hands them and its tables to the same call
+    stage = tc.PayloadStage(batch, k, P, quantized=True)
+    per_i = [[batch.payload_slice(i, di[p], fp32[p], k)[0].cpu() for p in range(P)] for i in range(T)]
+    per_c = [[codes[p].reshape(-1)[batch.offsets[i] * k:(batch.offsets[i] + batch.payload_rows(i)) * k].cpu()
+              for p in range(P)] for i in range(T)]
+    si, sc = stage.load(per_i, per_c, qps, expand=False)
+    staged_out = [torch.full(s, 7.0, device=dev) for s in shapes]
+    tc.batch_decompress_decode_codes_batch(tc.TensorBatch(staged_out), si, sc, qps, k, tables=stage.tables)
+    for a, b in zip(staged_out, got):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
     # the settings the kernel does not take (here: the transform) de-quantise first: same call, same semantics
     tc.batch_decompress_decode_codes_batch(tc.TensorBatch(got), di, codes, qps, k, use_dct=True)
     tc.batch_decompress_decode_batch(tc.TensorBatch(want), di, fp32, k, use_dct=True)
