@@ -342,3 +342,88 @@ def test_full_set_transform_and_selection_against_torch(dev, name):
         top = torch.topk(rows.abs(), k, dim=1, largest=True, sorted=True).values
         assert torch.equal(top, pv.abs())
     assert worst > 0.0
+
+
+def _random_payloads(dev, n, P, k, seed):
+    """P peers' flat payloads of n rows: k distinct indices per row, normal values growing with the peer."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    packed, vals = [], []
+    for p in range(P):
+        sel = torch.rand((n, 4096), device=dev, generator=g).topk(k, dim=-1).indices
+        packed.append(tc.pack_12bit_indices(sel.contiguous()))
+        vals.append(torch.randn((n, k), device=dev, generator=g) * (1 + p))
+        del sel
+    return packed, vals
+
+
+def test_full_set_aggregate_from_four_bin_codes(dev):
+    # templar's own settings on the 1B shapes (20 peers, k = 64, no transform, 4-bin quantiser), every chunk:
+    # the aggregate straight from the codes of a staged window (wide loads) is bitwise the fp32 aggregate of the
+    # de-quantised values with the same factors, and the whole call (norms from counts) agrees with de-quantise,
+    # norms, aggregate within rounding of the clip factors
+    P, k = 20, 64
+    shapes = [s for s in workloads.CONFIGS["cfg3_llama1b"]["shapes"] if len(s) == 2]
+    n = sum((a // 64) * (b // 64) for a, b in shapes)
+    T = len(shapes)
+    outs = [torch.empty(s, device=dev) for s in shapes]
+    batch = tc.TensorBatch(outs)
+    packed, vals = _random_payloads(dev, n, P, k, 99)
+    ibuf = torch.stack(packed)
+    cbuf = torch.empty((P, n, k), dtype=torch.uint8, device=dev)
+    qps = [[None] * P for _ in range(T)]
+    fp32 = []
+    for p in range(P):
+        c, shift, scale, lookup = tc.quantize_batch(batch, vals[p], k, 4, 6.0)
+        cbuf[p].copy_(c)
+        fp32.append(tc.dequantize_batch(batch, c.reshape(-1), None, k, tables=(lookup, shift)))
+        for i in range(T):
+            qps[i][p] = (shift[i], 1.0, 2, lookup[i], torch.float32)
+    del vals, packed
+    idxs, codes = [ibuf[p] for p in range(P)], [cbuf[p] for p in range(P)]
+    tables = tc.dequantised_tables(qps, dev)
+    want = [torch.empty(s, device=dev) for s in shapes]
+    tc.batch_decompress_decode_codes_batch(batch, idxs, codes, qps, k, tables=tables)
+    tc.batch_decompress_decode_batch(tc.TensorBatch(want), idxs, fp32, k, use_dct=False)
+    for t, (a, b) in enumerate(zip(outs, want)):
+        assert float((a - b).abs().max()) <= 1e-6 * float(b.abs().max()), t
+    # fixed factors: bit for bit
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    scale = torch.rand((T, P), device=dev, generator=g) * 0.5 + 0.5
+    import ctypes as C
+    from templar_amd import _lib
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+    cp = (C.c_void_p * P)(*[c.data_ptr() for c in codes])
+    st = _lib.load().tplr_decode_aggregate_codes_batch(ip, cp, tables[0].data_ptr(), scale.data_ptr(), P, k,
+                                                       batch.table.data_ptr(), T, n, _lib.REDUCE_MEAN, None, None)
+    assert st == 0
+    tc.batch_decompress_decode_batch(tc.TensorBatch(want), idxs, fp32, k, scale=scale, use_dct=False)
+    for t, (a, b) in enumerate(zip(outs, want)):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32)), t
+
+
+def test_full_set_normalised_mean_and_result_statistics(dev):
+    # the 1B shapes, 15 peers, k = 32: the per-tensor norms taken from the payloads before the one aggregate launch
+    # (orthonormal transform) give the tensors the literal order gives (aggregate, norms of the dense result,
+    # scaling pass), every tensor of unit norm; and the statistics the aggregate leaves on its way are those of
+    # the tensors it wrote
+    P, k = 15, 32
+    shapes = [s for s in workloads.CONFIGS["cfg3_llama1b"]["shapes"] if len(s) == 2]
+    n = sum((a // 64) * (b // 64) for a, b in shapes)
+    packed, vals = _random_payloads(dev, n, P, k, 123)
+    one = [torch.empty(s, device=dev) for s in shapes]
+    two = [torch.empty(s, device=dev) for s in shapes]
+    f1 = tc.aggregate_mean_normalised_batch(tc.TensorBatch(one), packed, vals, k)
+    f2 = tc.aggregate_mean_normalised_batch(tc.TensorBatch(two), packed, vals, k, two_pass=True)
+    assert float(((f1 - f2).abs() / f2).max()) <= 1e-5
+    for t, (a, b) in enumerate(zip(one, two)):
+        assert float((a - b).abs().max()) <= TOL * float(b.abs().max()), t
+        assert abs(float(torch.linalg.vector_norm(a.double())) - 1.0) <= 1e-5, t
+    del two
+    stats = tc.batch_decompress_decode_batch(tc.TensorBatch(one), packed, vals, k, stats=True)
+    for t, a in enumerate(one):
+        d = a.double()
+        assert abs(float(stats[t, 0]) - float(torch.linalg.vector_norm(d))) <= 1e-5 * float(torch.linalg.vector_norm(d)), t
+        assert abs(float(stats[t, 1]) - float(d.mean())) <= 1e-5 * float(d.abs().mean()), t
+        assert float(stats[t, 2]) == 1.0
