@@ -427,3 +427,45 @@ def test_full_set_normalised_mean_and_result_statistics(dev):
         assert abs(float(stats[t, 0]) - float(torch.linalg.vector_norm(d))) <= 1e-5 * float(torch.linalg.vector_norm(d)), t
         assert abs(float(stats[t, 1]) - float(d.mean())) <= 1e-5 * float(d.abs().mean()), t
         assert float(stats[t, 2]) == 1.0
+
+
+@pytest.mark.parametrize("P,k,chunks_y", [(20, 64, 70), (15, 32, 50), (7, 64, 33), (24, 32, 97)])
+def test_codes_aggregate_wave_ranges_of_a_few_chunks(dev, P, k, chunks_y):
+    # between the unit-test sizes (at most one chunk per wave) and the full sets (hundreds): wave ranges of one
+    # to five chunks, where the pipeline's prologue, its two register sets and its tail all meet - the codes
+    # aggregate of a staged window (wide loads) bit for bit against the fp32 aggregate of the de-quantised values
+    import ctypes as C
+    from templar_amd import _lib
+    shapes = [(chunks_y * 64, 128 * 64), (64, 64), (3 * 64, 5 * 64)]
+    T = len(shapes)
+    n = sum((a // 64) * (b // 64) for a, b in shapes)
+    outs = [torch.empty(s, device=dev) for s in shapes]
+    want = [torch.empty(s, device=dev) for s in shapes]
+    batch = tc.TensorBatch(outs)
+    packed, vals = _random_payloads(dev, n, P, k, 1000 + P + k)
+    ibuf, cbuf = torch.stack(packed), torch.empty((P, n, k), dtype=torch.uint8, device=dev)
+    qps = [[None] * P for _ in range(T)]
+    fp32 = []
+    for p in range(P):
+        c, shift, scale, lookup = tc.quantize_batch(batch, vals[p], k, 4, 6.0)
+        cbuf[p].copy_(c)
+        fp32.append(tc.dequantize_batch(batch, c.reshape(-1), None, k, tables=(lookup, shift)))
+        for i in range(T):
+            qps[i][p] = (shift[i], 1.0, 2, lookup[i], torch.float32)
+    idxs, codes = [ibuf[p] for p in range(P)], [cbuf[p] for p in range(P)]
+    deq, _ = tc.dequantised_tables(qps, dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(P)
+    scale = torch.rand((T, P), device=dev, generator=g) * 0.5 + 0.5
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+    cp = (C.c_void_p * P)(*[c.data_ptr() for c in codes])
+    for mode in (_lib.REDUCE_MEAN, _lib.REDUCE_SUM):
+        for o in outs:
+            o.fill_(float("nan"))
+        st = _lib.load().tplr_decode_aggregate_codes_batch(ip, cp, deq.data_ptr(), scale.data_ptr(), P, k,
+                                                           batch.table.data_ptr(), T, n, mode, None, None)
+        assert st == 0
+        tc.batch_decompress_decode_batch(tc.TensorBatch(want), idxs, fp32, k, scale=scale, use_dct=False,
+                                         mean=mode == _lib.REDUCE_MEAN)
+        for t, (a, b) in enumerate(zip(outs, want)):
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (mode, t)
