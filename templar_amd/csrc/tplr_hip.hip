@@ -2407,7 +2407,14 @@ __global__ __launch_bounds__(256) void k_tensor_rnorm(const float* __restrict__ 
     const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
     const float* s = sumsq + d.chunk_begin;
     double acc = 0.0;
-    for (int64_t i = threadIdx.x; i < n; i += 256) acc += static_cast<double>(s[i]);
+    {  // four independent loads in flight per thread: the largest tensors have tens of thousands of chunks
+        int64_t i = threadIdx.x;
+        for (; i + 768 < n; i += 1024) {
+            const float a0 = s[i], a1 = s[i + 256], a2 = s[i + 512], a3 = s[i + 768];
+            acc += (static_cast<double>(a0) + static_cast<double>(a1)) + (static_cast<double>(a2) + static_cast<double>(a3));
+        }
+        for (; i < n; i += 256) acc += static_cast<double>(s[i]);
+    }
     acc = block256_sum_f64(acc, part, threadIdx.x);
     if (threadIdx.x == 0) factor[blockIdx.x] = 1.0f / (static_cast<float>(sqrt(acc)) + eps);
 }
@@ -2580,7 +2587,14 @@ __global__ __launch_bounds__(256) void k_tensor_rnorm_scales(const float* __rest
     const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
     const float* s = sumsq + d.chunk_begin;
     double acc = 0.0;
-    for (int64_t i = threadIdx.x; i < n; i += 256) acc += static_cast<double>(s[i]);
+    {  // four independent loads in flight per thread: the largest tensors have tens of thousands of chunks
+        int64_t i = threadIdx.x;
+        for (; i + 768 < n; i += 1024) {
+            const float a0 = s[i], a1 = s[i + 256], a2 = s[i + 512], a3 = s[i + 768];
+            acc += (static_cast<double>(a0) + static_cast<double>(a1)) + (static_cast<double>(a2) + static_cast<double>(a3));
+        }
+        for (; i < n; i += 256) acc += static_cast<double>(s[i]);
+    }
     acc = block256_sum_f64(acc, part, threadIdx.x);
     if (threadIdx.x == 0) {
         const float f = 1.0f / (static_cast<float>(sqrt(acc)) * pre + eps);
@@ -2609,9 +2623,10 @@ __global__ __launch_bounds__(256) void k_tensor_stats(const float* __restrict__ 
     __syncthreads();
     double acc_ss = 0.0, acc_sm = 0.0;
     int bad = 0;
-    for (int64_t i = threadIdx.x; i < n; i += 256) {
-        double ss = static_cast<double>(chunk_stats[2 * (d.chunk_begin + i)]);
-        double sm = static_cast<double>(chunk_stats[2 * (d.chunk_begin + i) + 1]);
+    const float2* cs = reinterpret_cast<const float2*>(chunk_stats) + d.chunk_begin;
+    // one chunk's figures; not finite: the chunk is read back (rare)
+    auto take = [&](int64_t i, float2 got) {
+        double ss = static_cast<double>(got.x), sm = static_cast<double>(got.y);
         if (!isfinite(ss) || !isfinite(sm)) {
             const bool rows = use_dct || d.ld > 0;  // the (R, C) tensor itself, or chunk after chunk
             const int64_t y = i / d.x_chunks, x = i - y * d.x_chunks;
@@ -2620,7 +2635,9 @@ __global__ __launch_bounds__(256) void k_tensor_stats(const float* __restrict__ 
             const int64_t ld = rows ? d.ld : 64;
             ss = 0.0;
             sm = 0.0;
+#pragma unroll 1
             for (int r = 0; r < 64; ++r)
+#pragma unroll 1
                 for (int c = 0; c < 64; ++c) {
                     const float v = c0[r * ld + c];
                     if (!isfinite(v)) bad = 1;
@@ -2630,6 +2647,14 @@ __global__ __launch_bounds__(256) void k_tensor_stats(const float* __restrict__ 
         }
         acc_ss += ss;
         acc_sm += sm;
+    };
+    {  // four independent loads in flight per thread: the largest tensors have tens of thousands of chunks
+        int64_t i = threadIdx.x;
+        for (; i + 768 < n; i += 1024) {
+            const float2 g0 = cs[i], g1 = cs[i + 256], g2 = cs[i + 512], g3 = cs[i + 768];
+            take(i, g0), take(i + 256, g1), take(i + 512, g2), take(i + 768, g3);
+        }
+        for (; i < n; i += 256) take(i, cs[i]);
     }
     if (bad) bad_any = 1;  // (every writer writes the same value)
     acc_ss = block256_sum_f64(acc_ss, part, threadIdx.x);
