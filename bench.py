@@ -459,43 +459,80 @@ def main():
 
     # templar's own settings carry the values as the codes of a four-bin quantiser: the aggregate straight from
     # the codes against de-quantising every peer first (what outer_step does, src/tplr/neurons.py:325-364)
-    codes_path = None
-    if not DCT and k <= 64 and P <= 24 and args.profile is None:
-        T = len(out_batch)
-        cbuf = torch.empty((P, n_chunks, k), dtype=torch.uint8, device=dev)
-        qps = [[None] * P for _ in range(T)]
+    def codes_figures(idxs_, vals_, kk):
+        """idxs_/vals_: the peers' fp32 flat payloads of the 2-D set (views of a staged window) at top-k kk, chunks
+        not transformed; they are quantised with four bins here."""
+        PP, T = len(vals_), len(out_batch)
+        cbuf = torch.empty((PP, n_chunks, kk), dtype=torch.uint8, device=dev)
+        qps = [[None] * PP for _ in range(T)]
         peer_tables = []
-        for p in range(P):
-            c, q_shift, q_scale, q_lookup = tc.quantize_batch(out_batch, vals[p], k, 4, 6.0)
+        for p in range(PP):
+            c, q_shift, q_scale, q_lookup = tc.quantize_batch(out_batch, vals_[p], kk, 4, 6.0)
             cbuf[p].copy_(c)
             peer_tables.append((q_lookup, q_shift))
             for i in range(T):
                 qps[i][p] = (q_shift[i], 1.0, 2, q_lookup[i], torch.float32)
-        codes = [cbuf[p] for p in range(P)]
-        fp32_buf = torch.empty((P, n_chunks, k), dtype=torch.float32, device=dev)
-
+        codes = [cbuf[p] for p in range(PP)]
+        fp32_buf = torch.empty((PP, n_chunks, kk), dtype=torch.float32, device=dev)
         q_tables = tc.dequantised_tables(qps, dev)   # once per window, like the stage's own tables
 
         def from_codes():
-            tc.batch_decompress_decode_codes_batch(out_batch, idxs, codes, qps, k, validate=False, tables=q_tables)
+            tc.batch_decompress_decode_codes_batch(out_batch, idxs_, codes, qps, kk, validate=False, tables=q_tables)
 
         def dequantise_first():
-            fp = [tc.dequantize_batch(out_batch, codes[p].reshape(-1), None, k, out=fp32_buf[p], tables=peer_tables[p])
-                  for p in range(P)]
-            tc.batch_decompress_decode_batch(out_batch, idxs, fp, k, clip_norm=True, use_dct=False)
+            fp = [tc.dequantize_batch(out_batch, codes[p].reshape(-1), None, kk, out=fp32_buf[p], tables=peer_tables[p])
+                  for p in range(PP)]
+            tc.batch_decompress_decode_batch(out_batch, idxs_, fp, kk, clip_norm=True, use_dct=False)
 
-        c_ms, c_wall = event_ms(from_codes, agg_steps, 2)
+        c_ms, c_wall = event_ms(from_codes, agg_steps, 2, settle=True)
         d_ms, d_wall = event_ms(dequantise_first, agg_steps, 2)
-        code_bytes = n_chunks * (P * (k + k // 2 + k) + 16384)
-        codes_path = {"what": "aggregate of the 2-D set from 4-bin codes (index bytes + one byte per value read, dense "
-                              "written; norms from counts; no fp32 copy of the payload) against de-quantise every peer, "
-                              "norms, fp32 aggregate",
-                      "from_codes_ms": round(c_ms, 4), "from_codes_wall_ms": round(c_wall, 4),
-                      "dequantise_first_ms": round(d_ms, 4), "dequantise_first_wall_ms": round(d_wall, 4),
-                      "from_codes_bytes": code_bytes,
-                      "from_codes_GBps": round(code_bytes / (c_ms * 1e-3) / 1e9, 2),
-                      "from_codes_frac_of_hbm_peak": round(code_bytes / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
-        del cbuf, fp32_buf, codes
+        code_bytes = n_chunks * (PP * (kk + kk // 2 + kk) + 16384)
+        return {"what": f"aggregate of the 2-D set from 4-bin codes, {PP} peers, k = {kk}, chunks not transformed (index "
+                        "bytes + one byte per value read, dense written; norms from counts; no fp32 copy of the payload) "
+                        "against de-quantise every peer, norms, fp32 aggregate",
+                "from_codes_ms": round(c_ms, 4), "from_codes_wall_ms": round(c_wall, 4),
+                "dequantise_first_ms": round(d_ms, 4), "dequantise_first_wall_ms": round(d_wall, 4),
+                "from_codes_bytes": code_bytes,
+                "from_codes_GBps": round(code_bytes / (c_ms * 1e-3) / 1e9, 2),
+                "from_codes_frac_of_hbm_peak": round(code_bytes / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
+    codes_path = None
+    if not DCT and k <= 64 and P <= 24 and args.profile is None:
+        codes_path = codes_figures(idxs, vals, k)
+
+    # the same set at templar's own settings (hparams/hparams.json: topk_compression 64, use_dct false,
+    # quantization_bins 4, 20 gathered peers), when this run is not already made with them: the encode launch
+    # and the aggregate from codes, on payloads built here
+    templar_settings = None
+    if args.profile is None and args.workload == "cfg3_llama1b" and (DCT or k != 64 or P != 20):
+        tk, tP = 64, 20
+        g2 = [g for g in workloads.gradient_set(args.workload, device=dev) if g.dim() == 2]
+        b2 = tc.TensorBatch(g2)
+        t_idx = torch.empty(n_chunks * (tk // 2) * 3, dtype=torch.uint8, device=dev)
+        t_val = torch.empty((n_chunks, tk), dtype=torch.float32, device=dev)
+        te_ms, _ = event_ms(lambda: tc.encode_compress_batch(b2, tk, use_dct=False, idx12=t_idx, val=t_val),
+                            args.steps, args.warmup, settle=True)
+        te_bytes = n_chunks * (16384 + 11 * tk // 2)
+        t_win = tc.PayloadStage(batch, tk, tP, quantized=False)
+        t_idxs, t_vals = [], []
+        for p in range(tP):
+            own = [workloads.student_t3(tuple(g.shape), 3000 * (p + 1) + j, row_scale=True, device=dev).add_(g, alpha=0.5)
+                   for j, g in enumerate(g2)]
+            i12, v = t_win.regions(p)
+            tc.encode_compress_batch(tc.TensorBatch(own), tk, use_dct=False, idx12=i12, val=v)
+            torch.cuda.synchronize()
+            t_idxs.append(i12)
+            t_vals.append(v)
+            del own
+        del g2, b2
+        templar_settings = {
+            "what": "the same 1B set at templar's hparams.json settings: top-k 64 per chunk, chunks not transformed, "
+                    "4-bin quantiser, 20 peers",
+            "encode_ms": round(te_ms, 4), "encode_GBps": round(te_bytes / (te_ms * 1e-3) / 1e9, 2),
+            "encode_frac_of_hbm_peak": round(te_bytes / (te_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "aggregate": codes_figures(t_idxs, t_vals, tk),
+        }
+        del t_win, t_idxs, t_vals
 
     # a gathered window arriving as the reference's per-parameter host lists (torch.load output):
     # flat staging through one pinned buffer, against one transfer per tensor
@@ -546,6 +583,7 @@ def main():
                                               "reference's batch_decompress semantics",
         "aggregate_sum_mean_normalised_two_pass_ms": round(aggn2_ms, 4),
         "aggregate_from_quantised_codes": codes_path,
+        "templar_settings": templar_settings,
         "aggregate_with_result_stats": {"kernel_with_stats_ms": round(aggs_ms, 4), "kernel_ms": round(aggk_ms, 4),
                                         "same_stats_by_torch_ms": round(stats_torch_ms, 4),
                                         "what": "per-parameter L2 norm, mean and all-finite flag of the decoded "
