@@ -513,6 +513,14 @@ def main():
         te_ms, _ = event_ms(lambda: tc.encode_compress_batch(b2, tk, use_dct=False, idx12=t_idx, val=t_val),
                             args.steps, args.warmup, settle=True)
         te_bytes = n_chunks * (16384 + 11 * tk // 2)
+        # the miner's whole step at these settings (src/tplr/neurons.py:147-171): momentum update + select, the 4-bin
+        # quantiser over the payload, the sent values subtracted at their k positions per chunk
+        t_efs = [torch.zeros_like(g) for g in g2]
+        t_eb = tc.TensorBatch(t_efs)
+        q4 = tc.TopKCompressor(use_quantization=True, quantization_bins=4, quantization_range=6)
+        tm_ms, tm_wall = event_ms(lambda: tc.error_feedback_step_batch(t_eb, b2, 0.95, tk, use_dct=False, compressor=q4),
+                                  max(3, args.steps // 4), 2)
+        del t_efs, t_eb
         t_win = tc.PayloadStage(batch, tk, tP, quantized=False)
         t_idxs, t_vals = [], []
         for p in range(tP):
@@ -530,6 +538,7 @@ def main():
                     "4-bin quantiser, 20 peers",
             "encode_ms": round(te_ms, 4), "encode_GBps": round(te_bytes / (te_ms * 1e-3) / 1e9, 2),
             "encode_frac_of_hbm_peak": round(te_bytes / (te_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "miner_step_ms": round(tm_ms, 4), "miner_step_wall_ms": round(tm_wall, 4),
             "aggregate": codes_figures(t_idxs, t_vals, tk),
         }
         del t_win, t_idxs, t_vals

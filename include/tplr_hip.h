@@ -265,6 +265,15 @@ int tplr_ef_encode_topk_pack_batch(const tplr_tensor_desc* d_ef_desc, const tplr
 int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, const tplr_tensor_desc* d_ef_desc,
                            int n_tensors, int64_t total_chunks, int use_dct, void* stream);
 
+/* tplr_ef_subtract_batch with use_dct == 0 for the step's own payload, i.e. d_idx12 and d_own as
+ * tplr_ef_encode_topk_pack_batch (use_dct = 0) has just written them from these very tensors: a selected
+ * position then holds the payload's own value, so ef - sent there is own - sent and the tensors are not read:
+ * ef[position] <- d_own - d_sent, entry by entry (d_sent: what the reference would decompress - d_own itself
+ * without a quantiser, the de-quantised values with one).  The same bits as tplr_ef_subtract_batch; every
+ * row must name each position once, as a top-k selection does.  k <= 64. */
+int tplr_ef_subtract_own_batch(const uint8_t* d_idx12, const float* d_sent, const float* d_own, int k,
+                               const tplr_tensor_desc* d_ef_desc, int n_tensors, int64_t total_chunks, void* stream);
+
 /* ---- validator side: checks on the packed index streams ------------------------------
  * For up to 32 peers whose flat payloads share one row layout (d_desc: n_tensors descriptors, of
  * which only chunk_begin, x_chunks and y_chunks are read; a parameter of n rows that are not

@@ -1136,8 +1136,13 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
             copied = torch.cuda.Event()
             copied.record()
     with _on(dev):
-        st = lib.tplr_ef_subtract_batch(_ptr(idx12), _ptr(sent), k, _ptr(ef.table), len(ef), n, int(use_dct),
-                                        _stream(dev))
+        if use_dct:
+            st = lib.tplr_ef_subtract_batch(_ptr(idx12), _ptr(sent), k, _ptr(ef.table), len(ef), n, 1, _stream(dev))
+        else:
+            # the payload was selected from these very tensors: a selected position holds the payload's own value,
+            # so the tensors need not be read (k scattered stores per chunk instead of k read-modify-writes)
+            st = lib.tplr_ef_subtract_own_batch(_ptr(idx12), _ptr(sent), _ptr(val), k, _ptr(ef.table), len(ef), n,
+                                                _stream(dev))
     _lib.check(st, "tplr_ef_subtract_batch")
     if codes is not None:
         # the per-parameter form of the reference's compress output

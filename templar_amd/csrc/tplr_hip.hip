@@ -1745,6 +1745,44 @@ __global__ __launch_bounds__(64) void k_ef_subtract_sparse(const uint8_t* __rest
     }
 }
 
+// The same for the miner's own step, where the payload was selected from this very tensor a launch ago
+// (tplr_ef_encode_topk_pack_batch without the transform): what stands at a selected position is the
+// payload's own value, bit for bit, so ef - sent there is own - sent and nothing has to be read from the
+// tensor - k scattered four-byte stores per chunk instead of k read-modify-writes.  `own` are the payload's
+// values as selected, `sent` what the reference would decompress (the same, or their de-quantised form).  A
+// top-k selection names every position once; the next chunk's entries are requested before this chunk's are
+// stored.
+__global__ __launch_bounds__(64) void k_ef_overwrite_sparse(const uint8_t* __restrict__ idx12,
+                                                            const float* __restrict__ sent,
+                                                            const float* __restrict__ own, int k,
+                                                            const tplr_tensor_desc* __restrict__ table,
+                                                            const tplr_tensor_desc single, int n_tensors,
+                                                            int64_t total) {
+    const int lane = threadIdx.x;
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
+    Cursor c;
+    cursor_seek(c, table, single, n_tensors, g0);
+    const int64_t idx_stride = k + (k >> 1);
+    const int le = lane < k ? lane : 0;
+    auto fetch = [&](int64_t g, uint32_t& me, float& x) {
+        me = load_idx12(idx12 + g * idx_stride, le);
+        x = own[g * k + le] - sent[g * k + le];
+    };
+    uint32_t me, me_next = 0;
+    float x, x_next = 0.f;
+    fetch(g0, me, x);
+    for (int64_t g = g0; g < g1; ++g) {
+        if (g + 1 < g1) fetch(g + 1, me_next, x_next);
+        gfloat* chunk0 = c.base + (c.y * 64) * c.ld + static_cast<int64_t>(c.xc) * 64;
+        if (lane < k) chunk0[static_cast<int64_t>(me >> 6) * c.ld + (me & 63)] = x;
+        me = me_next;
+        x = x_next;
+        if (g + 1 < g1) cursor_next(c, g + 1);
+    }
+}
+
 // -----------------------------------------------------------------------------------------
 // Statistics of the packed index streams of up to 32 peers, per tensor:
 //   pair[t][p][q] (p < q) = number of entries of peer p that also occur in the same row of peer q,
@@ -3265,6 +3303,22 @@ int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, co
     pp.val[0] = d_val;
     return launch_decode_as(k_decode_aggregate<true, 8, 4, true, true>, pp, nullptr, 1, k, d_ef_desc, none, n_tensors,
                             total_chunks, TPLR_REDUCE_MEAN, 0, nullptr, stream);
+}
+
+int tplr_ef_subtract_own_batch(const uint8_t* d_idx12, const float* d_sent, const float* d_own, int k,
+                               const tplr_tensor_desc* d_ef_desc, int n_tensors, int64_t total_chunks, void* stream) {
+    if (!d_idx12 || !d_sent || !d_own || !d_ef_desc || n_tensors < 1 || total_chunks < 0 || k < 2 || (k & 1))
+        return TPLR_E_BADARG;
+    if (k > 64) return TPLR_E_TOOMANY;
+    if (total_chunks == 0) return 0;
+    tplr_tensor_desc none = {};
+    static int resident = 0;
+    if (resident == 0) resident = persistent_grid(k_ef_overwrite_sparse, int64_t{1} << 40);
+    const int64_t need = ((total_chunks + 7) / 8) * 8;
+    hipLaunchKernelGGL(k_ef_overwrite_sparse, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), d_idx12, d_sent, d_own, k, d_ef_desc, none, n_tensors,
+                       total_chunks);
+    return launch_status();
 }
 
 static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_scale, int n_peers,

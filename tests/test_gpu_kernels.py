@@ -603,7 +603,8 @@ def test_batch_encode_and_aggregate_match_per_tensor(dev):
 
 
 # ---------------------------------------------------------------- miner side: error-feedback step
-@pytest.mark.parametrize("use_dct,k,bins", [(True, 32, 0), (True, 64, 0), (False, 32, 0), (True, 32, 4), (False, 64, 256)])
+@pytest.mark.parametrize("use_dct,k,bins", [(True, 32, 0), (True, 64, 0), (False, 32, 0), (True, 32, 4), (False, 64, 256),
+                                            (False, 64, 4), (False, 2, 0)])
 def test_error_feedback_step_matches_reference_sequence(dev, use_dct, k, bins):
     # three tensors of different shapes, walked as one batch (src/tplr/neurons.py:147-171 per parameter)
     shapes = [(128, 192), (64, 64), (256, 128)]
@@ -660,6 +661,38 @@ def test_error_feedback_null_round_and_equivalence_with_separate_calls(dev):
     idx12, val, _ = tc.error_feedback_step_batch(eb, gb, 0.9, 32, use_dct=True, null_round=True)
     assert float(d_ef.abs().max()) == 0.0 and float(val.abs().max()) == 0.0
     assert np.array_equal(orc.unpack12(idx12.cpu().numpy(), (6, 32))[0], np.arange(32))
+
+
+@pytest.mark.parametrize("k,bins", [(64, 4), (32, 0), (16, 256)])
+def test_own_payload_subtraction_writes_what_the_read_modify_write_leaves(dev, k, bins):
+    # without the transform the step's own payload is subtracted by k stores per chunk (own - sent) instead of k
+    # read-modify-writes (ef - sent): the same bits in every element, ragged shapes and strided tensors included
+    shapes = [(128, 192), (64, 64), (320, 128)]
+    big = torch.from_numpy(t3((320, 512), 5).numpy()).to(dev)
+    efs = [t3(shapes[0], 1, row_scale=True).to(dev), t3(shapes[1], 2).to(dev), big[:, 128:256]]  # the last one a strided view
+    grads = [t3(s, 10 + i, row_scale=True).to(dev) for i, s in enumerate(shapes)]
+    eb, gb = tc.TensorBatch(efs), tc.TensorBatch(grads)
+    n = eb.total_chunks
+    lib = _lib.load()
+    idx12 = torch.empty(n * (k // 2) * 3, dtype=torch.uint8, device=dev)
+    val = torch.empty((n, k), dtype=torch.float32, device=dev)
+    assert lib.tplr_ef_encode_topk_pack_batch(eb.table.data_ptr(), gb.table.data_ptr(), len(eb), n, 0.9, k, 0,
+                                              idx12.data_ptr(), val.data_ptr(), None) == 0
+    sent = val
+    if bins:
+        codes, shift, scale, lookup = tc.quantize_batch(eb, val, k, bins, 6.0)
+        sent = tc.dequantize_batch(eb, codes.reshape(-1), None, k, tables=(lookup, shift))
+    keep = [e.clone() for e in efs]
+    assert lib.tplr_ef_subtract_batch(idx12.data_ptr(), sent.data_ptr(), k, eb.table.data_ptr(), len(eb), n, 0, None) == 0
+    want = [e.clone() for e in efs]
+    for e, b in zip(efs, keep):
+        e.copy_(b)
+    assert lib.tplr_ef_subtract_own_batch(idx12.data_ptr(), sent.data_ptr(), val.data_ptr(), k, eb.table.data_ptr(),
+                                          len(eb), n, None) == 0
+    torch.cuda.synchronize()
+    for a, b in zip(efs, want):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    assert torch.equal(big[:, :128], torch.from_numpy(t3((320, 512), 5).numpy()).to(dev)[:, :128])  # neighbours of the view untouched
 
 
 # ---------------------------------------------------------------- validator side: index checks
