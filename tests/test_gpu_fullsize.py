@@ -469,3 +469,65 @@ def test_codes_aggregate_wave_ranges_of_a_few_chunks(dev, P, k, chunks_y):
                                          mean=mode == _lib.REDUCE_MEAN)
         for t, (a, b) in enumerate(zip(outs, want)):
             assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (mode, t)
+
+
+def test_codes_aggregate_seeded_sweep(dev):
+    # forty seeded draws of (peers, k, bins, set of shapes, staged or separately allocated payloads): the aggregate
+    # from codes bit for bit against the fp32 aggregate of the de-quantised values, both reduce modes; and the sums
+    # of squares from the payloads against those of the dense sum-mode coefficients
+    import ctypes as C
+    from templar_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(20251)
+    for draw in range(40):
+        P = int(rng.integers(1, 25))
+        k = int(rng.choice([4, 8, 16, 32, 64]))
+        bins = int(rng.choice([2, 3, 4]))
+        staged = bool(rng.integers(0, 2))
+        shapes = [(int(rng.integers(1, 40)) * 64, int(rng.integers(1, 40)) * 64) for _ in range(int(rng.integers(1, 4)))]
+        T = len(shapes)
+        n = sum((a // 64) * (b // 64) for a, b in shapes)
+        outs = [torch.empty(s, device=dev) for s in shapes]
+        want = [torch.empty(s, device=dev) for s in shapes]
+        batch = tc.TensorBatch(outs)
+        packed, vals = _random_payloads(dev, n, P, k, 7000 + draw)
+        qps = [[None] * P for _ in range(T)]
+        fp32, codes = [], []
+        for p in range(P):
+            c, shift, scale, lookup = tc.quantize_batch(batch, vals[p], k, bins, 6.0)
+            codes.append(c)
+            fp32.append(tc.dequantize_batch(batch, c.reshape(-1), None, k, tables=(lookup, shift)))
+            for i in range(T):
+                qps[i][p] = (shift[i], 1.0, bins // 2, lookup[i], torch.float32)
+        if staged:
+            ibuf, cbuf = torch.stack(packed), torch.stack(codes)
+            packed, codes = [ibuf[p] for p in range(P)], [cbuf[p] for p in range(P)]
+        deq, _ = tc.dequantised_tables(qps, dev)
+        g = torch.Generator(device=dev)
+        g.manual_seed(draw)
+        scale = torch.rand((T, P), device=dev, generator=g) * 0.5 + 0.5
+        ip = (C.c_void_p * P)(*[i.data_ptr() for i in packed])
+        cp = (C.c_void_p * P)(*[c.data_ptr() for c in codes])
+        for mode in (_lib.REDUCE_MEAN, _lib.REDUCE_SUM):
+            for o in outs:
+                o.fill_(float("nan"))
+            st = lib.tplr_decode_aggregate_codes_batch(ip, cp, deq.data_ptr(), scale.data_ptr(), P, k,
+                                                       batch.table.data_ptr(), T, n, mode, None, None)
+            assert st == 0, (draw, st)
+            tc.batch_decompress_decode_batch(tc.TensorBatch(want), packed, fp32, k, scale=scale, use_dct=False,
+                                             mean=mode == _lib.REDUCE_MEAN)
+            for t, (a, b) in enumerate(zip(outs, want)):
+                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (draw, P, k, bins, staged, mode, t)
+        # `want` now holds the sum-mode coefficients (no transform): their sums of squares per chunk
+        ss = torch.empty(n, device=dev)
+        vp = (C.c_void_p * P)(*[v.data_ptr() for v in fp32])
+        assert lib.tplr_aggregate_sumsq_batch(ip, vp, scale.data_ptr(), P, k, batch.table.data_ptr(), T, n,
+                                              ss.data_ptr(), None) == 0
+        b0 = 0
+        for t, s in enumerate(shapes):
+            Y, X = s[0] // 64, s[1] // 64
+            d = want[t].double().reshape(Y, 64, X, 64).permute(0, 2, 1, 3).reshape(Y * X, 4096)
+            ref = (d * d).sum(dim=1)
+            got = ss[b0:b0 + Y * X].double()
+            assert float((got - ref).abs().max()) <= 1e-5 * float(ref.max()), (draw, t)
+            b0 += Y * X
