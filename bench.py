@@ -296,6 +296,12 @@ def main():
         k2 = lambda: _lib_mod.check(lib.tplr_ef_subtract_batch(  # noqa: E731
             idx_buf.data_ptr(), val_buf.data_ptr(), k, eb.table.data_ptr(), len(eb), n_chunks, 1, st), "ef_subtract")
         both = lambda: (k1(), k2())  # noqa: E731
+        fused_ms = None
+        if DCT:
+            kf = lambda: _lib_mod.check(lib.tplr_ef_step_batch(  # noqa: E731
+                eb.table.data_ptr(), batch.table.data_ptr(), len(eb), n_chunks, 0.95, k, idx_buf.data_ptr(),
+                val_buf.data_ptr(), st), "ef_step")
+            fused_ms, _ = event_ms(kf, steps, warmup)
         ms_both, _ = event_ms(both, steps, warmup)
         ms1, _ = event_ms(k1, steps, 1)
         ms2, _ = event_ms(k2, steps, 1)
@@ -313,6 +319,11 @@ def main():
             "update_encode_ms": round(ms1, 4), "update_encode_bytes": b1,
             "subtract_decoded_ms": round(ms2, 4), "subtract_decoded_bytes": b2,
             "with_4bin_quantiser_wall_ms": round(ms_q, 4),
+            "one_launch_ms": None if fused_ms is None else round(fused_ms, 4),
+            "one_launch_bytes": n_chunks * (2 * 16384 + 16384 + 11 * k // 2),
+            "one_launch_what": "the same step where no quantiser sits between its halves: update, transform, select, payload "
+                               "and subtraction of the payload's reconstruction in one launch, every chunk read once and "
+                               "written once",
         }
 
     # ---- P peers' flat payloads for the aggregation side (peer p = 0.5 shared + own); built before anything is

@@ -274,6 +274,13 @@ int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, co
 int tplr_ef_subtract_own_batch(const uint8_t* d_idx12, const float* d_sent, const float* d_own, int k,
                                const tplr_tensor_desc* d_ef_desc, int n_tensors, int64_t total_chunks, void* stream);
 
+/* Both launches in one where nothing sits between them (no quantiser) and the chunks are transformed:
+ * tplr_ef_encode_topk_pack_batch (use_dct = 1) followed by tplr_ef_subtract_batch (use_dct = 1) on the payload
+ * it wrote - the same payload and the same tensors, bit for bit - with every chunk of the error-feedback
+ * tensors read once and written once.  k even, 2 <= k <= 64. */
+int tplr_ef_step_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc* d_grad_desc, int n_tensors,
+                       int64_t total_chunks, float decay, int k, uint8_t* d_idx12, float* d_val, void* stream);
+
 /* ---- validator side: checks on the packed index streams ------------------------------
  * For up to 32 peers whose flat payloads share one row layout (d_desc: n_tensors descriptors, of
  * which only chunk_begin, x_chunks and y_chunks are read; a parameter of n rows that are not

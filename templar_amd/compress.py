@@ -1110,6 +1110,14 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
     dev, n = ef.device, ef.total_chunks
     idx12 = torch.empty(n * (k // 2) * 3, dtype=torch.uint8, device=dev)
     val = torch.empty((n, k), dtype=torch.float32, device=dev)
+    quantises = compressor is not None and compressor.use_quantization
+    if use_dct and not quantises and not null_round:
+        # nothing sits between the two halves of the step: one launch, every chunk read once and written once
+        with _on(dev):
+            st = lib.tplr_ef_step_batch(_ptr(ef.table), _ptr(grad.table), len(ef), n, C.c_float(decay), k, _ptr(idx12),
+                                        _ptr(val), _stream(dev))
+        _lib.check(st, "tplr_ef_step_batch")
+        return idx12, val, None
     with _on(dev):
         if null_round:
             for t in ef.tensors:

@@ -1691,6 +1691,69 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     redo_marked();
 }
 
+// The miner's whole error-feedback step for one chunk in one pass, where no quantiser sits between its two
+// halves (src/tplr/neurons.py:147-171): ef * decay + grad, the transform, top-k, the payload, and at once the
+// subtraction of that payload's reconstruction - what tplr_ef_encode_topk_pack_batch followed by
+// tplr_ef_subtract_batch leave, bit for bit, with the tensor read once and written once (48 KB of traffic per
+// chunk instead of 81 KB).  The updated chunk stays in 64 registers while it is transformed and selected from;
+// the k selected values go back into a cleared tile exactly as the one-peer decode adds them (0 + value * 2^-5),
+// through the inverse transform, and the difference is stored.  Two waves per SIMD (a whole tile, 64 more
+// registers): the launch moves 14 GB and is bound by that.
+template <bool kTwo>
+__global__ __launch_bounds__(64, 2) void k_ef_step(const tplr_tensor_desc* __restrict__ table,
+                                                   const tplr_tensor_desc* __restrict__ grad_table, int n_tensors,
+                                                   int64_t total, int k, float decay, uint8_t* __restrict__ idx12,
+                                                   float* __restrict__ val) {
+    __shared__ __align__(16) float tile[kTileFloats];
+    __shared__ uint64_t cand[kCandCap];
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
+    Cursor c, cg;
+    tplr_tensor_desc none = {};
+    cursor_seek(c, table, none, n_tensors, g0);
+    cursor_seek(cg, grad_table, none, n_tensors, g0);
+    for (int64_t g = g0; g < g1; ++g) {
+        // (lane-derived addresses are formed per chunk from a copy of the lane id the optimiser cannot see
+        // through: hoisted out of the loop they would be spilled)
+        int lane = threadIdx.x;
+        asm volatile("" : "+v"(lane));
+        float e[64], v[64], w[64];
+        load_chunk_cols(e, c, lane);
+        load_chunk_cols(w, cg, lane);
+#pragma unroll
+        for (int r = 0; r < 64; ++r) {
+            const float m = e[r] * decay;
+            e[r] = m + w[r];
+            v[r] = e[r];
+        }
+        gfloat* const dst = c.base + (c.y * 64) * c.ld + static_cast<int64_t>(c.xc) * 64;
+        const int64_t ld = c.ld;
+        if (g + 1 < g1) {
+            cursor_next(cg, g + 1);
+            cursor_next(c, g + 1);
+        }
+        chunk_forward<true>(v, w, tile, lane);
+        const Selected s = select_topk<kTwo, false>(w, tile, cand, lane, k, kDctPow2Scale, 0, 0);
+        emit_selected<kTwo>(s, lane, k, g, idx12, val);
+        // the payload's reconstruction
+        {
+            const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+            float4* row = reinterpret_cast<float4*>(tile + lane * kLd);
+#pragma unroll
+            for (int q = 0; q < 16; ++q) row[q] = z;
+        }
+        wave_lds_fence();
+        if (lane < k) tile[tile_pos(s.idx0)] = 0.0f + s.val0 * kDctPow2Scale;
+        wave_lds_fence();
+        chunk_inverse<true>(v, tile, lane);
+        wave_lds_fence();
+#pragma unroll
+        for (int r = 0; r < 64; ++r) v[r] = e[r] - v[r];
+        store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(dst)), uniform64(ld), lane);
+    }
+}
+
 // ef <- ef - (the payload's entries) for chunks that are not transformed (use_dct = 0): the
 // reconstruction is the payload itself, so only k elements per chunk change
 // (src/tplr/neurons.py:162-171 with decode a pure re-layout).  k <= 64: one entry per lane.  What
@@ -3280,6 +3343,29 @@ int tplr_ef_encode_topk_pack_batch(const tplr_tensor_desc* d_ef_desc, const tplr
                                 d_idx12, d_val, stream, d_grad_desc, decay);
     return launch_encode_as(k_encode_topk_pack<false, false, true>, d_ef_desc, none, n_tensors, total_chunks, k,
                             d_idx12, d_val, stream, d_grad_desc, decay);
+}
+
+int tplr_ef_step_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc* d_grad_desc, int n_tensors,
+                       int64_t total_chunks, float decay, int k, uint8_t* d_idx12, float* d_val, void* stream) {
+    if (!d_ef_desc || !d_grad_desc || n_tensors < 1 || total_chunks < 0 || !d_idx12 || !d_val || k < 2 || (k & 1))
+        return TPLR_E_BADARG;
+    if (k > 64) return TPLR_E_TOOMANY;
+    if (total_chunks == 0) return 0;
+    const int64_t need = ((total_chunks + 7) / 8) * 8;
+    if (k > 32) {
+        static int resident = 0;
+        if (resident == 0) resident = persistent_grid(k_ef_step<true>, int64_t{1} << 40);
+        hipLaunchKernelGGL(k_ef_step<true>, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+                           static_cast<hipStream_t>(stream), d_ef_desc, d_grad_desc, n_tensors, total_chunks, k, decay,
+                           d_idx12, d_val);
+    } else {
+        static int resident = 0;
+        if (resident == 0) resident = persistent_grid(k_ef_step<false>, int64_t{1} << 40);
+        hipLaunchKernelGGL(k_ef_step<false>, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+                           static_cast<hipStream_t>(stream), d_ef_desc, d_grad_desc, n_tensors, total_chunks, k, decay,
+                           d_idx12, d_val);
+    }
+    return launch_status();
 }
 
 int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, const tplr_tensor_desc* d_ef_desc,

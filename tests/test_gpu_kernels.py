@@ -663,6 +663,43 @@ def test_error_feedback_null_round_and_equivalence_with_separate_calls(dev):
     assert np.array_equal(orc.unpack12(idx12.cpu().numpy(), (6, 32))[0], np.arange(32))
 
 
+@pytest.mark.parametrize("k", [2, 32, 34, 64])
+def test_error_feedback_step_in_one_launch_equals_its_two_launches(dev, k):
+    # tplr_ef_step_batch (update, transform, select, payload, subtraction of the payload's reconstruction, every chunk
+    # read once and written once) against tplr_ef_encode_topk_pack_batch followed by tplr_ef_subtract_batch: the same
+    # payload and the same tensors bit for bit; ragged shapes and a strided view whose neighbours stay untouched
+    shapes = [(128, 192), (64, 64), (320, 128)]
+    base = t3((320, 512), 5)
+    def fresh():
+        big = base.clone().to(dev)
+        return big, [t3(shapes[0], 1, row_scale=True).to(dev), t3(shapes[1], 2).to(dev), big[:, 128:256]]
+    grads = [t3(s, 10 + i, row_scale=True).to(dev) for i, s in enumerate(shapes)]
+    gb = tc.TensorBatch(grads)
+    lib = _lib.load()
+    res = []
+    for fused in (False, True):
+        big, efs = fresh()
+        eb = tc.TensorBatch(efs)
+        n = eb.total_chunks
+        idx12 = torch.full((n * (k // 2) * 3,), 255, dtype=torch.uint8, device=dev)
+        val = torch.full((n, k), float("nan"), device=dev)
+        if fused:
+            assert lib.tplr_ef_step_batch(eb.table.data_ptr(), gb.table.data_ptr(), len(eb), n, 0.9, k, idx12.data_ptr(),
+                                          val.data_ptr(), None) == 0
+        else:
+            assert lib.tplr_ef_encode_topk_pack_batch(eb.table.data_ptr(), gb.table.data_ptr(), len(eb), n, 0.9, k, 1,
+                                                      idx12.data_ptr(), val.data_ptr(), None) == 0
+            assert lib.tplr_ef_subtract_batch(idx12.data_ptr(), val.data_ptr(), k, eb.table.data_ptr(), len(eb), n, 1,
+                                              None) == 0
+        torch.cuda.synchronize()
+        res.append((idx12, val, [e.clone() for e in efs], big))
+    (i0, v0, e0, b0), (i1, v1, e1, b1) = res
+    assert torch.equal(i0, i1) and torch.equal(v0.view(torch.int32), v1.view(torch.int32))
+    for a, b in zip(e0, e1):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    assert torch.equal(b1[:, :128], base.to(dev)[:, :128]) and torch.equal(b1[:, 256:], base.to(dev)[:, 256:])
+
+
 @pytest.mark.parametrize("k,bins", [(64, 4), (32, 0), (16, 256)])
 def test_own_payload_subtraction_writes_what_the_read_modify_write_leaves(dev, k, bins):
     # without the transform the step's own payload is subtracted by k stores per chunk (own - sent) instead of k
