@@ -349,6 +349,12 @@ int tplr_decode_aggregate_codes_batch(const uint8_t* const* h_idx12, const uint8
                                       const float* d_scale, int n_peers, int k, const tplr_tensor_desc* d_desc,
                                       int n_tensors, int64_t total_chunks, int reduce_mode, float* d_sumsq,
                                       void* stream);
+/* tplr_decode_aggregate_codes_batch with the per-parameter statistics of tplr_decode_aggregate_stats_batch
+ * (d_chunk_stats: 2 * total_chunks floats of scratch; d_tensor_stats: 4 floats per tensor). */
+int tplr_decode_aggregate_codes_stats_batch(const uint8_t* const* h_idx12, const uint8_t* const* h_codes,
+                                            const float* d_deq, const float* d_scale, int n_peers, int k,
+                                            const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks,
+                                            int reduce_mode, float* d_chunk_stats, float* d_tensor_stats, void* stream);
 
 /* tplr_decode_aggregate_batch together with what its caller looks at next, per parameter
  * (src/tplr/neurons.py:380-385: L2 norm and mean of the decoded gradient for the fingerprint; :411 and

@@ -41,6 +41,7 @@ SIGNATURES = {
     "tplr_decode_aggregate_stats_batch": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp]),
     "tplr_code_sumsq": (_i32, [_vp, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp]),
     "tplr_decode_aggregate_codes_batch": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _i32, _vp, _vp]),
+    "tplr_decode_aggregate_codes_stats_batch": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _i32, _vp, _vp, _vp]),
     "tplr_segment_sumsq": (_i32, [_vp, _i32, _i32, _vp, _i32, _i32, _vp, _vp]),
     "tplr_clip_scales_batch": (_i32, [_vp, _i32, _i32, _i32, _vp, _vp, _vp]),
     "tplr_decode_aggregate": (_i32, [_vp, _vp, _vp, _i32, _i32, _i64, _i64, _i32, _i32, _i32, _vp, _i64, _vp, _vp]),

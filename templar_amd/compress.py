@@ -1472,7 +1472,8 @@ def batch_decompress_decode_codes_batch(out: TensorBatch, idxs: Sequence[torch.T
                                         quant_params: Sequence[Sequence[QuantParamsT]], k: int, *,
                                         clip_norm: bool = True, use_dct: bool = False, mean: bool = True,
                                         validate: bool = True,
-                                        tables: "tuple[torch.Tensor, int] | None" = None) -> None:
+                                        tables: "tuple[torch.Tensor, int] | None" = None,
+                                        stats: bool = False) -> "torch.Tensor | None":
     """maybe_dequantize_values + block norms + batch_decompress + decode of every parameter
     (src/tplr/neurons.py:325-367) from the peers' QUANTISED flat payloads: codes[p] holds peer p's one-byte
     codes (total_chunks * k), quant_params[i][p] parameter i's 5-tuple from peer p.  With templar's settings - a
@@ -1482,7 +1483,8 @@ def batch_decompress_decode_codes_batch(out: TensorBatch, idxs: Sequence[torch.T
     fp32 path: the same results either way.  `validate` raises on a code the quantiser cannot have produced,
     as the reference's table lookup does, at the cost of a synchronisation.  `tables` = what
     dequantised_tables(quant_params, device) returns, for callers that build it once per window (a few thousand
-    small tensors are stacked to make it)."""
+    small tensors are stacked to make it).  stats=True returns the (T, 4) statistics of the decoded parameters
+    as batch_decompress_decode_batch does."""
     lib = _lib.load()
     P, T, n, dev = len(codes), len(out), out.total_chunks, out.device
     if tables is None and (len(quant_params) != T or any(len(q) != P for q in quant_params)):
@@ -1497,8 +1499,7 @@ def batch_decompress_decode_codes_batch(out: TensorBatch, idxs: Sequence[torch.T
         vals = []
         for p in range(P):
             vals.append(dequantize_batch(out, codes[p].reshape(-1), [quant_params[i][p] for i in range(T)], k))
-        batch_decompress_decode_batch(out, idxs, vals, k, clip_norm=clip_norm, use_dct=use_dct, mean=mean)
-        return
+        return batch_decompress_decode_batch(out, idxs, vals, k, clip_norm=clip_norm, use_dct=use_dct, mean=mean, stats=stats)
     deq, n_bins = tables if tables is not None else dequantised_tables(quant_params, dev)
     if deq.shape != (T, P, 4) or deq.dtype != torch.float32 or not deq.is_contiguous():
         raise ValueError(f"tables: expected a contiguous fp32 ({T}, {P}, 4) tensor, got {tuple(deq.shape)}")
@@ -1520,9 +1521,18 @@ def batch_decompress_decode_codes_batch(out: TensorBatch, idxs: Sequence[torch.T
             worst = int(bad.item())
             if worst:
                 raise IndexError(f"index {worst} is out of bounds for dimension 0 with size {n_bins}")
+        if stats:
+            per_chunk = torch.empty((max(n, 1), 2), dtype=torch.float32, device=dev)
+            per_tensor = torch.empty((T, 4), dtype=torch.float32, device=dev)
+            st = lib.tplr_decode_aggregate_codes_stats_batch(ip, cp, _ptr(deq), _ptr(scale), P, k, _ptr(out.table), T, n,
+                                                             _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM,
+                                                             _ptr(per_chunk), _ptr(per_tensor), _stream(dev))
+            _lib.check(st, "tplr_decode_aggregate_codes_stats_batch")
+            return per_tensor
         st = lib.tplr_decode_aggregate_codes_batch(ip, cp, _ptr(deq), _ptr(scale), P, k, _ptr(out.table), T, n,
                                                    _lib.REDUCE_MEAN if mean else _lib.REDUCE_SUM, None, _stream(dev))
     _lib.check(st, "tplr_decode_aggregate_codes_batch")
+    return None
 
 
 class PayloadStage:

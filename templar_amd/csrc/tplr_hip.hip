@@ -3541,6 +3541,24 @@ int tplr_decode_aggregate_codes_batch(const uint8_t* const* h_idx12, const uint8
                          n_tensors, total_chunks, reduce_mode, 0, 0, d_sumsq, stream, d_deq);
 }
 
+int tplr_decode_aggregate_codes_stats_batch(const uint8_t* const* h_idx12, const uint8_t* const* h_codes,
+                                            const float* d_deq, const float* d_scale, int n_peers, int k,
+                                            const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks,
+                                            int reduce_mode, float* d_chunk_stats, float* d_tensor_stats, void* stream) {
+    if (int s = check_decode(h_idx12, h_codes, n_peers, k, reduce_mode)) return s;
+    if (!d_desc || !d_deq || !d_chunk_stats || !d_tensor_stats || n_tensors < 1 || total_chunks < 0) return TPLR_E_BADARG;
+    if (k > 64 || n_peers > 24) return TPLR_E_TOOMANY;
+    if (total_chunks > 0) {
+        tplr_tensor_desc none = {};
+        if (int s = launch_decode(h_idx12, reinterpret_cast<const float* const*>(h_codes), d_scale, n_peers, k, d_desc, none,
+                                  n_tensors, total_chunks, reduce_mode, 2, 0, d_chunk_stats, stream, d_deq))
+            return s;
+    }
+    hipLaunchKernelGGL(k_tensor_stats, dim3(static_cast<unsigned>(n_tensors)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), d_chunk_stats, d_desc, 0, d_tensor_stats);
+    return launch_status();
+}
+
 int tplr_code_sumsq(const uint8_t* const* h_codes, int n_peers, int k, const tplr_tensor_desc* d_desc, int n_tensors,
                     int n_slices, int n_bins, const float* d_deq, float* d_sumsq, int32_t* d_bad, void* stream) {
     if (!h_codes || !d_desc || !d_deq || !d_sumsq || n_peers < 1 || n_tensors < 1 || k < 2 || (k & 1) || n_slices < 1 ||

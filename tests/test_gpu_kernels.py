@@ -1316,6 +1316,14 @@ def test_aggregate_straight_from_four_bin_codes_equals_dequantise_then_aggregate
         ref = orc.batch_decompress(ti, tv, (1, cnt, 64, 64), 4096).reshape(Y, X, 64, 64).transpose(0, 2, 1, 3)
         assert relerr(got[t].cpu().numpy(), ref.reshape(shapes[t])) <= TOL, t
         b0 += cnt
+    # with the statistics of the decoded parameters: the same tensors, their norms, means and finiteness
+    st_out = [torch.full(s, 7.0, device=dev) for s in shapes]
+    stt = tc.batch_decompress_decode_codes_batch(tc.TensorBatch(st_out), di, codes, qps, k, stats=True).cpu().numpy()
+    for t, (a, b) in enumerate(zip(st_out, got)):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+        d = a.double()
+        assert abs(stt[t, 0] - float(torch.linalg.vector_norm(d))) <= 1e-5 * float(torch.linalg.vector_norm(d))
+        assert abs(stt[t, 1] - float(d.mean())) <= 1e-5 * float(d.abs().mean()) and stt[t, 2] == 1.0
     # a stage that keeps the codes hands them and its tables to the same call
     stage = tc.PayloadStage(batch, k, P, quantized=True)
     per_i = [[batch.payload_slice(i, di[p], fp32[p], k)[0].cpu() for p in range(P)] for i in range(T)]
