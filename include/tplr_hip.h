@@ -359,7 +359,7 @@ int tplr_decode_aggregate_codes_stats_batch(const uint8_t* const* h_idx12, const
 /* tplr_decode_aggregate_batch together with what its caller looks at next, per parameter
  * (src/tplr/neurons.py:380-385: L2 norm and mean of the decoded gradient for the fingerprint; :411 and
  * :438: the parameter is skipped unless every element is finite), without another pass over the dense
- * tensors: the aggregate leaves two floats per chunk in d_chunk_stats (2 * total_chunks floats: sum of
+ * tensors: the aggregate leaves two floats per chunk in d_chunk_stats (2 * total_chunks floats, 8-byte aligned: sum of
  * squares and sum of the chunk's 4096 results) and one small launch turns them into
  * d_tensor_stats[4 t .. 4 t + 3] = {L2 norm, mean, 1.0 if every element is finite else 0.0, sum of squares}.
  * The flag is exact: a chunk whose figures are not finite is read back and examined element by element

@@ -1496,6 +1496,8 @@ def batch_decompress_decode_codes_batch(out: TensorBatch, idxs: Sequence[torch.T
             raise RuntimeError(f"flat payload mismatch: {i.numel()} index bytes / {c.numel()} codes for {n} chunks, k={k}")
     n_bins = int(tables[1]) if tables is not None else int(quant_params[0][0][3].numel())
     if n_bins > 4 or use_dct or k > _CH or P > 24:
+        if quant_params is None:
+            raise ValueError("these settings de-quantise first: pass quant_params, not only `tables`")
         vals = []
         for p in range(P):
             vals.append(dequantize_batch(out, codes[p].reshape(-1), [quant_params[i][p] for i in range(T)], k))
