@@ -471,6 +471,31 @@ def main():
         stats = {"what": f"pairwise index overlap + repeats + bounds of {P} peers' packed indices, one launch",
                  "ms": round(st_ms, 4), "GBps": round(st_bytes / (st_ms * 1e-3) / 1e9, 2), "bytes": st_bytes}
 
+    # the validator's per-peer evaluation update (neurons/validator.py:3595-3737): one peer's payload times its clip
+    # factor, decompress, decode, p.data.sub_(decoded, alpha) - one launch that reads and writes every parameter once,
+    # against decode into a dense gradient followed by the subtraction over the set
+    evaluation = None
+    if k <= 64:
+        params = [torch.zeros_like(o) for o in outs]
+        pb = tc.TensorBatch(params)
+        clip0 = scale.reshape(len(out_batch), -1)[:, 0].contiguous()
+        ev_ms, _ = event_ms(lambda: tc.apply_decoded_batch(pb, idxs[0], vals[0], k, alpha=0.01, clip=clip0, use_dct=DCT),
+                            agg_steps, 2)
+
+        def decode_then_subtract():
+            tc.batch_decompress_decode_batch(out_batch, idxs[:1], vals[:1], k, scale=clip0.reshape(-1, 1), use_dct=DCT)
+            torch._foreach_sub_(params, outs, alpha=0.01)
+
+        ev2_ms, _ = event_ms(decode_then_subtract, agg_steps, 1)
+        ev_bytes = n_chunks * (11 * k // 2 + (2 * 16384 if DCT else 8 * k))
+        evaluation = {"what": "one peer's payload applied to the parameters (values x clip factor, decompress, decode, "
+                              "p -= alpha * decoded) in one launch over the set, against decode into a dense gradient and "
+                              "a foreach subtraction; bytes: the payload + every chunk read and written (with the "
+                              "transform) or k elements per chunk read and written (without)",
+                      "ms": round(ev_ms, 4), "bytes": ev_bytes, "GBps": round(ev_bytes / (ev_ms * 1e-3) / 1e9, 2),
+                      "decode_then_subtract_ms": round(ev2_ms, 4)}
+        del params, pb
+
     # templar's own settings carry the values as the codes of a four-bin quantiser: the aggregate straight from
     # the codes against de-quantising every peer first (what outer_step does, src/tplr/neurons.py:325-364)
     def codes_figures(idxs_, vals_, kk):
@@ -648,6 +673,8 @@ def main():
         result["error_feedback_step"] = miner
     if stats is not None:
         result["index_stats"] = stats
+    if evaluation is not None:
+        result["evaluation_update"] = evaluation
     if staging is not None:
         result["payload_staging"] = staging
     if not args.no_cpu_baseline:

@@ -281,6 +281,17 @@ int tplr_ef_subtract_own_batch(const uint8_t* d_idx12, const float* d_sent, cons
 int tplr_ef_step_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc* d_grad_desc, int n_tensors,
                        int64_t total_chunks, float decay, int k, uint8_t* d_idx12, float* d_val, void* stream);
 
+/* The validator's per-peer evaluation update (neurons/validator.py:3595-3737, update_model_with_gradient): per
+ * parameter, the evaluated peer's values times its clip factor, decompress, decode, and
+ * p.data.sub_(decoded, alpha = lr * eval_lr_factor) - here one launch over the whole set that reads and writes
+ * every parameter once and never holds the dense gradient: param <- param - decode(decompress(payload)), every
+ * value of tensor t times d_factor[t] first (pass alpha * clip factor; the transform is linear, so this differs
+ * from scaling the decoded tensor by rounding only; NULL = 1).  The kernels are those of
+ * tplr_ef_subtract_batch; k <= 64; repeated indices in a row as in decompress (the mean of those entries). */
+int tplr_apply_decoded_batch(const uint8_t* d_idx12, const float* d_val, const float* d_factor, int k,
+                             const tplr_tensor_desc* d_param_desc, int n_tensors, int64_t total_chunks, int use_dct,
+                             void* stream);
+
 /* ---- validator side: checks on the packed index streams ------------------------------
  * For up to 32 peers whose flat payloads share one row layout (d_desc: n_tensors descriptors, of
  * which only chunk_begin, x_chunks and y_chunks are read; a parameter of n rows that are not

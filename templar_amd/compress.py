@@ -1087,6 +1087,36 @@ def aggregate_mean_normalised_batch(out: TensorBatch, idxs: Sequence[torch.Tenso
 
 
 @torch.no_grad()
+def apply_decoded_batch(params: TensorBatch, idx12: torch.Tensor, val: torch.Tensor, k: int, *, alpha: float = 1.0,
+                        clip: torch.Tensor | None = None, use_dct: bool = True) -> None:
+    """param <- param - alpha * decode(decompress(payload * clip)) for every parameter of the set in one launch:
+    the validator's per-peer evaluation update (neurons/validator.py:3595-3737, update_model_with_gradient: the
+    evaluated peer's values times its clip factor, decompress, decode, p.data.sub_(decoded, alpha=lr *
+    eval_lr_factor)).  `idx12`, `val`: that peer's flat payload (de-quantised values); `clip`: (T,) factors
+    min(1, median_t / (norm_t + 1e-8)) or None.  alpha and clip ride on the values (the transform is linear), so
+    the dense gradient is never formed and every parameter is read and written once.  k <= 64."""
+    lib = _lib.load()
+    T, n, dev = len(params), params.total_chunks, params.device
+    if idx12.dtype != torch.uint8:
+        raise ValueError(f"Expected uint8 for 12-bit packed indices, got {idx12.dtype}")
+    if val.dtype != torch.float32 or val.numel() != n * k or idx12.numel() * 2 != n * k * 3 or not val.is_contiguous():
+        raise RuntimeError(f"flat payload mismatch: {idx12.numel()} index bytes / {val.numel()} values for {n} chunks, k={k}")
+    if k > _CH:
+        raise NotImplementedError(f"top-{k}: the fused update handles k up to {_CH}")
+    factor = None
+    if clip is not None or alpha != 1.0:
+        factor = torch.full((T,), float(alpha), dtype=torch.float32, device=dev)
+        if clip is not None:
+            if clip.numel() != T:
+                raise IndexError(f"{clip.numel()} clip factors for {T} parameters")
+            factor = factor * clip.to(device=dev, dtype=torch.float32).reshape(T)
+    with _on(dev):
+        st = lib.tplr_apply_decoded_batch(_ptr(idx12), _ptr(val), _ptr(factor), k, _ptr(params.table), T, n, int(use_dct),
+                                          _stream(dev))
+    _lib.check(st, "tplr_apply_decoded_batch")
+
+
+@torch.no_grad()
 def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, topk: int, *, use_dct: bool = True,
                               compressor: "TopKCompressor | None" = None, null_round: bool = False):
     """The miner's per-parameter loop of src/tplr/neurons.py:147-171 for a whole set of 2-D
@@ -1770,6 +1800,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "apply_decoded_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

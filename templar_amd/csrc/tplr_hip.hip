@@ -1764,7 +1764,8 @@ __global__ __launch_bounds__(64) void k_ef_subtract_sparse(const uint8_t* __rest
                                                            const float* __restrict__ val, int k,
                                                            const tplr_tensor_desc* __restrict__ table,
                                                            const tplr_tensor_desc single, int n_tensors,
-                                                           int64_t total) {
+                                                           int64_t total, const float* __restrict__ factor) {
+    // factor (nullable): every value of tensor t times factor[t] before it is subtracted
     __shared__ uint16_t owner[4096];  // the last lane that named a position (never cleared: written before read)
     const int lane = threadIdx.x;
     int64_t g0, g1;
@@ -1780,6 +1781,10 @@ __global__ __launch_bounds__(64) void k_ef_subtract_sparse(const uint8_t* __rest
         if (lane < k) {
             me = static_cast<int>(load_idx12(idx12 + g * idx_stride, lane));
             x = val[g * k + lane];
+            if (factor) {
+                x *= factor[c.t];
+                asm volatile("" : "+v"(x));  // a product of its own rounding, never contracted into the subtraction
+            }
             owner[me] = static_cast<uint16_t>(lane);
         }
         wave_lds_fence();
@@ -3368,9 +3373,11 @@ int tplr_ef_step_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc
     return launch_status();
 }
 
-int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, const tplr_tensor_desc* d_ef_desc,
-                           int n_tensors, int64_t total_chunks, int use_dct, void* stream) {
-    if (!d_idx12 || !d_val || !d_ef_desc || n_tensors < 1 || total_chunks < 0 || k < 2 || (k & 1)) return TPLR_E_BADARG;
+// dst <- dst - decode(decompress(payload)), every value of tensor t times d_factor[t] first (d_factor nullable)
+static int subtract_decoded(const uint8_t* d_idx12, const float* d_val, const float* d_factor, int k,
+                            const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, int use_dct,
+                            void* stream) {
+    if (!d_idx12 || !d_val || !d_desc || n_tensors < 1 || total_chunks < 0 || k < 2 || (k & 1)) return TPLR_E_BADARG;
     if (k > 64) return TPLR_E_TOOMANY;  // the register-resident decode path
     if (total_chunks == 0) return 0;
     tplr_tensor_desc none = {};
@@ -3379,16 +3386,28 @@ int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, co
         if (resident == 0) resident = persistent_grid(k_ef_subtract_sparse, int64_t{1} << 40);
         const int64_t need = ((total_chunks + 7) / 8) * 8;
         hipLaunchKernelGGL(k_ef_subtract_sparse, dim3(static_cast<unsigned>(need < resident ? need : resident)),
-                           dim3(64), 0, static_cast<hipStream_t>(stream), d_idx12, d_val, k, d_ef_desc, none, n_tensors,
-                           total_chunks);
+                           dim3(64), 0, static_cast<hipStream_t>(stream), d_idx12, d_val, k, d_desc, none, n_tensors,
+                           total_chunks, d_factor);
         return launch_status();
     }
     PeerPtrs pp;
     for (int p = 0; p < TPLR_MAX_PEERS; ++p) pp.idx[p] = nullptr, pp.val[p] = nullptr;
     pp.idx[0] = d_idx12;
     pp.val[0] = d_val;
-    return launch_decode_as(k_decode_aggregate<true, 8, 4, true, true>, pp, nullptr, 1, k, d_ef_desc, none, n_tensors,
+    // (one peer: the factor table (n_tensors, 1) is the aggregate's clip-factor table)
+    return launch_decode_as(k_decode_aggregate<true, 8, 4, true, true>, pp, d_factor, 1, k, d_desc, none, n_tensors,
                             total_chunks, TPLR_REDUCE_MEAN, 0, nullptr, stream);
+}
+
+int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, const tplr_tensor_desc* d_ef_desc,
+                           int n_tensors, int64_t total_chunks, int use_dct, void* stream) {
+    return subtract_decoded(d_idx12, d_val, nullptr, k, d_ef_desc, n_tensors, total_chunks, use_dct, stream);
+}
+
+int tplr_apply_decoded_batch(const uint8_t* d_idx12, const float* d_val, const float* d_factor, int k,
+                             const tplr_tensor_desc* d_param_desc, int n_tensors, int64_t total_chunks, int use_dct,
+                             void* stream) {
+    return subtract_decoded(d_idx12, d_val, d_factor, k, d_param_desc, n_tensors, total_chunks, use_dct, stream);
 }
 
 int tplr_ef_subtract_own_batch(const uint8_t* d_idx12, const float* d_sent, const float* d_own, int k,

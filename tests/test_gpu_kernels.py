@@ -732,6 +732,82 @@ def test_own_payload_subtraction_writes_what_the_read_modify_write_leaves(dev, k
     assert torch.equal(big[:, :128], torch.from_numpy(t3((320, 512), 5).numpy()).to(dev)[:, :128])  # neighbours of the view untouched
 
 
+# ---------------------------------------------------------------- validator side: one peer's evaluation update
+@pytest.mark.parametrize("use_dct", [True, False])
+@pytest.mark.parametrize("k,repeats", [(32, False), (64, False), (2, False), (16, True)])
+def test_one_peers_payload_applied_to_the_parameters_in_one_launch(dev, use_dct, k, repeats):
+    # neurons/validator.py:3595-3737 per parameter: vals * clip, decompress, decode, p.data.sub_(decoded, alpha=...):
+    # here one launch over three parameters (ragged shapes, one a strided view), alpha and the clip factors riding on
+    # the values.  Without factors the call is tplr_ef_subtract_batch bit for bit.
+    shapes = [(128, 192), (64, 64), (320, 128)]
+    base = t3((320, 512), 5)
+    def fresh():
+        big = base.clone().to(dev)
+        return big, [t3(shapes[0], 1, row_scale=True).to(dev), t3(shapes[1], 2).to(dev), big[:, 128:256]]
+    rng = np.random.default_rng(900 + k)
+    big, params = fresh()
+    pb = tc.TensorBatch(params)
+    n = pb.total_chunks
+    idx = np.stack([rng.choice(4096, size=k, replace=False) for _ in range(n)]).astype(np.int64)
+    if repeats:
+        idx[::3, 1] = idx[::3, 0]          # a peer's row naming an entry twice: the mean of those entries
+        idx[1::5, 2:6] = idx[1::5, 6:7]
+    val = rng.standard_normal((n, k)).astype(np.float32)
+    idx12 = torch.from_numpy(orc.pack12(idx)).to(dev).reshape(-1)
+    d_val = torch.from_numpy(val).to(dev)
+    alpha, clip = 0.0375, np.array([1.0, 0.3125, 0.77], np.float32)
+    tc.apply_decoded_batch(pb, idx12, d_val, k, alpha=alpha, clip=torch.from_numpy(clip), use_dct=use_dct)
+    torch.cuda.synchronize()
+    row = 0
+    for i, s in enumerate(shapes):
+        rows = (s[0] // 64) * (s[1] // 64)
+        sl = slice(row, row + rows)
+        row += rows
+        xshape = (s[0] // 64, s[1] // 64, 64, 64)
+        dense = orc.decompress(orc.pack12(idx[sl]).reshape(xshape[0], xshape[1], -1),
+                               (val[sl] * clip[i]).reshape(xshape[0], xshape[1], k), xshape, 4096)
+        before = (base[:, 128:256] if i == 2 else t3(s, 1 + i, row_scale=(i == 0))).numpy()
+        want = before.astype(np.float64) - alpha * orc.decode2d(dense, use_dct=use_dct).astype(np.float64)
+        got = params[i].cpu().numpy()
+        assert np.abs(got - want).max() <= TOL * max(1.0, np.abs(before).max())
+        if not use_dct and not repeats:
+            # untouched elements keep their bits; touched ones are one multiply and one subtraction
+            flat = orc.encode2d(got, use_dct=False).reshape(rows, 4096)
+            keep = orc.encode2d(before, use_dct=False).reshape(rows, 4096)
+            mask = np.ones_like(flat, bool)
+            np.put_along_axis(mask, idx[sl], False, axis=1)
+            assert np.array_equal(flat[mask], keep[mask])
+            sent = np.take_along_axis(keep, idx[sl], axis=1) - val[sl] * np.float32(np.float32(alpha) * clip[i])
+            assert np.array_equal(np.take_along_axis(flat, idx[sl], axis=1), sent)
+    assert torch.equal(big[:, :128], base.to(dev)[:, :128]) and torch.equal(big[:, 256:], base.to(dev)[:, 256:])
+    # no factors: the miner's subtraction, bit for bit
+    lib = _lib.load()
+    big1, p1 = fresh()
+    big2, p2 = fresh()
+    b1, b2 = tc.TensorBatch(p1), tc.TensorBatch(p2)
+    tc.apply_decoded_batch(b1, idx12, d_val, k, use_dct=use_dct)
+    assert lib.tplr_ef_subtract_batch(idx12.data_ptr(), d_val.data_ptr(), k, b2.table.data_ptr(), len(b2), n, int(use_dct),
+                                      None) == 0
+    torch.cuda.synchronize()
+    for a, b in zip(p1, p2):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+
+
+def test_one_peers_payload_update_rejects_what_it_cannot_serve(dev):
+    params = [t3((64, 128), 3).to(dev)]
+    pb = tc.TensorBatch(params)
+    idx12 = torch.zeros(2 * 48, dtype=torch.uint8, device=dev)
+    val = torch.zeros((2, 32), device=dev)
+    with pytest.raises(ValueError):
+        tc.apply_decoded_batch(pb, idx12.to(torch.int16), val, 32)
+    with pytest.raises(RuntimeError):
+        tc.apply_decoded_batch(pb, idx12[:-3], val, 32)
+    with pytest.raises(IndexError):
+        tc.apply_decoded_batch(pb, idx12, val, 32, clip=torch.ones(2))
+    assert _lib.load().tplr_apply_decoded_batch(idx12.data_ptr(), val.data_ptr(), None, 128, pb.table.data_ptr(), 1, 2, 1,
+                                                None) == _lib.TPLR_E_TOOMANY
+
+
 # ---------------------------------------------------------------- validator side: index checks
 def test_index_stats_match_reference_overlap(dev):
     rng = np.random.default_rng(21)
