@@ -976,10 +976,12 @@ def encode_compress_batch(batch: TensorBatch, topk: int, *, use_dct: bool = True
 
 
 @torch.no_grad()
-def peer_clip_scales_batch(batch: TensorBatch, vals: Sequence[torch.Tensor], k: int) -> torch.Tensor:
+def peer_clip_scales_batch(batch: TensorBatch, vals: Sequence[torch.Tensor], k: int, *, return_median: bool = False):
     """(n_tensors, n_peers) clip factors min(1, median_t / (norm_tp + 1e-8)) from flat payloads:
     what outer_step's block_norms and batch_decompress's clip compute per parameter
-    (src/tplr/neurons.py:346, src/tplr/compress.py:526-556), for all parameters in two launches."""
+    (src/tplr/neurons.py:346, src/tplr/compress.py:526-556), for all parameters in two launches.
+    return_median: also the (n_tensors,) medians of the peers' norms, the per-parameter clip norms the validator
+    keeps for its evaluation updates (clip_norm_dict, neurons/validator.py:3568)."""
     lib = _lib.load()
     P = len(vals)
     if P > _lib.TPLR_MAX_PEERS:
@@ -989,13 +991,14 @@ def peer_clip_scales_batch(batch: TensorBatch, vals: Sequence[torch.Tensor], k: 
     slices = max(1, min(64, 4096 // (len(batch) * P)))
     ss = torch.empty((len(batch), P, slices), dtype=torch.float32, device=dev)
     scale = torch.empty((len(batch), P), dtype=torch.float32, device=dev)
+    median = torch.empty(len(batch), dtype=torch.float32, device=dev) if return_median else None
     vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
     with _on(dev):
         _lib.check(lib.tplr_segment_sumsq(vp, P, k, _ptr(batch.table), len(batch), slices, _ptr(ss), _stream(dev)),
                    "tplr_segment_sumsq")
-        _lib.check(lib.tplr_clip_scales_batch(_ptr(ss), len(batch), P, slices, _ptr(scale), None, _stream(dev)),
+        _lib.check(lib.tplr_clip_scales_batch(_ptr(ss), len(batch), P, slices, _ptr(scale), _ptr(median), _stream(dev)),
                    "tplr_clip_scales_batch")
-    return scale
+    return (scale, median) if return_median else scale
 
 
 @torch.no_grad()
@@ -1088,13 +1091,16 @@ def aggregate_mean_normalised_batch(out: TensorBatch, idxs: Sequence[torch.Tenso
 
 @torch.no_grad()
 def apply_decoded_batch(params: TensorBatch, idx12: torch.Tensor, val: torch.Tensor, k: int, *, alpha: float = 1.0,
-                        clip: torch.Tensor | None = None, use_dct: bool = True) -> None:
+                        clip: torch.Tensor | None = None, clip_norm: torch.Tensor | None = None,
+                        use_dct: bool = True) -> None:
     """param <- param - alpha * decode(decompress(payload * clip)) for every parameter of the set in one launch:
     the validator's per-peer evaluation update (neurons/validator.py:3595-3737, update_model_with_gradient: the
     evaluated peer's values times its clip factor, decompress, decode, p.data.sub_(decoded, alpha=lr *
-    eval_lr_factor)).  `idx12`, `val`: that peer's flat payload (de-quantised values); `clip`: (T,) factors
-    min(1, median_t / (norm_t + 1e-8)) or None.  alpha and clip ride on the values (the transform is linear), so
-    the dense gradient is never formed and every parameter is read and written once.  k <= 64."""
+    eval_lr_factor)).  `idx12`, `val`: that peer's flat payload (de-quantised values); `clip_norm`: (T,) clip norms
+    (the validator's clip_norm_dict, one per parameter): the factors min(1, clip_norm_t / (norm_t + 1e-8)) of
+    validator.py:3608-3612 are formed here from the payload's own per-parameter norms; or `clip`: (T,) ready
+    factors; or neither.  alpha and the factors ride on the values (the transform is linear), so the dense gradient
+    is never formed and every parameter is read and written once.  k <= 64."""
     lib = _lib.load()
     T, n, dev = len(params), params.total_chunks, params.device
     if idx12.dtype != torch.uint8:
@@ -1103,6 +1109,19 @@ def apply_decoded_batch(params: TensorBatch, idx12: torch.Tensor, val: torch.Ten
         raise RuntimeError(f"flat payload mismatch: {idx12.numel()} index bytes / {val.numel()} values for {n} chunks, k={k}")
     if k > _CH:
         raise NotImplementedError(f"top-{k}: the fused update handles k up to {_CH}")
+    if clip_norm is not None:
+        if clip is not None:
+            raise ValueError("give clip_norm or clip, not both")
+        if clip_norm.numel() != T:
+            raise IndexError(f"{clip_norm.numel()} clip norms for {T} parameters")
+        slices = max(1, min(64, 4096 // T))
+        ss = torch.empty((T, 1, slices), dtype=torch.float32, device=dev)
+        vp = (C.c_void_p * 1)(val.data_ptr())
+        with _on(dev):
+            _lib.check(lib.tplr_segment_sumsq(vp, 1, k, _ptr(params.table), T, slices, _ptr(ss), _stream(dev)),
+                       "tplr_segment_sumsq")
+        norm = ss.reshape(T, slices).sum(dim=1).sqrt()
+        clip = (clip_norm.to(device=dev, dtype=torch.float32).reshape(T) / (norm + 1e-8)).clamp(max=1)
     factor = None
     if clip is not None or alpha != 1.0:
         factor = torch.full((T,), float(alpha), dtype=torch.float32, device=dev)

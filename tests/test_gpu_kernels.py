@@ -564,13 +564,16 @@ def test_batch_encode_and_aggregate_match_per_tensor(dev):
               for i, g in enumerate(grads)]
         pay.append(tc.encode_compress_batch(tc.TensorBatch(pg), k))
     idxs, vals = [a for a, _ in pay], [b for _, b in pay]
-    scale = tc.peer_clip_scales_batch(batch, vals, k)
-    assert scale.shape == (len(shapes), P)
+    scale, med = tc.peer_clip_scales_batch(batch, vals, k, return_median=True)
+    assert scale.shape == (len(shapes), P) and med.shape == (len(shapes),)
+    assert torch.equal(scale, tc.peer_clip_scales_batch(batch, vals, k))
     for i in range(len(shapes)):
         norms = np.array([np.sqrt((batch.payload_slice(i, idxs[p], vals[p], k)[1].double() ** 2).sum().item())
                           for p in range(P)], np.float32)
-        _, want = orc.clip_scales(norms)
+        want_med, want = orc.clip_scales(norms)
         assert np.allclose(scale[i].cpu().numpy(), want, rtol=2e-6)
+        # the validator's per-parameter clip norm (neurons/validator.py:3766-3768): torch.median, the lower middle
+        assert np.isclose(float(med[i]), float(want_med), rtol=2e-6) and np.isclose(float(med[i]), np.sort(norms)[(P - 1) // 2], rtol=2e-6)
     outs = [torch.full(s, float("nan"), device=dev) for s in shapes]
     ss = torch.zeros(batch.total_chunks, device=dev)
     tc.batch_decompress_decode_batch(tc.TensorBatch(outs), idxs, vals, k, scale=scale, sumsq=ss)
@@ -780,6 +783,22 @@ def test_one_peers_payload_applied_to_the_parameters_in_one_launch(dev, use_dct,
             sent = np.take_along_axis(keep, idx[sl], axis=1) - val[sl] * np.float32(np.float32(alpha) * clip[i])
             assert np.array_equal(np.take_along_axis(flat, idx[sl], axis=1), sent)
     assert torch.equal(big[:, :128], base.to(dev)[:, :128]) and torch.equal(big[:, 256:], base.to(dev)[:, 256:])
+    # clip norms in place of ready factors (validator.py:3608-3612): min(1, clip_norm / (norm of the parameter's values + 1e-8))
+    row, norms = 0, []
+    for s in shapes:
+        rows = (s[0] // 64) * (s[1] // 64)
+        norms.append(np.sqrt((val[row:row + rows].astype(np.float64) ** 2).sum()))
+        row += rows
+    cn = np.array([norms[0] * 0.5, norms[1] * 2.0, norms[2] * 0.125], np.float32)   # clipped, not clipped, clipped
+    want_clip = np.minimum(1.0, cn / (np.array(norms) + 1e-8)).astype(np.float32)
+    big3, p3 = fresh()
+    big4, p4 = fresh()
+    tc.apply_decoded_batch(tc.TensorBatch(p3), idx12, d_val, k, alpha=alpha, clip_norm=torch.from_numpy(cn), use_dct=use_dct)
+    tc.apply_decoded_batch(tc.TensorBatch(p4), idx12, d_val, k, alpha=alpha, clip=torch.from_numpy(want_clip), use_dct=use_dct)
+    torch.cuda.synchronize()
+    for a, b, f in zip(p3, p4, want_clip):
+        assert float((a - b).abs().max()) <= 1e-6 * max(1.0, float(b.abs().max()))
+    assert want_clip[1] == 1.0 and want_clip[0] < 0.51
     # no factors: the miner's subtraction, bit for bit
     lib = _lib.load()
     big1, p1 = fresh()
