@@ -390,6 +390,113 @@ __device__ __forceinline__ void sort128_step(uint64_t& e0, uint64_t& e1) {
 
 __device__ __forceinline__ void sort128_desc(uint64_t& e0, uint64_t& e1, int) { sort128_step<2, 1>(e0, e1); }
 
+// ---- the same network on 32-bit keys, one per lane.  A subtract whose first source comes from the partner lane by a
+// data-parallel move leaves "partner < mine" as its borrow, a select with the same source takes the partner: two
+// vector instructions per compare-exchange where the partner is reachable by one such move (lane distances 1, 2
+// and 8), three at distance 4 (a reversal inside quads, then one inside groups of eight), and a trip through the
+// LDS crossbar for 16 and 32.  The wait states are those of the 64-bit form: a vector instruction reads a
+// condition two instructions after the vector instruction that first wrote it, a data-parallel move reads a
+// register two instructions after it was written.
+#define TPLR_CX32_DPP(NAME, CTRL)                                                          \
+    __device__ __forceinline__ uint32_t NAME(uint32_t e, uint64_t keepmax) {               \
+        uint32_t out, diff;                                                                \
+        asm("v_sub_co_u32_dpp %1, vcc, %2, %2 " CTRL " row_mask:0xf bank_mask:0xf\n\t"      \
+            "s_xnor_b64 vcc, vcc, %3\n\t"                                                  \
+            "s_nop 0\n\t"                                                                  \
+            "v_cndmask_b32_dpp %0, %2, %2, vcc " CTRL " row_mask:0xf bank_mask:0xf\n\t"     \
+            "s_nop 1"                                                                      \
+            : "=&v"(out), "=&v"(diff)                                                      \
+            : "v"(e), "s"(keepmax)                                                         \
+            : "vcc", "scc");                                                               \
+        return out;                                                                        \
+    }
+TPLR_CX32_DPP(cx32_xor1, "quad_perm:[1,0,3,2]")
+TPLR_CX32_DPP(cx32_xor2, "quad_perm:[2,3,0,1]")
+TPLR_CX32_DPP(cx32_xor8, "row_ror:8")
+#undef TPLR_CX32_DPP
+
+__device__ __forceinline__ uint32_t cx32_xor4(uint32_t e, uint64_t keepmax) {
+    uint32_t out, diff, rev;
+    asm("v_mov_b32_dpp %2, %3 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_sub_co_u32_dpp %1, vcc, %2, %3 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_xnor_b64 vcc, vcc, %4\n\t"
+        "s_nop 0\n\t"
+        "v_cndmask_b32_dpp %0, %2, %3, vcc row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "=&v"(out), "=&v"(diff), "=&v"(rev)
+        : "v"(e), "s"(keepmax)
+        : "vcc", "scc");
+    return out;
+}
+
+__device__ __forceinline__ uint32_t cx32_far(uint32_t e, uint32_t o, uint64_t keepmax) {
+    uint32_t out;
+    asm("v_cmp_lt_u32_e32 vcc, %1, %2\n\t"
+        "s_xnor_b64 vcc, vcc, %3\n\t"
+        "s_nop 0\n\t"
+        "v_cndmask_b32_e32 %0, %1, %2, vcc\n\t"
+        "s_nop 1"
+        : "=&v"(out)
+        : "v"(o), "v"(e), "s"(keepmax)
+        : "vcc", "scc");
+    return out;
+}
+
+template <int J>
+__device__ __forceinline__ uint32_t cx32(uint32_t e, uint64_t keep) {
+    if constexpr (J == 1)
+        return cx32_xor1(e, keep);
+    else if constexpr (J == 2)
+        return cx32_xor2(e, keep);
+    else if constexpr (J == 4)
+        return cx32_xor4(e, keep);
+    else if constexpr (J == 8)
+        return cx32_xor8(e, keep);
+    else
+        return cx32_far(e, static_cast<uint32_t>(__shfl_xor(static_cast<int>(e), J)), keep);
+}
+
+template <int K2, int J>
+__device__ __forceinline__ void sort64_u32_step(uint32_t& e) {
+    constexpr uint64_t keep = keepmax_mask(K2, J, 0);
+    e = cx32<J>(e, keep);
+    if constexpr (J > 1)
+        sort64_u32_step<K2, J / 2>(e);
+    else if constexpr (K2 < 64)
+        sort64_u32_step<K2 * 2, K2>(e);
+}
+
+// descending; keys must differ wherever their order matters
+__device__ __forceinline__ void sort64_desc_u32(uint32_t& e) {
+    asm("s_nop 1" : "+v"(e));  // (the first step reads e by a data-parallel move)
+    sort64_u32_step<2, 1>(e);
+}
+
+// two keys per lane: element i < 64 in lane i of e0, element 64 + i in lane i of e1
+template <int K2, int J>
+__device__ __forceinline__ void sort128_u32_step(uint32_t& e0, uint32_t& e1) {
+    if constexpr (J == 64) {
+        // only reached with K2 = 128: one descending block, the lower half keeps the max
+        const uint32_t a = e0 > e1 ? e0 : e1, b = e0 > e1 ? e1 : e0;
+        e0 = a;
+        e1 = b;
+        asm("s_nop 1" : "+v"(e0), "+v"(e1));  // (written by ordinary code, read next by data-parallel moves)
+    } else {
+        e0 = cx32<J>(e0, keepmax_mask(K2, J, 0));
+        e1 = cx32<J>(e1, keepmax_mask(K2, J, 64));
+    }
+    if constexpr (J > 1)
+        sort128_u32_step<K2, J / 2>(e0, e1);
+    else if constexpr (K2 < 128)
+        sort128_u32_step<K2 * 2, K2>(e0, e1);
+}
+
+__device__ __forceinline__ void sort128_desc_u32(uint32_t& e0, uint32_t& e1) {
+    asm("s_nop 1" : "+v"(e0), "+v"(e1));
+    sort128_u32_step<2, 1>(e0, e1);
+}
+
 // `out_scale` multiplies the gathered values (an exact power of two left over by the caller's
 // transform; the ordering is taken on the unscaled values).
 // `buf` is a kHalfFloats staging buffer, `cand` kCandCap slots; both are free on return.
@@ -400,10 +507,12 @@ template <bool kTwo, bool kOther = false>
 __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf, uint64_t* cand, int lane, int k,
                                                 float out_scale, uint32_t o1 = 0, uint32_t o2 = 0) {
     uint32_t mhi = 0, mlo = 0, cnt = 0, incl = 0, total = 0;
+    uint32_t floor_key;  // no candidate's key is below it (NaN and flushed denormals aside)
     {
         uint32_t b1, b2;
         lane_stats<kTwo>(w, b1, b2);
         const uint32_t t0 = kOther ? stat_threshold_either<kTwo>(b1, b2, o1, o2, k) : stat_threshold<kTwo>(b1, b2, k);
+        floor_key = t0;
         filter_masks(w, __uint_as_float(t0), mhi, mlo);
         cnt = __popc(mhi) + __popc(mlo);
         incl = wave_incl_scan_u32(cnt);
@@ -447,6 +556,7 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
             cnt = __popc(mhi) + __popc(mlo);
             incl = wave_incl_scan_u32(cnt);
             total = __builtin_amdgcn_readlane(incl, 63);
+            floor_key = t;
         }
     }
     uint32_t slot = incl - cnt;  // exclusive prefix of the per-lane counts
@@ -500,12 +610,35 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
     int slot_of_lane = lane;
     asm volatile("" : "+v"(slot_of_lane));
     if (total <= 64) {
-        e0 = lane < static_cast<int>(total) ? cand[slot_of_lane] : 0ull;
-        sort64_desc(e0, lane);
+        const bool mine = lane < static_cast<int>(total);
+        e0 = mine ? cand[slot_of_lane] : 0ull;
+        // Slots were filled in index order, so (magnitude, 63 - slot) orders the candidates as the 64-bit keys
+        // do; with the magnitudes taken from the floor it fits 32 bits while they span less than 2^26 (eight
+        // binades), and the sort costs a third.  The winner's slot comes back out of the key.
+        const uint32_t above = static_cast<uint32_t>(e0 >> 32) - floor_key;
+        if (__ballot(mine && above >= (1u << 26)) == 0) {  // wave-uniform
+            uint32_t key = mine ? (above << 6) | (63u - static_cast<uint32_t>(slot_of_lane)) : 0u;
+            sort64_desc_u32(key);
+            e0 = cand[63u - (key & 63u)];
+        } else {
+            sort64_desc(e0, lane);
+        }
     } else {
+        const bool mine = lane + 64 < static_cast<int>(total);
         e0 = cand[slot_of_lane];
-        e1 = lane + 64 < static_cast<int>(total) ? cand[slot_of_lane + 64] : 0ull;
-        sort128_desc(e0, e1, lane);
+        e1 = mine ? cand[slot_of_lane + 64] : 0ull;
+        // the same with seven bits of slot and magnitudes that span less than 2^25 (four binades)
+        const uint32_t above0 = static_cast<uint32_t>(e0 >> 32) - floor_key;
+        const uint32_t above1 = static_cast<uint32_t>(e1 >> 32) - floor_key;
+        if (__ballot(above0 >= (1u << 25) || (mine && above1 >= (1u << 25))) == 0) {  // wave-uniform
+            uint32_t key0 = (above0 << 7) | (127u - static_cast<uint32_t>(slot_of_lane));
+            uint32_t key1 = mine ? (above1 << 7) | (63u - static_cast<uint32_t>(slot_of_lane)) : 0u;
+            sort128_desc_u32(key0, key1);
+            e0 = cand[127u - (key0 & 127u)];
+            if (kTwo && k > 64) e1 = cand[127u - (key1 & 127u)];
+        } else {
+            sort128_desc(e0, e1, lane);
+        }
     }
     // a slot unpacks to index, and to the value itself: sign bit on top of the magnitude bits
     auto unpack = [&](uint64_t e, uint32_t& ix, float& val) {
