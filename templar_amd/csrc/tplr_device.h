@@ -156,11 +156,26 @@ __device__ __forceinline__ void lane_stats(const float (&v)[64], uint32_t& b1, u
     b2 = __float_as_uint(m2);
 }
 
-// k-th largest of the lane statistics, as magnitude bits (wave-uniform).
+// The search for the k-th largest lane statistic is a chain of dependent steps (vector compare, scalar count,
+// scalar select), one per bit, and a wave does little else meanwhile.  The threshold only has to be a lower bound
+// of the k-th largest magnitude: the search stops early and leaves the lower bits zero, which lets through the
+// few more candidates whose magnitudes lie within 2^-8 (two statistics per lane) or 2^-11 (one) of the exact
+// one.  With one statistic per lane a looser bound would also often leave more than 32 lanes holding candidates,
+// and the select then parks its rows in two turns.
+#ifndef TPLR_THRESHOLD_LOW_BIT_TWO
+#define TPLR_THRESHOLD_LOW_BIT_TWO 15
+#endif
+#ifndef TPLR_THRESHOLD_LOW_BIT_ONE
+#define TPLR_THRESHOLD_LOW_BIT_ONE 12
+#endif
+template <bool kTwo>
+constexpr int kThresholdLowBit = kTwo ? TPLR_THRESHOLD_LOW_BIT_TWO : TPLR_THRESHOLD_LOW_BIT_ONE;
+
+// A lower bound of the k-th largest of the lane statistics, as magnitude bits (wave-uniform): its leading bits.
 template <bool kTwo>
 __device__ __forceinline__ uint32_t stat_threshold(uint32_t b1, uint32_t b2, int k) {
     uint32_t t = 0;
-    for (int bit = 30; bit >= 0; --bit) {
+    for (int bit = 30; bit >= kThresholdLowBit<kTwo>; --bit) {
         const uint32_t c = t | (1u << bit);
         int cnt = __popcll(__ballot(b1 >= c));
         if (kTwo) cnt += __popcll(__ballot(b2 >= c));
@@ -175,7 +190,7 @@ __device__ __forceinline__ uint32_t stat_threshold(uint32_t b1, uint32_t b2, int
 template <bool kTwo>
 __device__ __forceinline__ uint32_t stat_threshold_either(uint32_t b1, uint32_t b2, uint32_t c1, uint32_t c2, int k) {
     uint32_t t = 0;
-    for (int bit = 30; bit >= 0; --bit) {
+    for (int bit = 30; bit >= kThresholdLowBit<kTwo>; --bit) {
         const uint32_t c = t | (1u << bit);
         int nb = __popcll(__ballot(b1 >= c)), nc = __popcll(__ballot(c1 >= c));
         if (kTwo) nb += __popcll(__ballot(b2 >= c)), nc += __popcll(__ballot(c2 >= c));
