@@ -236,6 +236,35 @@ def test_topk_special_values(dev):
         assert np.array_equal(val.cpu().numpy().view(np.uint32), want_v.view(np.uint32))
 
 
+@pytest.mark.parametrize("k", [32, 64, 100])
+def test_topk_candidates_at_the_limits_of_the_short_sort_keys(dev, k):
+    # The candidates are sorted on 32-bit keys (magnitude above the threshold, slot) while their magnitudes span
+    # fewer than eight (one key per lane) or four (two keys) binades, on 64-bit keys otherwise; the threshold is
+    # the leading bits of the k-th largest lane statistic.  Rows built to sit on both sides of each limit; the
+    # selection is the oracle's bit for bit in every case.
+    rng = np.random.default_rng(4242 + k)
+    base = (rng.standard_normal((12, 4096)) * 1e-3).astype(np.float32)
+    rows = base.copy()
+    rows[0, rng.choice(4096, 5, replace=False)] *= np.float32(2.0 ** 3)      # span of three binades: short keys
+    rows[1, rng.choice(4096, 5, replace=False)] *= np.float32(2.0 ** 5)      # five: short keys only with one key per lane
+    rows[2, rng.choice(4096, 5, replace=False)] *= np.float32(2.0 ** 9)      # nine: long keys
+    rows[3, rng.choice(4096, 3, replace=False)] = np.float32(3e38)           # near the largest finite value
+    rows[4, rng.choice(4096, 3, replace=False)] = np.nan                     # NaN candidates rank first
+    rows[5, rng.choice(4096, 3, replace=False)] = -np.inf
+    # magnitudes that differ only below the bits the threshold search looks at: many near-ties around the bound
+    lvl = np.float32(2.5e-3)
+    near = rng.choice(4096, 200, replace=False)
+    rows[6, near] = (lvl * (1 + np.arange(200, dtype=np.float32) * np.float32(2.0 ** -20))) * rng.choice([-1, 1], 200)
+    rows[7, near] = lvl                                                       # exact ties at the bound, index order decides
+    rows[8] = np.abs(rows[8])
+    rows[8, ::64] = np.float32(1.0)                                           # one large value per lane of the chunk layout
+    rows[9, :64] = np.float32(1.0) + np.arange(64, dtype=np.float32) * np.float32(2.0 ** -23)   # all candidates in one lane
+    rows[10] = np.float32(1e-30) * base[10] / np.float32(1e-3)                # tiny but normal magnitudes
+    rows[11] = np.float32(1e-39)                                              # denormals: the compare may flush them
+    rows[11, rng.choice(4096, 40, replace=False)] = np.float32(2e-39)
+    check_topk(rows, k, dev)
+
+
 @pytest.mark.parametrize("n,k", [(64, 32), (64, 64), (100, 10), (37, 6), (4095, 32), (2048, 128), (2, 2), (2048, 512),
                                  (300, 300), (4095, 4094)])
 def test_topk_generic_rows(dev, n, k):
