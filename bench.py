@@ -58,10 +58,11 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--topk", type=int, default=0, help="top-k per chunk instead of the workload's own (templar runs 64)")
     ap.add_argument("--no-dct", action="store_true", help="chunks are selected and scattered untransformed (templar's use_dct=false)")
-    ap.add_argument("--profile", choices=["encode", "aggregate", "miner", "copy", "calib", "fill"], default=None,
+    ap.add_argument("--profile", choices=["encode", "aggregate", "miner", "copy", "calib", "fill", "read"], default=None,
                     help="run only that phase's batched launches --steps times (for rocprofv3) and print nothing; "
                          "'copy' runs the library's calibration copy of 1 GiB instead (counter scaling); 'calib' / 'fill' "
-                         "run the memory-only form of the aggregate kernel with / without its payload loads")
+                         "run the memory-only form of the aggregate kernel with / without its payload loads, 'read' the "
+                         "memory-only form of the encode kernel")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline sample")
     return ap.parse_args()
 
@@ -356,6 +357,12 @@ def main():
     if args.profile == "encode":
         event_ms(encode2d_only, args.steps, args.warmup)
         return
+    if args.profile == "read":
+        lib_r = _lib_mod.load()
+        st_r = torch.cuda.current_stream(dev).cuda_stream
+        event_ms(lambda: _lib_mod.check(lib_r.tplr_calib_encode(batch.table.data_ptr(), len(batch), n_chunks, st_r),
+                                        "tplr_calib_encode"), args.steps, args.warmup)
+        return
     if args.profile is None:
         enc_ms, enc_wall = event_ms(encode_pass, args.steps, args.warmup, settle=True)
     enc_bytes = workloads.encode_bytes(shapes, k)
@@ -363,6 +370,12 @@ def main():
         enc_spread = launch_stats(encode_pass, args.steps)
         enc2d_ms, _ = event_ms(encode2d_only, args.steps, 1)      # the fused 2-D kernel alone (dominant)
         enc2d_spread = launch_stats(encode2d_only, args.steps)
+        # what the memory system alone needs to hand the kernel its input: the library's calibration kernel issues
+        # the encode's row loads (same grid, ranges, instructions) and nothing else
+        _lib_enc = _lib_mod.load()
+        _st_enc = torch.cuda.current_stream(dev).cuda_stream
+        enc_read_ms, _ = event_ms(lambda: _lib_mod.check(_lib_enc.tplr_calib_encode(
+            batch.table.data_ptr(), len(batch), n_chunks, _st_enc), "tplr_calib_encode"), args.steps, 2)
         enc_pt_ms, _ = event_ms(encode_per_tensor, max(3, args.steps // 2), 1)
         enc_rc_ms, _ = event_ms(encode_reference_calls, 3, 1)
     enc2d_bytes = n_chunks * (16384 + 11 * k // 2)
@@ -656,6 +669,12 @@ def main():
                               "not measured by this run; null for other workloads",
             "launches_per_step": 1, "bytes_per_launch": enc2d_bytes, "ms_per_launch": round(enc2d_ms, 4),
             "ms_per_launch_median": enc2d_spread[0], "ms_per_launch_min": enc2d_spread[1],
+            "ceiling": {"read_only_ms": round(enc_read_ms, 4),
+                        "frac_of_hbm_peak": round(n_chunks * 16384 / (enc_read_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                        "kernel_over_read_only": round(enc2d_ms / enc_read_ms, 4),
+                        "what": "tplr_calib_encode: the kernel's own row loads (same grid, chunk ranges and "
+                                "instructions) with no transform, no select and no payload stores - what this box's "
+                                "memory system needs to deliver the launch's input"},
         },
         "roofline_aggregate": {
             "bound": "hbm", "kernel": "k_decode_aggregate",

@@ -429,6 +429,12 @@ int tplr_quantize_batch_static(const float* d_val, int k, const tplr_tensor_desc
  * Profilers' HBM traffic counters are scaled by what they report for this kernel. */
 int tplr_calib_copy(const void* d_src, void* d_dst, int64_t n_bytes, void* stream);
 
+/* Measurement aid, no counterpart in the reference: the memory side of tplr_encode_topk_pack_batch alone.  Same
+ * grid, same chunk ranges and the same 64 streaming row loads per chunk from the tensors of d_desc, without the
+ * transform, the select and the payload stores.  Its duration is the time the memory system needs to hand the
+ * encode its input in that access pattern - the ceiling the real kernel is held against. */
+int tplr_calib_encode(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, void* stream);
+
 /* Measurement aid, no counterpart in the reference: the memory side of tplr_decode_aggregate_batch alone.
  * Same grid, same chunk ranges, the same streaming payload loads (n_peers <= 24, k <= 64) and the same 64 row
  * stores per chunk into the tensors of d_desc, without the scatter and the transform; what it stores is

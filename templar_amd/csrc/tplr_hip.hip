@@ -603,6 +603,28 @@ __global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_de
     }
 }
 
+// Measurement aid: the memory side of the encode alone - the same grid, chunk ranges and row loads, nothing else
+// (the 64 values of a lane are added up so that the loads are not dropped, and the sum never leaves the wave).
+__global__ __launch_bounds__(64, 3) void k_calib_encode(const tplr_tensor_desc* __restrict__ table,
+                                                        const tplr_tensor_desc single, int n_tensors, int64_t total,
+                                                        float* __restrict__ sink) {
+    const int lane = threadIdx.x;
+    int64_t g0, g1;
+    my_range(total, g0, g1);
+    if (g0 >= g1) return;
+    Cursor c;
+    cursor_seek(c, table, single, n_tensors, g0);
+    float s = 0.0f;
+    for (int64_t g = g0; g < g1; ++g) {
+        float v[64];
+        load_chunk_cols(v, c, lane);
+        if (g + 1 < g1) cursor_next(c, g + 1);
+#pragma unroll
+        for (int r = 0; r < 64; ++r) s += v[r];
+    }
+    if (__float_as_uint(s) == 0x7fedcba9u && sink) sink[0] = s;  // (a NaN pattern no sum produces)
+}
+
 // =========================================================================================
 // decode side
 // =========================================================================================
@@ -4059,6 +4081,19 @@ int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_va
         hipLaunchKernelGGL(k_calib_aggregate<4>, grid, dim3(64), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
     else
         hipLaunchKernelGGL(k_calib_aggregate<2>, grid, dim3(64), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
+    return launch_status();
+}
+
+int tplr_calib_encode(const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, void* stream) {
+    if (!d_desc || n_tensors < 1 || total_chunks < 0) return TPLR_E_BADARG;
+    if (total_chunks == 0) return 0;
+    static int resident = 0;
+    if (resident == 0) resident = persistent_grid(k_encode_topk_pack<false, true>, int64_t{1} << 40);  // the grid it stands in for
+    const int64_t need = ((total_chunks + 7) / 8) * 8;
+    tplr_tensor_desc none = {};
+    hipLaunchKernelGGL(k_calib_encode, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), d_desc, none, n_tensors, total_chunks,
+                       static_cast<float*>(nullptr));
     return launch_status();
 }
 
