@@ -576,42 +576,55 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
     }
     uint32_t slot = incl - cnt;  // exclusive prefix of the per-lane counts
 
-    // compaction: lanes park their rows in the staging buffer, so that a lane can fetch its own
-    // candidates with a run-time column index
-    auto compact = [&](const float* row) {
-        while (mhi | mlo) {
-            const bool hi = mhi != 0;
-            const uint32_t m = hi ? mhi : mlo;
-            const int z = __builtin_clz(m);
-            const uint32_t cleared = m & ~(0x80000000u >> z);
-            mhi = hi ? cleared : mhi;
-            mlo = hi ? mlo : cleared;
-            const int d = hi ? z : 32 + z;
-            const uint32_t bits = __float_as_uint(row[d]);
-            const uint32_t ix = lane * 64 + d;
-            cand[slot++] = (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - ix) << 1) | (bits >> 31);
+    // compaction: lanes park their rows in the staging buffer together with a header in the row's four padding
+    // words - the two masks, the first slot and the lane the row came from - and the whole wave then reads the
+    // candidates out with run-time column indices: lane j takes the columns 0-31 of row j & 31 when j < 32 and its
+    // columns 32-63 otherwise, one candidate per trip of a lane-divergent loop.  Two lanes per row halve the
+    // length of that loop where a few rows hold most of the candidates, and nobody waits for the other half of
+    // the wave.
+    auto park = [&](int r) {
+        regs_to_tile_rows(w, buf, r);
+        *reinterpret_cast<uint4*>(buf + r * kLd + 64) = make_uint4(mhi, mlo, slot, static_cast<uint32_t>(lane));
+    };
+    auto compact = [&](int n_rows) {
+        int who = lane;
+        asm volatile("" : "+v"(who));  // (the row address is formed here, not kept across a caller's loop)
+        const int r = who & 31;
+        if (r < n_rows) {
+            const float* row = buf + r * kLd;
+            const uint4 h = *reinterpret_cast<const uint4*>(row + 64);
+            const bool upper = who >= 32;
+            uint32_t m = upper ? h.y : h.x;
+            uint32_t at = upper ? h.z + __popc(h.x) : h.z;
+            const uint32_t ix0 = h.w * 64 + (upper ? 32u : 0u);
+            row += upper ? 32 : 0;
+            while (m) {
+                const int z = __builtin_clz(m);
+                m &= ~(0x80000000u >> z);
+                const uint32_t bits = __float_as_uint(row[z]);
+                const uint32_t ix = ix0 + z;
+                cand[at++] = (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - ix) << 1) | (bits >> 31);
+            }
         }
     };
-    // The threshold is the k-th largest lane maximum, so with k <= 32 and no ties there are exactly k lanes
-    // that hold candidates: their rows fit the buffer's 32 together, each at its rank among those lanes, and
-    // one pass serves all of them (its length is the largest number of candidates in one lane).  Otherwise
-    // each half of the wave takes its turn.
+    // The threshold is about the k-th largest lane maximum, so with k <= 32 and no ties there are k lanes that
+    // hold candidates: their rows fit the buffer's 32 together, each at its rank among those lanes, and one pass
+    // serves all of them.  Otherwise each half of the wave parks its rows in turn.
     const uint64_t holders = __ballot(cnt != 0);
-    if (!kTwo && __popcll(holders) <= 32) {  // wave-uniform
-        if (cnt != 0) {
-            const int r = static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(holders >> 32),
-                                           __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(holders), 0u)));
-            regs_to_tile_rows(w, buf, r);
-            compact(buf + r * kLd);
-        }
+    const int n_holders = __popcll(holders);
+    if (!kTwo && n_holders <= 32) {  // wave-uniform
+        if (cnt != 0)
+            park(static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(holders >> 32),
+                                  __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(holders), 0u))));
+        wave_lds_fence();
+        compact(n_holders);
         wave_lds_fence();
     } else {
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-            if ((lane >> 5) == half) {
-                regs_to_tile_rows(w, buf, lane & 31);
-                compact(buf + (lane & 31) * kLd);
-            }
+            if ((lane >> 5) == half) park(lane & 31);
+            wave_lds_fence();
+            compact(32);
             wave_lds_fence();
         }
     }
