@@ -129,12 +129,14 @@ __device__ __forceinline__ void tile_to_flat(const float* tile, float* __restric
 //
 // Method: a cheap lower bound T0 for the k-th largest magnitude comes from per-lane maxima
 // (k <= 32) or per-lane top-2 (k <= 128): the k-th largest of those is met by at least k
-// elements.  Everything
-// >= T0 (typically 1.1-1.5 k elements) is compacted into 8-byte candidate slots - (magnitude
-// bits, 4095 - index, sign) - and bitonic-sorted.  If more than 128 elements pass, an exact
-// bitwise search for the k-th largest magnitude runs instead (rare: constant or all-zero
-// chunks, pathological ties).  The only LDS needed besides the 128 slots is a 32-row staging
-// buffer through which each half of the wave reads its own row with a run-time index.
+// elements, and so are its leading bits with the rest cleared, which is as far as the search
+// goes.  Everything >= T0 (typically 1.1-1.5 k elements) is compacted into 8-byte candidate
+// slots - (magnitude bits, 4095 - index, sign) - in index order and bitonic-sorted, on 32-bit
+// keys (magnitude above T0, slot) while the magnitudes span few enough binades, on the slots
+// themselves otherwise.  If more than 128 elements pass, an exact bitwise search for the k-th
+// largest magnitude runs instead (rare: constant or all-zero chunks, pathological ties).  The
+// only LDS needed besides the 128 slots is a 32-row staging buffer (its rows' padding words
+// included) from which the candidates are read with run-time column indices.
 // NaN payload bits are not kept: a selected NaN comes out as the quiet NaN of its sign.
 // ---------------------------------------------------------------------------------------
 struct Selected {
