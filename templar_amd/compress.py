@@ -743,7 +743,8 @@ class TopKCompressor:
     def _quantize_values(self, val: torch.Tensor) -> tuple[torch.Tensor, QuantParamsT]:
         half = self.n_bins // 2
         n = val.numel()
-        if val.is_cuda and val.dtype == torch.float32 and n >= 4 and n % 4 == 0 and self.n_bins <= 256:
+        if (val.is_cuda and val.dtype == torch.float32 and n >= 4 and n % 4 == 0 and self.n_bins <= 256
+                and (val.data_ptr() % 16 == 0 or not val.is_contiguous())):  # (the kernel reads 16 bytes at a time)
             # one launch (sums in double) instead of a dozen reductions and scatters; the scale is the
             # only value that travels to the host, as in the reference (float(scale), :620)
             lib = _lib.load()
@@ -1180,11 +1181,7 @@ def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, 
     quant, sent, codes = None, val, None
     if compressor is not None and compressor.use_quantization:
         codes, shift, scale, lookup = quantize_batch(ef, val, k, compressor.n_bins, compressor.range_in_sigmas)
-        sent = torch.empty_like(val)
-        with _on(dev):
-            st = lib.tplr_dequantize_batch(_ptr(codes), _ptr(lookup), _ptr(shift), compressor.n_bins, k, _ptr(ef.table),
-                                           len(ef), n, _ptr(sent), _stream(dev))
-        _lib.check(st, "tplr_dequantize_batch")
+        sent = dequantize_batch(ef, codes.reshape(-1), None, k, out=torch.empty_like(val), tables=(lookup, shift))
         # the reference's quant_params carry the scale as a Python float (:620): the copy to the host
         # is queued here and read after the subtraction has been launched
         with _on(dev):
@@ -1467,6 +1464,17 @@ def quantize_batch(batch: TensorBatch, val: torch.Tensor, k: int, n_bins: int = 
     shift = torch.empty(T, dtype=torch.float32, device=dev)
     scale = torch.empty(T, dtype=torch.float32, device=dev)
     lookup = torch.empty((T, n_bins), dtype=torch.float32, device=dev)
+    if k % 4:
+        # the whole-set kernel reads the values four at a time; a top-k that is not a multiple of four (the clamp
+        # only makes it even) goes parameter by parameter through the compressor's own quantiser, on the device
+        comp = TopKCompressor(use_quantization=True, quantization_bins=n_bins, quantization_range=range_in_sigmas)
+        for i in range(T):
+            b, rows = batch.offsets[i], batch.payload_rows(i)
+            q, (sh, sc, _, lk, _) = comp._quantize_values(val[b:b + rows])
+            codes[b:b + rows].copy_(q)
+            shift[i], scale[i] = sh, sc
+            lookup[i].copy_(lk)
+        return codes, shift, scale, lookup
     slices = max(1, min(64, 2048 // T))  # enough workgroups to fill the device
     work = torch.empty(T * slices * (2 + 2 * n_bins), dtype=torch.float64, device=dev)
     with _on(dev):
@@ -1497,6 +1505,12 @@ def dequantize_batch(batch: TensorBatch, codes: torch.Tensor, qparams: Sequence[
         lookup, shift, n_bins = _qparam_tables(qparams, dev)
     if out is None:
         out = torch.empty((n, k), dtype=torch.float32, device=dev)
+    if k % 4:  # (see quantize_batch) lookup[t][code] + shift[t] per parameter by torch's device ops
+        codes2 = codes.reshape(n, k)
+        for i in range(len(batch)):
+            b, rows = batch.offsets[i], batch.payload_rows(i)
+            out[b:b + rows] = lookup[i][codes2[b:b + rows].long()] + shift[i]
+        return out
     with _on(dev):
         st = lib.tplr_dequantize_batch(_ptr(codes.contiguous()), _ptr(lookup), _ptr(shift), n_bins, k, _ptr(batch.table),
                                        len(batch), n, _ptr(out), _stream(dev))

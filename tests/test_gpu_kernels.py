@@ -673,6 +673,37 @@ def test_error_feedback_step_matches_reference_sequence(dev, use_dct, k, bins):
             assert np.array_equal(q.cpu().numpy(), wq)
 
 
+@pytest.mark.parametrize("use_dct,k,bins", [(True, 6, 4), (False, 10, 256), (False, 2, 4)])
+def test_error_feedback_step_with_quantiser_for_a_topk_that_is_not_a_multiple_of_four(dev, use_dct, k, bins):
+    # the whole-set quantiser kernels read values four at a time; other (even) k go parameter by parameter through
+    # torch's device ops: the payload is the oracle's, the codes are the oracle's except where a sum rounded
+    # differently moves a value across a bin edge, and what is subtracted is what the codes de-quantise to
+    shapes = [(128, 192), (64, 64), (192, 128)]
+    decay = 0.9
+    efs = [t3(s, 700 + i, row_scale=True) for i, s in enumerate(shapes)]
+    grads = [t3(s, 800 + i, row_scale=True) * 0.5 for i, s in enumerate(shapes)]
+    d_ef = [e.clone().to(dev) for e in efs]
+    comp = tc.TopKCompressor(use_quantization=True, quantization_bins=bins, quantization_range=6)
+    eb, gb = tc.TensorBatch(d_ef), tc.TensorBatch([g.to(dev) for g in grads])
+    idx12, val, quant = tc.error_feedback_step_batch(eb, gb, decay, k, use_dct=use_dct, compressor=comp)
+    tr = tc.ChunkingTransformer(_Stub(d_ef), 64)
+    for i, s in enumerate(shapes):
+        acc = (efs[i] * decay) + grads[i]
+        coef = tr.encode(acc.to(dev), use_dct=use_dct).cpu().numpy()
+        _, want_i, want_v, _ = orc.error_feedback_step(efs[i].numpy(), grads[i].numpy(), decay, k, use_dct=use_dct,
+                                                       quant_bins=0, coef_override=coef)
+        got_i, got_v = eb.payload_slice(i, idx12, val, k)
+        assert np.array_equal(got_i.cpu().numpy(), want_i) and np.array_equal(got_v.cpu().numpy(), want_v)
+        q, qp = quant[i]
+        wq, wqp = orc.quantize(want_v, bins, 6.0)
+        assert (q.cpu().numpy() != wq).mean() <= 2e-3
+        sent = orc.dequantize(q.cpu().numpy(), (float(qp[0]), qp[1], qp[2], qp[3].cpu().numpy()))
+        y, x = s[0] // 64, s[1] // 64
+        dense = orc.decompress(want_i, sent.reshape(y, x, k), (y, x, 64, 64), 4096)
+        want_new = acc.numpy().astype(np.float64) - orc.decode2d(dense, use_dct=use_dct)
+        assert np.abs(d_ef[i].cpu().numpy() - want_new).max() <= TOL * np.abs(acc.numpy()).max()
+
+
 def test_error_feedback_null_round_and_equivalence_with_separate_calls(dev):
     shape = (192, 128)
     ef0 = t3(shape, 77, row_scale=True)
