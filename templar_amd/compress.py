@@ -1663,14 +1663,10 @@ class PayloadStage:
         if not self.quantized:
             return out_i, out_v
         lookup, shift = self._tables
-        lib = _lib.load()
-        dev, T, n_rows = self.dev.device, len(self.batch), self.batch.total_chunks
-        with _on(dev):
-            for p in range(n_peers):
-                st = lib.tplr_dequantize_batch(_ptr(out_v[p]), _ptr(lookup[p * T:(p + 1) * T]), _ptr(shift[p * T:(p + 1) * T]),
-                                               int(lookup.shape[1]), self.k, _ptr(self.batch.table), T, n_rows,
-                                               _ptr(self.values[p]), _stream(dev))
-                _lib.check(st, "tplr_dequantize_batch")
+        T = len(self.batch)
+        for p in range(n_peers):
+            dequantize_batch(self.batch, out_v[p].reshape(-1), None, self.k, out=self.values[p],
+                             tables=(lookup[p * T:(p + 1) * T], shift[p * T:(p + 1) * T]))
         return out_i, [self.values[p] for p in range(n_peers)]
 
     def regions(self, p: int) -> tuple[torch.Tensor, torch.Tensor]:
@@ -1760,14 +1756,9 @@ class PayloadStage:
             self.tables = dequantised_tables(quant_params, self.dev.device)
             return out_i, out_v
         lookup, shift, n_bins = _qparam_tables([quant_params[i][p] for p in range(P) for i in range(T)], self.dev.device)
-        lib = _lib.load()
-        dev, n = self.dev.device, self.batch.total_chunks
-        with _on(dev):
-            for p in range(P):
-                st = lib.tplr_dequantize_batch(_ptr(out_v[p]), _ptr(lookup[p * T:(p + 1) * T]), _ptr(shift[p * T:(p + 1) * T]),
-                                               n_bins, self.k, _ptr(self.batch.table), T, n, _ptr(self.values[p]),
-                                               _stream(dev))
-                _lib.check(st, "tplr_dequantize_batch")
+        for p in range(P):
+            dequantize_batch(self.batch, out_v[p].reshape(-1), None, self.k, out=self.values[p],
+                             tables=(lookup[p * T:(p + 1) * T], shift[p * T:(p + 1) * T]))
         self._tables = (lookup, shift)  # alive until the launches above have run
         return out_i, [self.values[p] for p in range(P)]
 

@@ -1114,12 +1114,13 @@ def test_aggregate_without_transform_writes_the_gradient_layout(dev):
 
 
 # ---------------------------------------------------------------- a gathered window as flat buffers
-@pytest.mark.parametrize("quantized,where", [(True, "cpu"), (False, "cpu"), (True, "cuda")])
-def test_payload_stage_equals_per_parameter_path(dev, quantized, where):
+@pytest.mark.parametrize("quantized,where,k", [(True, "cpu", 32), (False, "cpu", 32), (True, "cuda", 32), (True, "cpu", 6),
+                                               (True, "cuda", 10)])
+def test_payload_stage_equals_per_parameter_path(dev, quantized, where, k):
     # the reference's per-parameter lists (src/tplr/comms.py:1938-1963) of P peers, staged flat and
     # aggregated in one launch, against the per-parameter calls of src/tplr/neurons.py:309-367
     shapes = [(128, 192), (64, 64), (256, 128), (64, 320)]
-    k, P = 32, 5
+    P = 5
     comp = tc.TopKCompressor(use_quantization=quantized, quantization_bins=256, quantization_range=6)
     tr = tc.ChunkingTransformer(_Stub([torch.empty(s) for s in shapes]), 64)
     idxs, vals, qps = [[] for _ in shapes], [[] for _ in shapes], [[] for _ in shapes]
@@ -1412,7 +1413,7 @@ def test_sums_of_squares_of_the_summed_coefficients_from_the_payloads(dev, P, k,
 
 
 @pytest.mark.parametrize("P,k,bins,staged", [(20, 64, 4, True), (15, 32, 4, False), (5, 64, 2, False), (8, 16, 3, True),
-                                             (24, 4, 4, False)])
+                                             (24, 4, 4, False), (3, 6, 4, False), (4, 10, 4, True)])
 def test_aggregate_straight_from_four_bin_codes_equals_dequantise_then_aggregate(dev, P, k, bins, staged):
     # templar's own settings (hparams.json: quantization_bins 4, topk 64, use_dct false, 20 peers): the aggregate
     # picks every entry's value among its peer's four and the norms come from four counts - against
