@@ -693,7 +693,7 @@ __device__ __forceinline__ void emit_selected(const Selected& s, int lane, int k
     // they are recomputed here instead of being kept, or spilled, across a caller's chunk loop)
     asm volatile("" : "+v"(lane));
     if (lane < k) vrow[lane] = s.val0;
-    const uint32_t p0 = __shfl_xor(s.idx0, 1);
+    const uint32_t p0 = lane_xor_u32<1>(s.idx0);  // (the neighbour's index by a data-parallel move, no LDS trip)
     if (!(lane & 1) && lane < k) {
         const uint32_t w = s.idx0 | (p0 << 12);
         uint8_t* o = irow + 3 * (lane >> 1);
@@ -703,7 +703,7 @@ __device__ __forceinline__ void emit_selected(const Selected& s, int lane, int k
     }
     if (kTwo && k > 64) {
         if (lane + 64 < k) vrow[lane + 64] = s.val1;
-        const uint32_t p1 = __shfl_xor(s.idx1, 1);
+        const uint32_t p1 = lane_xor_u32<1>(s.idx1);
         if (!(lane & 1) && lane + 64 < k) {
             const uint32_t w = s.idx1 | (p1 << 12);
             uint8_t* o = irow + 3 * ((lane + 64) >> 1);
