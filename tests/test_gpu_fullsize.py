@@ -208,6 +208,43 @@ def test_full_set_error_feedback_step(dev):
 
 
 
+@pytest.mark.parametrize("use_dct", [True, False])
+def test_full_set_evaluation_update_properties(dev, use_dct):
+    # neurons/validator.py:3595-3737 on the 1B set: p <- p - alpha * decode(decompress(vals * clip)), one launch.
+    # Linearity gives size-independent checks: the update equals p - alpha * (the one-peer decode with the same clip
+    # factors) within fp32 tolerance, and applying it again with -alpha brings the parameters back.
+    grads, k = _set("cfg3_llama1b", dev)
+    batch = tc.TensorBatch(grads)
+    idx12, val = tc.encode_compress_batch(batch, k, use_dct=use_dct)
+    del grads, batch
+    gen = torch.Generator(device=dev).manual_seed(11)
+    shapes = [tuple(s) for s in workloads.CONFIGS["cfg3_llama1b"]["shapes"] if len(s) == 2]
+    params = [torch.randn(s, device=dev, generator=gen) * 0.02 for s in shapes]
+    start = [p.clone() for p in params]
+    pb = tc.TensorBatch(params)
+    T = len(params)
+    clip = torch.rand(T, device=dev, generator=gen) * 0.9 + 0.1
+    alpha = 0.37
+    tc.apply_decoded_batch(pb, idx12, val, k, alpha=alpha, clip=clip, use_dct=use_dct)
+    dense = [torch.empty(s, device=dev) for s in shapes]
+    tc.batch_decompress_decode_batch(tc.TensorBatch(dense), [idx12], [val], k, scale=clip.reshape(T, 1).contiguous(),
+                                     use_dct=use_dct)
+    worst = 0.0
+    for p, p0, d in zip(params, start, dense):
+        want = p0 - alpha * d
+        worst = max(worst, float((p - want).abs().max()) / max(1e-30, float(want.abs().max())))
+    assert worst <= TOL
+    del dense
+    tc.apply_decoded_batch(pb, idx12, val, k, alpha=-alpha, clip=clip, use_dct=use_dct)
+    back = max(float((p - p0).abs().max()) / float(p0.abs().max()) for p, p0 in zip(params, start))
+    assert back <= TOL
+    if not use_dct:
+        # without the transform only the k named positions of a chunk change
+        tc.apply_decoded_batch(pb, idx12, val, k, alpha=alpha, clip=clip, use_dct=False)
+        changed = sum(int((p != p0).sum()) for p, p0 in zip(params, start))
+        assert changed <= pb.total_chunks * k
+
+
 @pytest.mark.parametrize("P,k", [(20, 64), (15, 32), (12, 64)])
 def test_full_size_index_statistics_against_bitmaps(dev, P, k):
     # the 1B set's 294 144 rows: every wave walks 144 rows, so the per-lane bit-plane counters are
