@@ -244,6 +244,23 @@ int tplr_segment_sumsq(const float* const* h_val, int n_peers, int k, const tplr
 int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int n_partials, float* d_scale,
                            float* d_median, void* stream);
 
+/* The same norms in two steps, so that the pass over the values is made once, when a payload arrives, and the
+ * clip factors of a window (src/tplr/neurons.py:346, src/tplr/compress.py:526-556) cost one float per row:
+ * tplr_row_sumsq: h_row_sumsq[p][r] = sum of squares of row r (k values, 1 <= k <= 4096) of peer p's flat values,
+ * n_rows rows per peer (h_val, h_row_sumsq: HOST arrays of n_peers DEVICE pointers), one launch.  The additions
+ * have a fixed order: a pairwise tree over the row's squares placed in the next power of two of lanes (rows
+ * longer than 64: lane j first adds the squares of values j, j + 64, ...).
+ * tplr_clip_scales_rows: d_scale[t * n_peers + p] = min(1, med_t / (norm_tp + 1e-8)) with norm_tp = sqrt of
+ * the sum, in double and in a fixed order, of the row figures of tensor t (rows chunk_begin ... of d_desc;
+ * x_chunks * y_chunks of them), med_t the lower median over the peers; d_median (nullable) receives med_t.
+ * d_partial: workspace of n_tensors * n_peers * n_slices doubles (n_slices >= 1 cuts large tensors so that a
+ * few of them still fill the device).  Two launches. */
+int tplr_row_sumsq(const float* const* h_val, int n_peers, int k, int64_t n_rows, float* const* h_row_sumsq,
+                   void* stream);
+int tplr_clip_scales_rows(const float* const* h_row_sumsq, int n_peers, const tplr_tensor_desc* d_desc,
+                          int n_tensors, int n_slices, double* d_partial, float* d_scale, float* d_median,
+                          void* stream);
+
 /* ---- miner side: error-feedback step (src/tplr/neurons.py:147-171) ------------------
  * The reference runs, per parameter: ef.mul_(decay); ef.add_(grad); encode(ef); compress;
  * decompress; decode; ef.sub_(decoded).  Two launches over a whole gradient set do the same:
@@ -428,6 +445,13 @@ int tplr_quantize_batch_static(const float* d_val, int k, const tplr_tensor_desc
  * (a multiple of 16, both pointers 16-byte aligned) that moves exactly n_bytes each way.
  * Profilers' HBM traffic counters are scaled by what they report for this kernel. */
 int tplr_calib_copy(const void* d_src, void* d_dst, int64_t n_bytes, void* stream);
+
+/* Measurement aid, no counterpart in the reference: a plain fill of n_bytes (a multiple of 16, pointer 16-byte
+ * aligned) over a linear address range with 16-byte stores, the write rate of the memory system under the
+ * friendliest access pattern.  pattern 0: grid-stride (neighbouring workgroups write neighbouring kilobytes);
+ * 1: the same with streaming stores; 2: every wave walks one contiguous span, as a persistent kernel would.
+ * The aggregate's chunk-pattern fill (tplr_calib_aggregate with no peers) is held against it. */
+int tplr_calib_fill(void* d_dst, int64_t n_bytes, int pattern, void* stream);
 
 /* Measurement aid, no counterpart in the reference: the memory side of tplr_encode_topk_pack_batch alone.  Same
  * grid, same chunk ranges and the same 64 streaming row loads per chunk from the tensors of d_desc, without the

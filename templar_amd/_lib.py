@@ -44,6 +44,8 @@ SIGNATURES = {
     "tplr_decode_aggregate_codes_stats_batch": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _i32, _vp, _vp, _vp]),
     "tplr_segment_sumsq": (_i32, [_vp, _i32, _i32, _vp, _i32, _i32, _vp, _vp]),
     "tplr_clip_scales_batch": (_i32, [_vp, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "tplr_row_sumsq": (_i32, [_vp, _i32, _i32, _i64, _vp, _vp]),
+    "tplr_clip_scales_rows": (_i32, [_vp, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _vp]),
     "tplr_decode_aggregate": (_i32, [_vp, _vp, _vp, _i32, _i32, _i64, _i64, _i32, _i32, _i32, _vp, _i64, _vp, _vp]),
     "tplr_scatter_rows": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp]),
     "tplr_flat_update": (_i32, [_vp, _vp, _i64, C.c_float, _i32, _vp]),
@@ -53,6 +55,7 @@ SIGNATURES = {
     "tplr_clip_scales": (_i32, [_vp, _i32, _i32, _vp, _vp, _vp]),
     "tplr_calib_encode": (_i32, [_vp, _i32, _i64, _vp]),
     "tplr_calib_copy": (_i32, [_vp, _vp, _i64, _vp]),
+    "tplr_calib_fill": (_i32, [_vp, _i64, _i32, _vp]),
     "tplr_calib_aggregate": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _i32, _i64, _vp]),
     "tplr_ef_encode_topk_pack_batch": (_i32, [_vp, _vp, _i32, _i64, C.c_float, _i32, _i32, _vp, _vp, _vp]),
     "tplr_ef_subtract_batch": (_i32, [_vp, _vp, _i32, _vp, _i32, _i64, _i32, _vp]),

@@ -929,6 +929,7 @@ class TensorBatch:
         self.tensors = list(tensors)  # keeps the storage alive
         self.total_chunks = begin
         self.device = dev
+        self.desc = desc  # host copy of the table
         self.table = torch.from_numpy(desc.view(np.uint8).copy()).to(dev)
 
     def __len__(self) -> int:
@@ -976,30 +977,131 @@ def encode_compress_batch(batch: TensorBatch, topk: int, *, use_dct: bool = True
     return idx12, val
 
 
+class PeerNorms:
+    """The peers' per-parameter norms of a window, kept as one float per payload row.
+
+    The reference takes `torch.linalg.vector_norm` of every peer's values of every parameter when it
+    aggregates (src/tplr/neurons.py:346) and batch_decompress clips by their median
+    (src/tplr/compress.py:526-556): a pass over all values on the aggregate's critical path.  Here the pass is
+    made once per peer when its payload arrives (`arrived`: a row's sum of squares, one launch, which runs
+    while the next peer is still in transfer), and the clip factors of the whole window come from those
+    figures in two small launches (`clip_scales`), for several batches at once (a model's 2-D parameters and
+    its 1-D ones).  The additions have a fixed order, so factors computed on arrival and factors computed from
+    the values at aggregate time (`peer_clip_scales_batch`) are the same bits."""
+
+    def __init__(self, batches: "Sequence[TensorBatch | RowBatch]", max_peers: int):
+        import numpy as np
+
+        if not batches:
+            raise ValueError("PeerNorms needs at least one batch")
+        if max_peers < 1 or max_peers > _lib.TPLR_MAX_PEERS:
+            raise ValueError(f"max_peers must be in [1, {_lib.TPLR_MAX_PEERS}]")
+        dev = batches[0].device
+        self.batches, self.max_peers, self.device = list(batches), max_peers, dev
+        self.row_begin: list[int] = []
+        self.tensor_begin: list[int] = []
+        tables, rows, tensors = [], 0, 0
+        for b in batches:
+            if b.device != dev:
+                raise ValueError("PeerNorms: the batches live on different devices")
+            d = b.desc.copy()
+            d["chunk_begin"] += rows  # this batch's rows follow the previous batches' in the row figures
+            tables.append(d)
+            self.row_begin.append(rows)
+            self.tensor_begin.append(tensors)
+            rows += b.total_chunks
+            tensors += len(b)
+        self.total_rows, self.n_tensors = rows, tensors
+        self.table = batches[0].table if len(batches) == 1 else \
+            torch.from_numpy(np.concatenate(tables).view(np.uint8).copy()).to(dev)
+        self.row_sumsq = torch.empty((max_peers, max(rows, 1)), dtype=torch.float32, device=dev)
+        self.slices = max(1, min(64, 4096 // (tensors * max_peers)))
+        self._partial = torch.empty((tensors, max_peers, self.slices), dtype=torch.float64, device=dev)
+        self._scale = torch.empty((tensors, max_peers), dtype=torch.float32, device=dev)
+        self._median = torch.empty(tensors, dtype=torch.float32, device=dev)
+
+    @torch.no_grad()
+    def arrived(self, p: int, vals: "Sequence[torch.Tensor | None]") -> None:
+        """Peer p's fp32 values have arrived: vals[b] is its flat payload for batch b ((rows, k) or flat; None:
+        that part is not here yet).  One launch per part, on the current stream."""
+        if not 0 <= p < self.max_peers:
+            raise IndexError(f"peer {p} of a window of {self.max_peers}")
+        if len(vals) != len(self.batches):
+            raise IndexError(f"{len(vals)} payload parts for {len(self.batches)} batches")
+        lib = _lib.load()
+        with _on(self.device):
+            for b, v in zip(range(len(self.batches)), vals):
+                if v is None:
+                    continue
+                n = self.batches[b].total_chunks
+                _need_device(v, "PeerNorms.arrived")
+                if v.dtype != torch.float32 or not v.is_contiguous() or n == 0 or v.numel() % n:
+                    raise RuntimeError(f"batch {b}: {v.numel()} values of {v.dtype} for {n} rows")
+                vp = (C.c_void_p * 1)(v.data_ptr())
+                op = (C.c_void_p * 1)(self.row_sumsq[p].data_ptr() + 4 * self.row_begin[b])
+                _lib.check(lib.tplr_row_sumsq(vp, 1, v.numel() // n, n, op, _stream(self.device)), "tplr_row_sumsq")
+
+    @torch.no_grad()
+    def arrived_all(self, b: int, vals: Sequence[torch.Tensor]) -> None:
+        """All peers' values of batch b at once (peer p = vals[p]), one launch."""
+        P, n = len(vals), self.batches[b].total_chunks
+        if P < 1 or P > self.max_peers:
+            raise ValueError(f"{P} peers for a window of {self.max_peers}")
+        k = vals[0].numel() // max(n, 1)
+        for v in vals:
+            _need_device(v, "PeerNorms.arrived_all")
+            if v.dtype != torch.float32 or not v.is_contiguous() or n == 0 or v.numel() != n * k:
+                raise RuntimeError(f"batch {b}: {v.numel()} values of {v.dtype} for {n} rows of {k}")
+        lib = _lib.load()
+        vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
+        op = (C.c_void_p * P)(*[self.row_sumsq[p].data_ptr() + 4 * self.row_begin[b] for p in range(P)])
+        with _on(self.device):
+            _lib.check(lib.tplr_row_sumsq(vp, P, k, n, op, _stream(self.device)), "tplr_row_sumsq")
+
+    @torch.no_grad()
+    def clip_scales(self, n_peers: int, *, return_median: bool = False):
+        """Clip factors min(1, median_t / (norm_tp + 1e-8)) of the first n_peers peers for every parameter of
+        every batch, two launches: a list with one (T_b, n_peers) tensor per batch (views of one buffer, valid
+        until the next call); return_median: also the list of (T_b,) medians of the peers' norms."""
+        if n_peers < 1 or n_peers > self.max_peers:
+            raise ValueError(f"{n_peers} peers for a window of {self.max_peers}")
+        lib = _lib.load()
+        T = self.n_tensors
+        rp = (C.c_void_p * n_peers)(*[self.row_sumsq[p].data_ptr() for p in range(n_peers)])
+        scale = self._scale.reshape(-1)[:T * n_peers].view(T, n_peers)
+        with _on(self.device):
+            _lib.check(lib.tplr_clip_scales_rows(rp, n_peers, _ptr(self.table), T, self.slices, _ptr(self._partial),
+                                                 _ptr(scale), _ptr(self._median), _stream(self.device)),
+                       "tplr_clip_scales_rows")
+        ends = self.tensor_begin[1:] + [T]
+        scales = [scale[a:e] for a, e in zip(self.tensor_begin, ends)]
+        if return_median:
+            return scales, [self._median[a:e] for a, e in zip(self.tensor_begin, ends)]
+        return scales
+
+
 @torch.no_grad()
-def peer_clip_scales_batch(batch: TensorBatch, vals: Sequence[torch.Tensor], k: int, *, return_median: bool = False):
+def peer_clip_scales_batch(batch: "TensorBatch | RowBatch", vals: Sequence[torch.Tensor], k: int, *,
+                           return_median: bool = False):
     """(n_tensors, n_peers) clip factors min(1, median_t / (norm_tp + 1e-8)) from flat payloads:
     what outer_step's block_norms and batch_decompress's clip compute per parameter
-    (src/tplr/neurons.py:346, src/tplr/compress.py:526-556), for all parameters in two launches.
+    (src/tplr/neurons.py:346, src/tplr/compress.py:526-556), for all parameters in three launches (the rows'
+    sums of squares of all peers, their sums per parameter, the factors); a window whose payloads were noted
+    on arrival (PeerNorms) skips the first, the only one that reads the values.
     return_median: also the (n_tensors,) medians of the peers' norms, the per-parameter clip norms the validator
     keeps for its evaluation updates (clip_norm_dict, neurons/validator.py:3568)."""
-    lib = _lib.load()
     P = len(vals)
     if P > _lib.TPLR_MAX_PEERS:
         raise NotImplementedError(f"{P} peers: the HIP aggregate kernel takes up to {_lib.TPLR_MAX_PEERS}")
-    dev = batch.device
-    # enough blocks to fill the device even when the set is a few very large tensors
-    slices = max(1, min(64, 4096 // (len(batch) * P)))
-    ss = torch.empty((len(batch), P, slices), dtype=torch.float32, device=dev)
-    scale = torch.empty((len(batch), P), dtype=torch.float32, device=dev)
-    median = torch.empty(len(batch), dtype=torch.float32, device=dev) if return_median else None
-    vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
-    with _on(dev):
-        _lib.check(lib.tplr_segment_sumsq(vp, P, k, _ptr(batch.table), len(batch), slices, _ptr(ss), _stream(dev)),
-                   "tplr_segment_sumsq")
-        _lib.check(lib.tplr_clip_scales_batch(_ptr(ss), len(batch), P, slices, _ptr(scale), _ptr(median), _stream(dev)),
-                   "tplr_clip_scales_batch")
-    return (scale, median) if return_median else scale
+    for v in vals:
+        if v.numel() != batch.total_chunks * k:
+            raise RuntimeError(f"flat payload mismatch: {v.numel()} values for {batch.total_chunks} rows, k={k}")
+    norms = PeerNorms([batch], P)
+    norms.arrived_all(0, vals)
+    if return_median:
+        scales, medians = norms.clip_scales(P, return_median=True)
+        return scales[0], medians[0]
+    return norms.clip_scales(P)[0]
 
 
 @torch.no_grad()
@@ -1251,6 +1353,7 @@ class RowBatch:
                                                       ("x_chunks", "<i4"), ("y_chunks", "<i4")]))
         for i, (b, n) in enumerate(zip(self.offsets, self.rows)):
             desc[i] = (tensors[i].data_ptr(), _CH, b, n, 1)
+        self.desc = desc  # host copy of the table
         self.table = torch.from_numpy(desc.view(np.uint8).copy()).to(dev)
         self.total_groups = sum((n + _CH - 1) // _CH for n in self.rows)  # waves of up to 64 rows of one tensor
 
@@ -1298,7 +1401,7 @@ def encode_compress_rows_batch(batch: RowBatch, topk: int, *, use_dct: bool = Tr
 @torch.no_grad()
 def batch_decompress_decode_rows_batch(out: RowBatch, idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], k: int,
                                        *, clip_norm: bool = True, use_dct: bool = True, validate: bool = True,
-                                       two_step: bool = False) -> None:
+                                       two_step: bool = False, scale: torch.Tensor | None = None) -> None:
     """batch_decompress + decode (src/tplr/neurons.py:341-367) of every 1-D parameter at once: peer p's
     flat payload is (idxs[p], vals[p]).  Per parameter and peer the values are clipped to the median
     norm over the peers (reference :526-556), every row takes the mean over the peers that sent each
@@ -1306,7 +1409,8 @@ def batch_decompress_decode_rows_batch(out: RowBatch, idxs: Sequence[torch.Tenso
     The payloads are a few hundred KB: a fixed, small number of launches whatever the number of
     parameters.  `validate` (default) raises on an index of 64 or more, as torch's scatter does, which
     costs a synchronisation; without it such entries are dropped.  `two_step` keeps the aggregate and the
-    transform as two launches with the rows in a buffer between them (the same bits)."""
+    transform as two launches with the rows in a buffer between them (the same bits).  `scale`: ready (T, P) clip
+    factors (PeerNorms.clip_scales) instead of the norms taken here."""
     lib = _lib.load()
     P, R, T, dev = len(vals), out.total_rows, len(out), out.device
     for i, v in zip(idxs, vals):
@@ -1316,7 +1420,10 @@ def batch_decompress_decode_rows_batch(out: RowBatch, idxs: Sequence[torch.Tenso
             raise RuntimeError(f"flat payload mismatch: {i.numel()} index bytes / {v.numel()} values for {R} rows, k={k}")
     vals = [_val_on(x, dev) for x in vals]
     idxs = [_idx_on(i, dev) for i in idxs]
-    scale = peer_clip_scales_batch(out, vals, k) if clip_norm else None               # (T, P), two launches
+    if scale is None and clip_norm:
+        scale = peer_clip_scales_batch(out, vals, k)                                  # (T, P), three launches
+    elif scale is not None and (tuple(scale.shape) != (T, P) or scale.dtype != torch.float32 or not scale.is_contiguous()):
+        raise ValueError(f"scale: expected a contiguous fp32 ({T}, {P}) tensor, got {tuple(scale.shape)}")
     err = torch.zeros(1, dtype=torch.int32, device=dev) if validate else None
     ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
     vp = (C.c_void_p * P)(*[x.data_ptr() for x in vals])
@@ -1615,7 +1722,7 @@ class PayloadStage:
     _ALIGN = 256
 
     def __init__(self, batch: TensorBatch, k: int, max_peers: int, *, quantized: bool = True,
-                 host_threads: int | None = None):
+                 host_threads: int | None = None, norms: "PeerNorms | None" = None):
         if max_peers < 1 or max_peers > _lib.TPLR_MAX_PEERS:
             raise ValueError(f"max_peers must be in [1, {_lib.TPLR_MAX_PEERS}]")
         if k < 2 or k % 2:
@@ -1629,11 +1736,17 @@ class PayloadStage:
         self.stride = self.val_off + up(self.val_bytes)
         self.host = torch.empty(max_peers * self.stride, dtype=torch.uint8, pin_memory=True)
         self.dev = torch.empty(max_peers * self.stride, dtype=torch.uint8, device=batch.device)
-        self.values = torch.empty((max_peers, n, k), dtype=torch.float32, device=batch.device) if quantized else None
+        self.values: torch.Tensor | None = None  # fp32 copy of a quantised window, made by the first load that expands
         self._copied: torch.cuda.Event | None = None  # the last host-to-device copy out of `host`
         self._val_sizes = [batch.payload_rows(i) * k for i in range(len(batch))]
         self._idx_sizes = [v // 2 * 3 for v in self._val_sizes]
         self._threads = max(1, min(64, host_threads if host_threads else min(8, os.cpu_count() or 1)))
+        # norms: a PeerNorms whose first batch is `batch`; every load then leaves each peer's row figures there as
+        # soon as the peer's fp32 values are on the device, so the window's clip factors need no pass over them
+        if norms is not None and (norms.batches[0] is not batch or norms.max_peers < max_peers):
+            raise ValueError("norms: its first batch must be this stage's batch, its window at least as wide")
+        self.norms = norms
+        self.tables = None
 
     @torch.no_grad()
     def offload(self, n_peers: int) -> None:
@@ -1664,10 +1777,17 @@ class PayloadStage:
             return out_i, out_v
         lookup, shift = self._tables
         T = len(self.batch)
+        values = self._expanded()
         for p in range(n_peers):
-            dequantize_batch(self.batch, out_v[p].reshape(-1), None, self.k, out=self.values[p],
+            dequantize_batch(self.batch, out_v[p].reshape(-1), None, self.k, out=values[p],
                              tables=(lookup[p * T:(p + 1) * T], shift[p * T:(p + 1) * T]))
-        return out_i, [self.values[p] for p in range(n_peers)]
+        return out_i, [values[p] for p in range(n_peers)]
+
+    def _expanded(self) -> torch.Tensor:
+        if self.values is None:
+            self.values = torch.empty((self.max_peers, self.batch.total_chunks, self.k), dtype=torch.float32,
+                                      device=self.dev.device)
+        return self.values
 
     def regions(self, p: int) -> tuple[torch.Tensor, torch.Tensor]:
         """Peer p's place in the device buffer: (packed indices, values (n, k) or codes).  The peers'
@@ -1744,11 +1864,13 @@ class PayloadStage:
                 torch.cat([idxs[i][p].reshape(-1) for i in range(T)], out=ri)
                 torch.cat([vals[i][p].reshape(-1) for i in range(T)], out=rv)
         out_i, out_v = [], []
+        self.tables = None
         for p in range(P):
             ri, rv = self._regions(self.dev, p)
             out_i.append(ri)
             out_v.append(rv.view(-1, self.k))
         if not self.quantized:
+            self._note_arrivals(out_v)
             return out_i, out_v
         if quant_params is None or len(quant_params) != T or any(len(q) != P for q in quant_params):
             raise IndexError("quant_params must hold one entry per parameter and peer")
@@ -1756,11 +1878,19 @@ class PayloadStage:
             self.tables = dequantised_tables(quant_params, self.dev.device)
             return out_i, out_v
         lookup, shift, n_bins = _qparam_tables([quant_params[i][p] for p in range(P) for i in range(T)], self.dev.device)
+        values = self._expanded()
         for p in range(P):
-            dequantize_batch(self.batch, out_v[p].reshape(-1), None, self.k, out=self.values[p],
+            dequantize_batch(self.batch, out_v[p].reshape(-1), None, self.k, out=values[p],
                              tables=(lookup[p * T:(p + 1) * T], shift[p * T:(p + 1) * T]))
         self._tables = (lookup, shift)  # alive until the launches above have run
-        return out_i, [self.values[p] for p in range(P)]
+        self._note_arrivals([values[p] for p in range(P)])
+        return out_i, [values[p] for p in range(P)]
+
+    def _note_arrivals(self, vals: Sequence[torch.Tensor]) -> None:
+        if self.norms is not None:
+            rest = [None] * (len(self.norms.batches) - 1)
+            for p, v in enumerate(vals):
+                self.norms.arrived(p, [v] + rest)
 
 
 @torch.no_grad()
@@ -1824,6 +1954,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "apply_decoded_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "apply_decoded_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "PeerNorms", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

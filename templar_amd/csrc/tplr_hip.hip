@@ -2482,8 +2482,132 @@ __global__ __launch_bounds__(1024) void k_segment_sumsq(const ValPtrs vp, int P,
     }
 }
 
+// Sum of squares of every row of k values of a flat payload: what a peer's norms are made of, taken once,
+// when the payload arrives, so that the clip factors of a window cost a pass over one float per row instead
+// of a second pass over the values.  The order of the additions is fixed: value j's square sits in lane j of
+// a group of kW lanes (the power of two that holds k; zero where j >= k; rows longer than 64: lane j first adds
+// the squares of values j, j + 64, ... in that order) and lane j adds lane j ^ off for off = kW/2 ... 1.
+// 64 / kW rows per wave instruction, eight of them in flight per wave.
+struct RowSumPtrs {
+    float* out[TPLR_MAX_PEERS];
+};
+template <int kW>
+__global__ __launch_bounds__(256) void k_row_sumsq(const ValPtrs vp, const RowSumPtrs op, int k, int64_t n_rows) {
+    constexpr int kRows = 64 / kW;  // rows per trip of a wave
+    constexpr int kFlight = 8;
+    const int lane = threadIdx.x & 63;
+    const int j = lane & (kW - 1);
+    const float* __restrict__ val = vp.val[blockIdx.y];
+    float* __restrict__ out = op.out[blockIdx.y];
+    const int64_t waves = static_cast<int64_t>(gridDim.x) * 4;
+    const int64_t wave = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    const int64_t trips = (n_rows + kRows - 1) / kRows;
+    for (int64_t t0 = wave * kFlight; t0 < trips; t0 += waves * kFlight) {
+        float x[kFlight];
+#pragma unroll
+        for (int u = 0; u < kFlight; ++u) {
+            const int64_t row = (t0 + u) * kRows + lane / kW;
+            float acc = 0.f;
+            if (row < n_rows) {
+                if (kW < 64 || k <= 64) {
+                    const float v = j < k ? __builtin_nontemporal_load(val + row * k + j) : 0.f;
+                    acc = v * v;
+                } else {
+                    for (int e = j; e < k; e += 64) {
+                        const float v = __builtin_nontemporal_load(val + row * k + e);
+                        acc = __builtin_fmaf(v, v, acc);
+                    }
+                }
+            }
+            x[u] = acc;
+        }
+#pragma unroll
+        for (int u = 0; u < kFlight; ++u) {
+#pragma unroll
+            for (int off = kW / 2; off > 0; off >>= 1) x[u] += __shfl_xor(x[u], off);
+            const int64_t row = (t0 + u) * kRows + lane / kW;
+            if (j == 0 && row < n_rows) out[row] = x[u];
+        }
+    }
+}
+
+// The same figures with 16-byte loads, for rows of k <= 64 values with k a multiple of four that start on
+// 16-byte boundaries: kW / 4 lanes per row, lane m holds the squares of values 4m .. 4m + 3 (zero past k).  The
+// tree above pairs value j with value j ^ off: for off >= 4 that is the same component of lane m ^ (off / 4),
+// for off = 2 and 1 components of the lane itself - the same additions in the same order, so the same bits.
+template <int kW>
+__global__ __launch_bounds__(256) void k_row_sumsq_vec(const ValPtrs vp, const RowSumPtrs op, int k, int64_t n_rows) {
+    constexpr int kLanes = kW / 4;      // lanes per row
+    constexpr int kRows = 64 / kLanes;  // rows per trip of a wave
+    constexpr int kFlight = 8;
+    const int lane = threadIdx.x & 63;
+    const int m = lane & (kLanes - 1);
+    const float* __restrict__ val = vp.val[blockIdx.y];
+    float* __restrict__ out = op.out[blockIdx.y];
+    const int64_t waves = static_cast<int64_t>(gridDim.x) * 4;
+    const int64_t wave = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    const int64_t trips = (n_rows + kRows - 1) / kRows;
+    const bool in_row = 4 * m < k;
+    for (int64_t t0 = wave * kFlight; t0 < trips; t0 += waves * kFlight) {
+        v4f x[kFlight];
+#pragma unroll
+        for (int u = 0; u < kFlight; ++u) {
+            const int64_t row = (t0 + u) * kRows + lane / kLanes;
+            x[u] = (v4f){0.f, 0.f, 0.f, 0.f};
+            if (row < n_rows && in_row)
+                x[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(val + row * k) + m);
+        }
+#pragma unroll
+        for (int u = 0; u < kFlight; ++u) {
+            v4f q = x[u] * x[u];
+#pragma unroll
+            for (int off = kLanes / 2; off > 0; off >>= 1) {
+                q.x += __shfl_xor(q.x, off);
+                q.y += __shfl_xor(q.y, off);
+                q.z += __shfl_xor(q.z, off);
+                q.w += __shfl_xor(q.w, off);
+            }
+            const float r = (q.x + q.z) + (q.y + q.w);
+            const int64_t row = (t0 + u) * kRows + lane / kLanes;
+            if (m == 0 && row < n_rows) out[row] = r;
+        }
+    }
+}
+
+// Partial sums over a tensor's rows of such per-row figures, in double: block (tensor t, peer p, slice s) adds
+// the rows of slice s of tensor t (thread i the rows i, i + 256, ... in that order, then the fixed tree of
+// block256_sum_f64) into partial[(t * P + p) * S + s].
+struct RowSumConstPtrs {
+    const float* in[TPLR_MAX_PEERS];
+};
+__global__ __launch_bounds__(256) void k_rowsum_partials(const RowSumConstPtrs rp, int P, int S,
+                                                         const tplr_tensor_desc* __restrict__ table,
+                                                         double* __restrict__ partial) {
+    __shared__ double part[4];
+    const int tp = blockIdx.x / S, sl = blockIdx.x - tp * S;
+    const int t = tp / P, p = tp - t * P;
+    const tplr_tensor_desc d = table[t];
+    const int64_t n = static_cast<int64_t>(d.x_chunks) * d.y_chunks;
+    const int64_t c0 = n * sl / S, c1 = n * (sl + 1) / S;
+    const float* __restrict__ s = rp.in[p] + d.chunk_begin;
+    double acc = 0.0;
+    int64_t i = c0 + threadIdx.x;
+    for (; i + 768 < c1; i += 1024) {  // four independent loads in flight, added in the order of the rows
+        const float a0 = s[i], a1 = s[i + 256], a2 = s[i + 512], a3 = s[i + 768];
+        acc += static_cast<double>(a0);
+        acc += static_cast<double>(a1);
+        acc += static_cast<double>(a2);
+        acc += static_cast<double>(a3);
+    }
+    for (; i < c1; i += 256) acc += static_cast<double>(s[i]);
+    acc = block256_sum_f64(acc, part, threadIdx.x);
+    if (threadIdx.x == 0) partial[blockIdx.x] = acc;
+}
+
 // one block per tensor: scale[t][p] = min(1, med_t / (norm[t][p] + 1e-8))
-__global__ __launch_bounds__(128) void k_clip_scales(const float* __restrict__ norm, int P, int n_partials,
+// Partial: float (partial sums of squares added in float) or double (added in double, the norm rounded once)
+template <typename Partial>
+__global__ __launch_bounds__(128) void k_clip_scales(const Partial* __restrict__ norm, int P, int n_partials,
                                                      float* __restrict__ scale, float* __restrict__ median) {
     __shared__ float nv[TPLR_MAX_PEERS];
     __shared__ float med;
@@ -2491,12 +2615,15 @@ __global__ __launch_bounds__(128) void k_clip_scales(const float* __restrict__ n
     const int64_t off = static_cast<int64_t>(blockIdx.x) * P;
     if (i < P) {
         if (n_partials > 0) {  // partial sums of squares, added in order
-            const float* ps = norm + (off + i) * n_partials;
-            float tot = 0.f;
+            const Partial* ps = norm + (off + i) * n_partials;
+            Partial tot = 0;
             for (int s = 0; s < n_partials; ++s) tot += ps[s];
-            nv[i] = __builtin_sqrtf(tot);
+            if constexpr (sizeof(Partial) == 4)
+                nv[i] = __builtin_sqrtf(tot);
+            else
+                nv[i] = static_cast<float>(__builtin_sqrt(tot));
         } else {
-            nv[i] = norm[off + i];
+            nv[i] = static_cast<float>(norm[off + i]);
         }
     }
     __syncthreads();
@@ -2983,6 +3110,30 @@ __global__ __launch_bounds__(256) void k_code_sumsq4(const CodePtrs cp, int P, i
 __global__ __launch_bounds__(256) void k_calib_copy(const v4f* __restrict__ src, v4f* __restrict__ dst, int64_t n16) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+// Plain fill over a linear address range (16 bytes per lane per step): the write rate of the memory system with
+// the friendliest access pattern there is, the figure the aggregate's chunk-pattern stores are held against.
+// kPattern 0: grid-stride, neighbouring workgroups write neighbouring kilobytes; 1: the same with streaming stores;
+// 2: every wave walks a contiguous span of its own, one kilobyte per step, as a persistent kernel would.
+template <int kPattern>
+__global__ __launch_bounds__(256) void k_calib_fill(v4f* __restrict__ dst, int64_t n16, float value) {
+    const v4f v = {value, value, value, value};
+    if constexpr (kPattern == 2) {
+        const int64_t waves = static_cast<int64_t>(gridDim.x) * 4;
+        const int64_t wave = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+        const int64_t per = ((n16 + waves - 1) / waves + 63) & ~int64_t{63};
+        const int64_t a = wave * per, b = a + per < n16 ? a + per : n16;
+        for (int64_t i = a + (threadIdx.x & 63); i < b; i += 64) dst[i] = v;
+    } else {
+        const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+        for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += stride) {
+            if constexpr (kPattern == 1)
+                __builtin_nontemporal_store(v, dst + i);
+            else
+                dst[i] = v;
+        }
+    }
 }
 
 // The memory side of the fast aggregate alone: same grid, same chunk ranges, the same payload loads and the
@@ -3843,8 +3994,72 @@ int tplr_clip_scales_batch(const float* d_norm, int n_tensors, int n_peers, int 
                            float* d_median, void* stream) {
     if (!d_norm || !d_scale || n_peers < 1 || n_tensors < 1 || n_partials < 0) return TPLR_E_BADARG;
     if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
-    hipLaunchKernelGGL(k_clip_scales, dim3(n_tensors), dim3(128), 0, static_cast<hipStream_t>(stream), d_norm, n_peers,
-                       n_partials, d_scale, d_median);
+    hipLaunchKernelGGL(k_clip_scales<float>, dim3(n_tensors), dim3(128), 0, static_cast<hipStream_t>(stream), d_norm,
+                       n_peers, n_partials, d_scale, d_median);
+    return launch_status();
+}
+
+int tplr_row_sumsq(const float* const* h_val, int n_peers, int k, int64_t n_rows, float* const* h_row_sumsq,
+                   void* stream) {
+    if (!h_val || !h_row_sumsq || n_peers < 1 || k < 1 || k > TPLR_MAX_ROW || n_rows < 0) return TPLR_E_BADARG;
+    if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
+    if (n_rows == 0) return 0;
+    ValPtrs vp;
+    RowSumPtrs op;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        vp.val[p] = p < n_peers ? h_val[p] : nullptr;
+        op.out[p] = p < n_peers ? h_row_sumsq[p] : nullptr;
+        if (p < n_peers && (!vp.val[p] || !op.out[p])) return TPLR_E_BADARG;
+    }
+    int w = 2;
+    while (w < k && w < 64) w <<= 1;
+    bool vec = w >= 4 && k <= 64 && (k & 3) == 0;
+    for (int p = 0; p < n_peers; ++p) vec = vec && (reinterpret_cast<uintptr_t>(h_val[p]) & 15) == 0;
+    const int rows_per_trip = vec ? 256 / w : 64 / w;
+    const int64_t trips = (n_rows + rows_per_trip - 1) / rows_per_trip;
+    // a wave takes eight trips per round; one resident round of four-wave workgroups is enough for a long list
+    int64_t blocks = (trips + 31) / 32;
+    const int64_t cap = (256 * 8 + n_peers - 1) / n_peers;
+    blocks = blocks < 1 ? 1 : blocks > cap ? cap : blocks;
+    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(n_peers)), block(256);
+    const hipStream_t on = static_cast<hipStream_t>(stream);
+    if (vec) {
+        switch (w) {
+            case 4: hipLaunchKernelGGL(k_row_sumsq_vec<4>, grid, block, 0, on, vp, op, k, n_rows); break;
+            case 8: hipLaunchKernelGGL(k_row_sumsq_vec<8>, grid, block, 0, on, vp, op, k, n_rows); break;
+            case 16: hipLaunchKernelGGL(k_row_sumsq_vec<16>, grid, block, 0, on, vp, op, k, n_rows); break;
+            case 32: hipLaunchKernelGGL(k_row_sumsq_vec<32>, grid, block, 0, on, vp, op, k, n_rows); break;
+            default: hipLaunchKernelGGL(k_row_sumsq_vec<64>, grid, block, 0, on, vp, op, k, n_rows); break;
+        }
+        return launch_status();
+    }
+    switch (w) {
+        case 2: hipLaunchKernelGGL(k_row_sumsq<2>, grid, block, 0, on, vp, op, k, n_rows); break;
+        case 4: hipLaunchKernelGGL(k_row_sumsq<4>, grid, block, 0, on, vp, op, k, n_rows); break;
+        case 8: hipLaunchKernelGGL(k_row_sumsq<8>, grid, block, 0, on, vp, op, k, n_rows); break;
+        case 16: hipLaunchKernelGGL(k_row_sumsq<16>, grid, block, 0, on, vp, op, k, n_rows); break;
+        case 32: hipLaunchKernelGGL(k_row_sumsq<32>, grid, block, 0, on, vp, op, k, n_rows); break;
+        default: hipLaunchKernelGGL(k_row_sumsq<64>, grid, block, 0, on, vp, op, k, n_rows); break;
+    }
+    return launch_status();
+}
+
+int tplr_clip_scales_rows(const float* const* h_row_sumsq, int n_peers, const tplr_tensor_desc* d_desc, int n_tensors,
+                          int n_slices, double* d_partial, float* d_scale, float* d_median, void* stream) {
+    if (!h_row_sumsq || !d_desc || !d_partial || !d_scale || n_peers < 1 || n_tensors < 1 || n_slices < 1)
+        return TPLR_E_BADARG;
+    if (n_peers > TPLR_MAX_PEERS) return TPLR_E_TOOMANY;
+    if (static_cast<int64_t>(n_tensors) * n_peers * n_slices > 0x7fffffff) return TPLR_E_TOOMANY;
+    RowSumConstPtrs rp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        rp.in[p] = p < n_peers ? h_row_sumsq[p] : nullptr;
+        if (p < n_peers && !rp.in[p]) return TPLR_E_BADARG;
+    }
+    const hipStream_t on = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(k_rowsum_partials, dim3(static_cast<unsigned>(n_tensors) * n_peers * n_slices), dim3(256), 0, on,
+                       rp, n_peers, n_slices, d_desc, d_partial);
+    hipLaunchKernelGGL(k_clip_scales<double>, dim3(n_tensors), dim3(128), 0, on, d_partial, n_peers, n_slices, d_scale,
+                       d_median);
     return launch_status();
 }
 
@@ -4103,6 +4318,22 @@ int tplr_calib_copy(const void* d_src, void* d_dst, int64_t n_bytes, void* strea
     if (n_bytes == 0) return 0;
     hipLaunchKernelGGL(k_calib_copy, dim3(256 * 16), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const v4f*>(d_src), static_cast<v4f*>(d_dst), n_bytes >> 4);
+    return launch_status();
+}
+
+int tplr_calib_fill(void* d_dst, int64_t n_bytes, int pattern, void* stream) {
+    if (!d_dst || n_bytes < 0 || (n_bytes & 15) || pattern < 0 || pattern > 2) return TPLR_E_BADARG;
+    if (reinterpret_cast<uintptr_t>(d_dst) & 15) return TPLR_E_BADARG;
+    if (n_bytes == 0) return 0;
+    const dim3 grid(256 * 8), block(256);  // one resident round: eight workgroups of four waves per CU
+    const hipStream_t on = static_cast<hipStream_t>(stream);
+    v4f* dst = static_cast<v4f*>(d_dst);
+    if (pattern == 0)
+        hipLaunchKernelGGL(k_calib_fill<0>, grid, block, 0, on, dst, n_bytes >> 4, 1.f);
+    else if (pattern == 1)
+        hipLaunchKernelGGL(k_calib_fill<1>, grid, block, 0, on, dst, n_bytes >> 4, 1.f);
+    else
+        hipLaunchKernelGGL(k_calib_fill<2>, grid, block, 0, on, dst, n_bytes >> 4, 1.f);
     return launch_status();
 }
 
