@@ -304,10 +304,16 @@ int tplr_ef_step_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc
  * every parameter once and never holds the dense gradient: param <- param - decode(decompress(payload)), every
  * value of tensor t times d_factor[t] first (pass alpha * clip factor; the transform is linear, so this differs
  * from scaling the decoded tensor by rounding only; NULL = 1).  The kernels are those of
- * tplr_ef_subtract_batch; k <= 64; repeated indices in a row as in decompress (the mean of those entries). */
+ * tplr_ef_subtract_batch; k <= 64; repeated indices in a row as in decompress (the mean of those entries).
+ * d_nonfinite (nullable): n_tensors ints, zeroed by the caller.  The reference tests the decoded gradient for
+ * NaN and infinities before it touches the parameter and rejects the peer (validator.py:3646-3660, :3677-3680).
+ * Here a chunk whose decoded values are not all finite is left unwritten - the parameter keeps its bits there -
+ * and d_nonfinite[t] becomes 1 for its tensor; every other chunk is updated, so a caller that finds a flag set
+ * rejects the peer and takes the update back with a second call with the factors negated (the same chunks are
+ * skipped again).  NULL: no test, everything is subtracted. */
 int tplr_apply_decoded_batch(const uint8_t* d_idx12, const float* d_val, const float* d_factor, int k,
-                             const tplr_tensor_desc* d_param_desc, int n_tensors, int64_t total_chunks, int use_dct,
-                             void* stream);
+                             const tplr_tensor_desc* d_param_desc, int n_tensors, int64_t total_chunks,
+                             int use_dct, int32_t* d_nonfinite, void* stream);
 
 /* ---- validator side: checks on the packed index streams ------------------------------
  * For up to 32 peers whose flat payloads share one row layout (d_desc: n_tensors descriptors, of

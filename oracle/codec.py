@@ -252,16 +252,20 @@ def dequantize(q, qparams) -> np.ndarray:
 
 # ---------------------------------------------------------------- miner step (src/tplr/neurons.py:147-171)
 def error_feedback_step(ef, grad, decay: float, topk: int, *, use_dct: bool = True, quant_bins: int = 0,
-                        quant_range: float = 6.0, coef_override=None):
+                        quant_range: float = 6.0, coef_override=None, null_round: bool = False):
     """One parameter's momentum / compress / error-feedback update, line by line:
     ef.mul_(decay); ef.add_(grad) (:151-152); encode (:155); compress (:157-159); decompress (:164-166);
     decode (:169); ef.sub_(decoded) (:171).  `quant_bins` > 0 runs the values through the statistical
     quantiser as compress/decompress do when the compressor quantises.  `coef_override`, if given,
     replaces the encoded tensor that is compressed (to compare selections on another
-    implementation's coefficients).  Returns (ef_accumulated, packed idx, val, ef_new)."""
+    implementation's coefficients).  `null_round` zeroes the error feedback instead of updating it (:148-149).
+    Returns (ef_accumulated, packed idx, val, ef_new)."""
     ef = _c(ef, np.float32).copy()
-    ef *= np.float32(decay)           # one rounding
-    ef += _c(grad, np.float32)        # a second one
+    if null_round:
+        ef[...] = 0.0                     # :149
+    else:
+        ef *= np.float32(decay)           # one rounding (:151)
+        ef += _c(grad, np.float32)        # a second one (:152)
     enc = encode2d(ef, use_dct=use_dct) if coef_override is None else _c(coef_override, np.float32)
     idx12, val, xshape, totalk = compress(enc, topk)
     sent = val

@@ -1195,7 +1195,7 @@ def aggregate_mean_normalised_batch(out: TensorBatch, idxs: Sequence[torch.Tenso
 @torch.no_grad()
 def apply_decoded_batch(params: TensorBatch, idx12: torch.Tensor, val: torch.Tensor, k: int, *, alpha: float = 1.0,
                         clip: torch.Tensor | None = None, clip_norm: torch.Tensor | None = None,
-                        use_dct: bool = True) -> None:
+                        use_dct: bool = True, on_nonfinite: str = "raise") -> "torch.Tensor | None":
     """param <- param - alpha * decode(decompress(payload * clip)) for every parameter of the set in one launch:
     the validator's per-peer evaluation update (neurons/validator.py:3595-3737, update_model_with_gradient: the
     evaluated peer's values times its clip factor, decompress, decode, p.data.sub_(decoded, alpha=lr *
@@ -1203,7 +1203,19 @@ def apply_decoded_batch(params: TensorBatch, idx12: torch.Tensor, val: torch.Ten
     (the validator's clip_norm_dict, one per parameter): the factors min(1, clip_norm_t / (norm_t + 1e-8)) of
     validator.py:3608-3612 are formed here from the payload's own per-parameter norms; or `clip`: (T,) ready
     factors; or neither.  alpha and the factors ride on the values (the transform is linear), so the dense gradient
-    is never formed and every parameter is read and written once.  k <= 64."""
+    is never formed and every parameter is read and written once.  k <= 64.
+
+    The reference tests every decoded gradient for NaN and infinities before it subtracts it and raises
+    ValueError for the peer (validator.py:3646-3660, :3677-3680).  The launch makes the same test on the decoded
+    values (alpha and the clip factor included, so an overflow of that product counts) chunk by chunk: a chunk
+    that holds a non-finite value is not subtracted - the parameter keeps its bits there.  on_nonfinite="raise"
+    (default) then raises the reference's ValueError, at the cost of one synchronisation, as the reference's own
+    test; every chunk that decoded to finite values HAS been subtracted by then (the reference, too, has
+    updated the parameters that precede the offending one), and the same call with `alpha` negated takes the
+    update back up to rounding, skipping the same chunks.  "flags" returns the (T,) int32 tensor of flags without
+    synchronising (1: some chunk of that parameter was skipped); "ignore" makes no test and subtracts everything."""
+    if on_nonfinite not in ("raise", "flags", "ignore"):
+        raise ValueError(f"on_nonfinite must be 'raise', 'flags' or 'ignore', got {on_nonfinite!r}")
     lib = _lib.load()
     T, n, dev = len(params), params.total_chunks, params.device
     if idx12.dtype != torch.uint8:
@@ -1232,10 +1244,18 @@ def apply_decoded_batch(params: TensorBatch, idx12: torch.Tensor, val: torch.Ten
             if clip.numel() != T:
                 raise IndexError(f"{clip.numel()} clip factors for {T} parameters")
             factor = factor * clip.to(device=dev, dtype=torch.float32).reshape(T)
+    flags = None if on_nonfinite == "ignore" else torch.zeros(T, dtype=torch.int32, device=dev)
     with _on(dev):
         st = lib.tplr_apply_decoded_batch(_ptr(idx12), _ptr(val), _ptr(factor), k, _ptr(params.table), T, n, int(use_dct),
-                                          _stream(dev))
+                                          _ptr(flags), _stream(dev))
     _lib.check(st, "tplr_apply_decoded_batch")
+    if on_nonfinite == "raise":
+        bad = torch.nonzero(flags).reshape(-1).tolist()  # synchronises, as the reference's isnan().any() does
+        if bad:
+            raise ValueError(f"Invalid gradient: the decoded gradient of parameter {bad[0]} contains NaN/Inf "
+                             f"({len(bad)} of {T} parameters affected; their non-finite chunks were not applied)")
+        return None
+    return flags
 
 
 @torch.no_grad()

@@ -6,8 +6,6 @@
 #include <string.h>
 
 #include <mutex>
-#include <thread>
-#include <vector>
 
 #include "../../include/tplr_hip.h"
 #include "tplr_device.h"
@@ -703,7 +701,10 @@ struct Counters {
 // Generic path (kUnits == 0): any k and peer count, entries loaded where they are used.
 // kSubtract (fast path with the transform only): the destination receives destination - result
 // instead of the result (the error-feedback update of src/tplr/neurons.py:171); its rows are
-// requested before the second pass and arrive during it.
+// requested before the second pass and arrive during it.  With `guard` (one int per tensor, zeroed by the
+// caller) a chunk whose result holds a NaN or an infinity is not subtracted - its destination keeps its
+// bits - and guard[tensor] becomes 1: the validator's check of the decoded gradient before
+// p.data.sub_ (neurons/validator.py:3646-3660).
 // kStrided (fast path): the peers' payloads are equally spaced in memory - peer p's index bytes at
 // pp.idx[0] + p * stride_idx, its values at pp.val[0] + p * stride_val floats, as a staged window lays
 // them out - so every payload address is scalar arithmetic on two base pointers instead of a pair of
@@ -729,7 +730,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                                                             int64_t first, int64_t total, int reduce_mode,
                                                             int options, float* __restrict__ sumsq,
                                                             int64_t stride_idx, int64_t stride_val,
-                                                            const float* __restrict__ deq) {
+                                                            const float* __restrict__ deq,
+                                                            int32_t* __restrict__ guard) {
     static_assert(!kCodes || (kUnits > 0 && !kUseDct && !kSubtract), "codes are served by the fast path without the transform");
     static_assert(kWideK == 0 || (kCodes && kStrided && (kWideK == 32 || kWideK == 64)), "wide loads: codes, equally spaced payloads");
     // this launch covers the chunks first .. first + total - 1 of the batch
@@ -758,6 +760,17 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         } else if (lane_ == 0 && !skip) {
             sumsq[g] = ss;
         }
+    };
+    // kSubtract with a guard: true (wave-uniform) when the result in registers holds a NaN or an infinity, and
+    // then the chunk's tensor is flagged; x * 0 is zero for every finite x and NaN otherwise
+    auto guard_trips = [&](const float (&v)[64], int t) -> bool {
+        if (!kSubtract || !guard) return false;  // wave-uniform
+        float z = 0.f;
+#pragma unroll
+        for (int r = 0; r < 64; ++r) z = __builtin_fmaf(v[r], 0.0f, z);
+        const bool bad = __ballot(z != z) != 0;
+        if (bad && threadIdx.x == 0) guard[t] = 1;
+        return bad;
     };
     using Cnt = Counters<kCntBits>;
     // kPark: lanes and units without an entry scatter "coefficient 4096 + lane", which the address
@@ -1096,7 +1109,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             }
         }
         wave_lds_fence();
+        bool tripped = false;
         if constexpr (kSubtract) {
+            tripped = guard_trips(v, cs.t);
             const __amdgpu_buffer_rsrc_t rs = chunk_rsrc((const void*)dst, ld);
             const int ld4 = static_cast<int>(ld) * 4;
 #pragma unroll
@@ -1105,7 +1120,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
         chunk_stats(v, g, false);
         if (rows) {
-            store_chunk_rows(v, (void*)dst, ld, lane);
+            store_chunk_rows(v, (void*)dst, ld, lane, tripped);
         } else {
 #pragma unroll
             for (int q0 = 0; q0 < 16; ++q0)
@@ -1400,7 +1415,10 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                     }
                 }
             });
+            bool tripped = false;
             if constexpr (kSubtract) {
+                // (a chunk that is to be done again on the exact path holds claim marks: it is tested there)
+                if (!skip0) tripped = guard_trips(v, o0.t);
 #pragma unroll
                 for (int r = 0; r < 64; ++r) v[r] = before[r] - v[r];
             }
@@ -1412,7 +1430,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             repeat = 0;
             mean_pass();
             // a chunk that is to be done again is not stored: its descriptor gets a range of zero bytes
-            store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane, skip0);
+            store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane,
+                             skip0 || tripped);
             skip0 = skip1;
             o0 = o1;
             o1 = o2;
@@ -1786,8 +1805,11 @@ __global__ __launch_bounds__(64) void k_ef_subtract_sparse(const uint8_t* __rest
                                                            const float* __restrict__ val, int k,
                                                            const tplr_tensor_desc* __restrict__ table,
                                                            const tplr_tensor_desc single, int n_tensors,
-                                                           int64_t total, const float* __restrict__ factor) {
+                                                           int64_t total, const float* __restrict__ factor,
+                                                           int32_t* __restrict__ guard) {
     // factor (nullable): every value of tensor t times factor[t] before it is subtracted
+    // guard (nullable, one int per tensor, zeroed by the caller): a chunk with an entry that is NaN or infinite
+    // after the factor is left as it is and guard[tensor] becomes 1
     __shared__ uint16_t owner[4096];  // the last lane that named a position (never cleared: written before read)
     const int lane = threadIdx.x;
     int64_t g0, g1;
@@ -1826,7 +1848,12 @@ __global__ __launch_bounds__(64) void k_ef_subtract_sparse(const uint8_t* __rest
             }
             x = n > 1 ? sum / static_cast<float>(n) : sum;
         }
-        if (me >= 0 && first) {
+        bool tripped = false;
+        if (guard) {  // wave-uniform
+            tripped = __ballot(me >= 0 && (__builtin_bit_cast(uint32_t, x) & 0x7f800000u) == 0x7f800000u) != 0;
+            if (tripped && lane == 0) guard[c.t] = 1;
+        }
+        if (me >= 0 && first && !tripped) {
             gfloat* t = chunk0 + static_cast<int64_t>(me >> 6) * c.ld + (me & 63);
             *t = *t - x;
         }
@@ -3256,7 +3283,8 @@ template <typename Kernel>
 static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_scale, int n_peers, int k,
                             const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single, int n_tensors,
                             int64_t total, int reduce_mode, int normalise, float* d_sumsq, void* stream,
-                            int64_t stride_idx = 0, int64_t stride_val = 0, const float* d_deq = nullptr) {
+                            int64_t stride_idx = 0, int64_t stride_val = 0, const float* d_deq = nullptr,
+                            int32_t* d_guard = nullptr) {
     static int resident = 0;  // per kernel variant
     if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
     // a wave keeps one mark per chunk of its range (chunks to be done again on the exact path), so
@@ -3268,7 +3296,8 @@ static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_sc
         const int64_t need = ((count + 7) / 8) * 8;
         const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
         hipLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale, n_peers, k, d_desc,
-                           single, n_tensors, first, count, reduce_mode, normalise, d_sumsq, stride_idx, stride_val, d_deq);
+                           single, n_tensors, first, count, reduce_mode, normalise, d_sumsq, stride_idx, stride_val, d_deq,
+                           d_guard);
     }
     return launch_status();
 }
@@ -3311,71 +3340,7 @@ int tplr_unpack12(const uint8_t* d_packed, int64_t n, int64_t* d_idx, void* stre
     return launch_status();
 }
 
-int tplr_pack12_host(const int64_t* idx, int64_t n, uint8_t* packed, int64_t* bad) {
-    if (n < 0) return TPLR_E_BADARG;
-    if (n & 1) return TPLR_E_ODD;
-    if (n == 0) return 0;
-    if (!idx || !packed) return TPLR_E_BADARG;
-    int64_t worst = 0;
-    for (int64_t p = 0; p < n / 2; ++p) {
-        const int64_t a = idx[2 * p], b = idx[2 * p + 1];
-        worst = a > worst ? a : worst;
-        worst = b > worst ? b : worst;
-        const uint32_t w = (static_cast<uint32_t>(a) & 0xfffu) | ((static_cast<uint32_t>(b) & 0xfffu) << 12);
-        packed[3 * p] = static_cast<uint8_t>(w);
-        packed[3 * p + 1] = static_cast<uint8_t>(w >> 8);
-        packed[3 * p + 2] = static_cast<uint8_t>(w >> 16);
-    }
-    if (bad) *bad = worst > 4095 ? worst : 0;
-    return 0;
-}
-
-int tplr_gather_host(const void* const* h_src, const int64_t* h_bytes, int64_t n_parts, void* h_dst,
-                     int n_threads) {
-    if (n_parts < 0 || n_threads < 1 || n_threads > 64) return TPLR_E_BADARG;
-    if (n_parts == 0) return 0;
-    if (!h_src || !h_bytes || !h_dst) return TPLR_E_BADARG;
-    int64_t total = 0;
-    for (int64_t i = 0; i < n_parts; ++i) {
-        if (h_bytes[i] < 0 || (h_bytes[i] > 0 && !h_src[i])) return TPLR_E_BADARG;
-        total += h_bytes[i];
-    }
-    // every thread copies an equal share of the concatenated bytes, cutting parts where its share ends
-    auto work = [=](int t) {
-        const int64_t lo = total * t / n_threads, hi = total * (t + 1) / n_threads;
-        int64_t at = 0;
-        for (int64_t i = 0; i < n_parts && at < hi; at += h_bytes[i], ++i) {
-            const int64_t b = at > lo ? at : lo, e = at + h_bytes[i] < hi ? at + h_bytes[i] : hi;
-            if (b < e)
-                memcpy(static_cast<char*>(h_dst) + b, static_cast<const char*>(h_src[i]) + (b - at),
-                       static_cast<size_t>(e - b));
-        }
-    };
-    if (n_threads == 1 || total < (1 << 20)) {
-        for (int t = 0; t < n_threads; ++t) work(t);
-        return 0;
-    }
-    std::vector<std::thread> pool;
-    pool.reserve(n_threads - 1);
-    for (int t = 1; t < n_threads; ++t) pool.emplace_back(work, t);
-    work(0);
-    for (auto& th : pool) th.join();
-    return 0;
-}
-
-int tplr_unpack12_host(const uint8_t* packed, int64_t n, int64_t* idx) {
-    if (n < 0) return TPLR_E_BADARG;
-    if (n & 1) return TPLR_E_ODD;
-    if (n == 0) return 0;
-    if (!idx || !packed) return TPLR_E_BADARG;
-    for (int64_t p = 0; p < n / 2; ++p) {
-        const uint32_t w = packed[3 * p] | (static_cast<uint32_t>(packed[3 * p + 1]) << 8) |
-                           (static_cast<uint32_t>(packed[3 * p + 2]) << 16);
-        idx[2 * p] = w & 0xfffu;
-        idx[2 * p + 1] = w >> 12;
-    }
-    return 0;
-}
+// (tplr_pack12_host, tplr_unpack12_host and tplr_gather_host touch host memory only: tplr_host.cpp)
 
 static int check_2d(const void* a, const void* b, int64_t R, int64_t C) {
     if (!a || !b || R < 0 || C < 0) return TPLR_E_BADARG;
@@ -3549,7 +3514,7 @@ int tplr_ef_step_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc
 // dst <- dst - decode(decompress(payload)), every value of tensor t times d_factor[t] first (d_factor nullable)
 static int subtract_decoded(const uint8_t* d_idx12, const float* d_val, const float* d_factor, int k,
                             const tplr_tensor_desc* d_desc, int n_tensors, int64_t total_chunks, int use_dct,
-                            void* stream) {
+                            int32_t* d_guard, void* stream) {
     if (!d_idx12 || !d_val || !d_desc || n_tensors < 1 || total_chunks < 0 || k < 2 || (k & 1)) return TPLR_E_BADARG;
     if (k > 64) return TPLR_E_TOOMANY;  // the register-resident decode path
     if (total_chunks == 0) return 0;
@@ -3560,7 +3525,7 @@ static int subtract_decoded(const uint8_t* d_idx12, const float* d_val, const fl
         const int64_t need = ((total_chunks + 7) / 8) * 8;
         hipLaunchKernelGGL(k_ef_subtract_sparse, dim3(static_cast<unsigned>(need < resident ? need : resident)),
                            dim3(64), 0, static_cast<hipStream_t>(stream), d_idx12, d_val, k, d_desc, none, n_tensors,
-                           total_chunks, d_factor);
+                           total_chunks, d_factor, d_guard);
         return launch_status();
     }
     PeerPtrs pp;
@@ -3569,18 +3534,19 @@ static int subtract_decoded(const uint8_t* d_idx12, const float* d_val, const fl
     pp.val[0] = d_val;
     // (one peer: the factor table (n_tensors, 1) is the aggregate's clip-factor table)
     return launch_decode_as(k_decode_aggregate<true, 8, 4, true, true>, pp, d_factor, 1, k, d_desc, none, n_tensors,
-                            total_chunks, TPLR_REDUCE_MEAN, 0, nullptr, stream);
+                            total_chunks, TPLR_REDUCE_MEAN, 0, nullptr, stream, 0, 0, nullptr, d_guard);
 }
 
 int tplr_ef_subtract_batch(const uint8_t* d_idx12, const float* d_val, int k, const tplr_tensor_desc* d_ef_desc,
                            int n_tensors, int64_t total_chunks, int use_dct, void* stream) {
-    return subtract_decoded(d_idx12, d_val, nullptr, k, d_ef_desc, n_tensors, total_chunks, use_dct, stream);
+    return subtract_decoded(d_idx12, d_val, nullptr, k, d_ef_desc, n_tensors, total_chunks, use_dct, nullptr, stream);
 }
 
 int tplr_apply_decoded_batch(const uint8_t* d_idx12, const float* d_val, const float* d_factor, int k,
                              const tplr_tensor_desc* d_param_desc, int n_tensors, int64_t total_chunks, int use_dct,
-                             void* stream) {
-    return subtract_decoded(d_idx12, d_val, d_factor, k, d_param_desc, n_tensors, total_chunks, use_dct, stream);
+                             int32_t* d_nonfinite, void* stream) {
+    return subtract_decoded(d_idx12, d_val, d_factor, k, d_param_desc, n_tensors, total_chunks, use_dct, d_nonfinite,
+                            stream);
 }
 
 int tplr_ef_subtract_own_batch(const uint8_t* d_idx12, const float* d_sent, const float* d_own, int k,

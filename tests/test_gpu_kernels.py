@@ -884,7 +884,65 @@ def test_one_peers_payload_update_rejects_what_it_cannot_serve(dev):
     with pytest.raises(IndexError):
         tc.apply_decoded_batch(pb, idx12, val, 32, clip=torch.ones(2))
     assert _lib.load().tplr_apply_decoded_batch(idx12.data_ptr(), val.data_ptr(), None, 128, pb.table.data_ptr(), 1, 2, 1,
-                                                None) == _lib.TPLR_E_TOOMANY
+                                                None, None) == _lib.TPLR_E_TOOMANY
+    with pytest.raises(ValueError, match="on_nonfinite"):
+        tc.apply_decoded_batch(pb, idx12, val, 32, on_nonfinite="skip")
+
+
+@pytest.mark.parametrize("use_dct", [True, False])
+@pytest.mark.parametrize("kind", ["nan", "inf", "overflow"])
+def test_evaluation_update_refuses_a_non_finite_decoded_gradient(dev, use_dct, kind):
+    # neurons/validator.py:3646-3660, :3677-3680: a decoded gradient with a NaN or an infinity is never subtracted
+    # from the parameter and the peer is rejected with ValueError.  The launch leaves every chunk whose decoded
+    # values are not all finite as it was, flags its parameter, and updates the rest exactly as without the test.
+    shapes = [(128, 192), (64, 64), (256, 128)]
+    k, alpha = 32, 0.25
+    grads = [t3(s, 70 + i, row_scale=True).to(dev) for i, s in enumerate(shapes)]
+    batch = tc.TensorBatch(grads)
+    idx12, val = tc.encode_compress_batch(batch, k, use_dct=use_dct)
+    clip = torch.tensor([1.0, 0.5, 1.0], device=dev)
+    bad_row = batch.offsets[2] + 3  # chunk 3 of parameter 2
+    if kind == "nan":
+        val[bad_row, 5] = float("nan")
+    elif kind == "inf":
+        val[bad_row, 0] = float("-inf")
+    else:  # finite in the payload and as a decoded gradient, infinite once alpha is on it
+        val[bad_row, 7] = 3e38
+        alpha = 1e3
+    start = [torch.randn(s, device=dev) for s in shapes]
+    # what the update is without the test
+    plain = [p.clone() for p in start]
+    assert tc.apply_decoded_batch(tc.TensorBatch(plain), idx12, val, k, alpha=alpha, clip=clip, use_dct=use_dct,
+                                  on_nonfinite="ignore") is None
+    assert not torch.isfinite(plain[2]).all()   # the poison the reference's check exists for
+    # with it
+    guarded = [p.clone() for p in start]
+    flags = tc.apply_decoded_batch(tc.TensorBatch(guarded), idx12, val, k, alpha=alpha, clip=clip, use_dct=use_dct,
+                                   on_nonfinite="flags")
+    assert flags.tolist() == [0, 0, 1]
+    assert torch.equal(guarded[0], plain[0]) and torch.equal(guarded[1], plain[1])
+    y, x = 3 // (shapes[2][1] // 64), 3 % (shapes[2][1] // 64)
+    mask = torch.zeros(shapes[2], dtype=torch.bool, device=dev)
+    mask[64 * y:64 * y + 64, 64 * x:64 * x + 64] = True
+    assert torch.equal(guarded[2][mask], start[2][mask])         # the offending chunk keeps its bits
+    assert torch.equal(guarded[2][~mask], plain[2][~mask])       # every other chunk is updated as before
+    assert all(torch.isfinite(p).all() for p in guarded)
+    # the default raises as the reference does, and the opposite sign takes the update back
+    raised = [p.clone() for p in start]
+    with pytest.raises(ValueError, match="NaN/Inf"):
+        tc.apply_decoded_batch(tc.TensorBatch(raised), idx12, val, k, alpha=alpha, clip=clip, use_dct=use_dct)
+    assert all(torch.equal(a, b) for a, b in zip(raised, guarded))
+    with pytest.raises(ValueError):
+        tc.apply_decoded_batch(tc.TensorBatch(raised), idx12, val, k, alpha=-alpha, clip=clip, use_dct=use_dct)
+    back = max(float((p - p0).abs().max()) / float(p0.abs().max()) for p, p0 in zip(raised, start))
+    assert back <= TOL
+    # a clean payload raises nothing and equals the unguarded update bit for bit
+    val[bad_row] = 1e-3
+    a = [p.clone() for p in start]
+    b = [p.clone() for p in start]
+    tc.apply_decoded_batch(tc.TensorBatch(a), idx12, val, k, alpha=0.25, clip=clip, use_dct=use_dct)
+    tc.apply_decoded_batch(tc.TensorBatch(b), idx12, val, k, alpha=0.25, clip=clip, use_dct=use_dct, on_nonfinite="ignore")
+    assert all(torch.equal(p, q) for p, q in zip(a, b))
 
 
 # ---------------------------------------------------------------- validator side: index checks

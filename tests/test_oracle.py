@@ -426,3 +426,84 @@ def test_index_overlap_reference_known_answers():
             assert inter[i, j] == want and abs(frac[i, j] - want / (7 * 16)) < 1e-6
     assert orc.index_bounds(np.array([0, 63]), 64) is None and orc.index_bounds(np.array([1, 64, 70]), 64) == 64
 
+
+
+# ---------------------------------------------------------------- miner step (src/tplr/neurons.py:147-171)
+@pytest.mark.parametrize("use_dct", [True, False])
+@pytest.mark.parametrize("bins", [0, 4, 256])
+@pytest.mark.parametrize("null_round", [False, True])
+def test_error_feedback_step_against_the_torch_op_sequence(use_dct, bins, null_round):
+    # orc.error_feedback_step against the reference's own order of operations replayed with torch on the CPU
+    # (oracle/torch_cpu_path.py holds its compress.py halves; the neurons.py lines are written out here):
+    # :148-152 zero or decay-and-add, :155 encode, :157-159 compress (+ quantise), :164-166 decompress
+    # (+ de-quantise), :169 decode, :171 subtract
+    torch.manual_seed(7)
+    R, Cc, k, decay = 128, 192, 32, 0.95
+    ef0 = torch.randn(R, Cc) * 1e-3
+    grad = torch.distributions.StudentT(3.0).sample((R, Cc)) * 1e-3
+    b64 = tcp.basis(64)
+    ef = ef0.clone()
+    if null_round:
+        ef.zero_()
+    else:
+        ef.mul_(decay)
+        ef.add_(grad)
+    enc = tcp.encode(ef, 64, 64, b64[0], b64[0], use_dct=use_dct)
+    idx12, val, xshape, totalk = tcp.compress(enc, k)
+    sent = val
+    if bins:
+        q, qp = tcp.quantize(val, bins, 6.0)
+        sent = tcp.dequantize(q, qp)
+    new = ef - tcp.decode(tcp.decompress(idx12, sent, xshape, totalk), b64[1], b64[1], use_dct=use_dct)
+
+    got_acc, got_idx, got_val, got_new = orc.error_feedback_step(ef0.numpy(), grad.numpy(), decay, k, use_dct=use_dct,
+                                                                 quant_bins=bins, null_round=null_round)
+    assert np.array_equal(got_acc, ef.numpy())        # two roundings, as mul_ then add_; zeros on a null round
+    if null_round:
+        # nothing to select from: every chunk sends zeros and the error feedback stays zero
+        assert not got_val.any() and not got_new.any() and not new.any()
+        return
+    scale = float(ef.abs().max())
+    if use_dct:
+        # with the oracle's own transform the selections are made on coefficients that differ from torch's in
+        # their last bits: the sent sets agree wherever the k-th and (k+1)-th magnitudes are further apart
+        want_idx = tcp.unpack12(idx12, val.shape).numpy().reshape(-1, k)
+        mine = orc.unpack12(got_idx, (want_idx.shape[0], k))
+        assert np.mean([set(a) == set(b) for a, b in zip(want_idx.tolist(), mine.tolist())]) > 0.9
+        # on torch's coefficients (identical inputs to the selection) everything downstream is pinned: the same
+        # bytes and values, and the same remainder to fp32 tolerance
+        _, got_idx, got_val, got_new = orc.error_feedback_step(ef0.numpy(), grad.numpy(), decay, k, use_dct=True,
+                                                               quant_bins=bins, coef_override=enc.numpy())
+        tol = 1e-5
+    else:
+        tol = 1e-6  # no transform: only the subtraction rounds
+    assert np.array_equal(got_idx, idx12.numpy()) and np.array_equal(got_val.reshape(-1), val.numpy().reshape(-1))
+    assert np.abs(got_new - new.numpy()).max() <= tol * scale
+
+
+def test_error_feedback_step_closed_form_against_scipy():
+    # ef_new = ef_acc - IDCT(top-k(DCT(ef_acc))) with scipy's orthonormal transforms and a brute-force selection:
+    # the remainder has nothing left at the sent coefficients and everything at the others
+    rng = np.random.default_rng(3)
+    ef0 = (rng.standard_normal((64, 128)) * 1e-3).astype(np.float32)
+    grad = (rng.standard_t(3, (64, 128)) * 1e-3).astype(np.float32)
+    decay, k = 0.9, 16
+    acc, idx12, val, new = orc.error_feedback_step(ef0, grad, decay, k, use_dct=True)
+    want_acc = (ef0 * np.float32(decay) + grad).astype(np.float32)
+    assert np.array_equal(acc, want_acc)
+    chunks = want_acc.astype(np.float64).reshape(1, 64, 2, 64).transpose(0, 2, 1, 3)
+    coef = scipy.fft.dctn(chunks, axes=(-2, -1), norm="ortho").reshape(-1, 4096)
+    keep = np.zeros_like(coef)
+    order = np.argsort(-np.abs(coef), axis=1, kind="stable")[:, :k]
+    np.put_along_axis(keep, order, np.take_along_axis(coef, order, 1), 1)
+    recon = scipy.fft.idctn(keep.reshape(1, 2, 64, 64), axes=(-2, -1), norm="ortho")
+    want_new = chunks - recon
+    want_new = want_new.transpose(0, 2, 1, 3).reshape(64, 128)
+    assert np.abs(new - want_new).max() <= 1e-5 * np.abs(want_acc).max()
+    # what was sent: the k largest coefficients of each chunk, by index set and by value
+    mine = orc.unpack12(idx12, (2, k))
+    assert all(set(a) == set(b) for a, b in zip(mine.tolist(), order.tolist()))
+    assert np.allclose(np.sort(val.reshape(2, k), 1), np.sort(np.take_along_axis(coef, order, 1), 1), atol=1e-5 * np.abs(coef).max())
+    # the remainder's own transform is zero at the sent coefficients
+    left = scipy.fft.dctn(new.astype(np.float64).reshape(1, 64, 2, 64).transpose(0, 2, 1, 3), axes=(-2, -1), norm="ortho").reshape(-1, 4096)
+    assert np.abs(np.take_along_axis(left, order, 1)).max() <= 2e-5 * np.abs(coef).max()
