@@ -557,8 +557,9 @@ def main():
         params = [torch.zeros_like(o) for o in outs]
         pb = tc.TensorBatch(params)
         clip0 = scale.reshape(len(out_batch), -1)[:, 0].contiguous()
-        ev_ms, _ = event_ms(lambda: tc.apply_decoded_batch(pb, idxs[0], vals[0], k, alpha=0.01, clip=clip0, use_dct=DCT),
-                            agg_steps, 2)
+        # (the per-parameter non-finite flags are left on the device: a caller reads them once per peer)
+        ev_ms, _ = event_ms(lambda: tc.apply_decoded_batch(pb, idxs[0], vals[0], k, alpha=0.01, clip=clip0, use_dct=DCT,
+                                                           on_nonfinite="flags"), agg_steps, 2)
 
         def decode_then_subtract():
             tc.batch_decompress_decode_batch(out_batch, idxs[:1], vals[:1], k, scale=clip0.reshape(-1, 1), use_dct=DCT)

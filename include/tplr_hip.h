@@ -10,6 +10,12 @@
  *     work is enqueued on it and the call returns without synchronising;
  *   - return value: 0 = ok, negative = TPLR_E_* (bad argument, nothing launched),
  *     positive = a hipError_t from the launch;
+ *   - the persistent kernels' grid sizes (one resident round of workgroups, from the occupancy
+ *     calculator) are worked out on an entry point's first call and kept per process in plain
+ *     statics: the figure belongs to the device that was current then, and first calls racing
+ *     on several threads merely compute it twice.  A process that drives GPUs of different sizes
+ *     would launch the first one's grid on all of them (correct, since every kernel splits the
+ *     work by its own grid size, but not a full round on the larger device);
  *   - "chunk" = one 64x64 fp32 tile of a 2-D tensor, stored row-major inside the
  *     chunked layout (Y, X, 64, 64); flat index inside a chunk = row*64 + col
  *     (reference: rearrange "y x h w -> y x (h w)", src/tplr/compress.py:402-403);

@@ -1563,8 +1563,14 @@ def check_compressed_indices(param_name: str, idxs, totalk: int, allowed_topk: i
 
 def _qparam_tables(qparams: Sequence[QuantParamsT], dev: torch.device) -> tuple[torch.Tensor, torch.Tensor, int]:
     """(rows, n_bins) lookups and (rows,) shifts of a list of quant_params 5-tuples on `dev`: stacked
-    where they live, moved once."""
+    where they live, moved once.  The reference de-quantises to `(lookup[code] + shift).to(orig_dtype)`
+    (src/tplr/compress.py:641-643): a tuple whose fifth entry is not float32 gets its row as that sum rounded
+    through that dtype, with a zero shift, so that the kernels' fp32 `lookup[code] + shift` gives the rounded
+    value exactly.  All tuples must come from quantisers of one size."""
     n_bins = int(qparams[0][3].numel())
+    if any(int(qp[3].numel()) != n_bins for qp in qparams):
+        sizes = sorted({int(qp[3].numel()) for qp in qparams})
+        raise ValueError(f"quant_params of quantisers of different sizes in one call: lookup tables of {sizes} entries")
     try:  # the usual case: every lookup a flat fp32 tensor, every shift a 0-dim fp32 tensor, one device
         lookup = torch.stack([qp[3] for qp in qparams])
         shift = torch.stack([qp[0] for qp in qparams])
@@ -1575,6 +1581,15 @@ def _qparam_tables(qparams: Sequence[QuantParamsT], dev: torch.device) -> tuple[
         lookup = torch.stack([qp[3].reshape(n_bins).float() for qp in qparams])
         shift = torch.stack([torch.as_tensor(qp[0], dtype=torch.float32, device=lookup.device).reshape(())
                              for qp in qparams])
+    narrow = [r for r, qp in enumerate(qparams) if len(qp) > 4 and isinstance(qp[4], torch.dtype) and qp[4] != torch.float32]
+    if narrow:
+        lookup, shift = lookup.clone(), shift.clone()
+        for r in narrow:
+            dt = qparams[r][4]
+            if not dt.is_floating_point:
+                raise NotImplementedError(f"quant_params with orig_dtype {dt}")
+            lookup[r] = (lookup[r] + shift[r]).to(dt).float()
+            shift[r] = 0.0
     return lookup.to(dev).contiguous(), shift.to(dev).contiguous(), n_bins
 
 
@@ -1688,6 +1703,10 @@ def batch_decompress_decode_codes_batch(out: TensorBatch, idxs: Sequence[torch.T
     if n_bins > 4 or use_dct or k > _CH or P > 24:
         if quant_params is None:
             raise ValueError("these settings de-quantise first: pass quant_params, not only `tables`")
+        if validate:  # the reference's table lookup raises on a code past the table (the batch kernel would clamp it)
+            worst = int(torch.stack([c.max() for c in codes]).max().item()) if n else 0
+            if worst >= n_bins:
+                raise IndexError(f"index {worst} is out of bounds for dimension 0 with size {n_bins}")
         vals = []
         for p in range(P):
             vals.append(dequantize_batch(out, codes[p].reshape(-1), [quant_params[i][p] for i in range(T)], k))

@@ -300,3 +300,29 @@ def test_check_compressed_indices_reference_cases():
     with pytest.raises(ValueError, match="Expected tensor but got"):
         chk("param", [0, 1, 2, 3], 10, vals=v(4))
 
+
+
+def test_quantiser_tables_round_through_the_senders_dtype():
+    # src/tplr/compress.py:641-643: (lookup[code] + shift).to(orig_dtype); the flat tables carry that rounding as
+    # lookup' = round(lookup + shift), shift' = 0, so that the kernels' fp32 sum reproduces it
+    import torch
+
+    import templar_amd.compress as tc
+    from oracle import torch_cpu_path as tcp
+
+    torch.manual_seed(5)
+    lookup = torch.randn(4) * 1e-2
+    shift = torch.tensor(3.3e-3)
+    qp32 = (shift, 1.0, 2, lookup, torch.float32)
+    qp16 = (shift, 1.0, 2, lookup, torch.bfloat16)
+    lk, sh, n_bins = tc._qparam_tables([qp32, qp16], torch.device("cpu"))
+    assert n_bins == 4
+    codes = torch.arange(4, dtype=torch.uint8)
+    assert torch.equal(lk[0][codes.long()] + sh[0], tcp.dequantize(codes, qp32))
+    want16 = tcp.dequantize(codes, qp16)
+    assert want16.dtype == torch.bfloat16
+    assert torch.equal(lk[1][codes.long()] + sh[1], want16.float())
+    deq, _ = tc.dequantised_tables([[qp32, qp16]], torch.device("cpu"))
+    assert torch.equal(deq[0, 0], tcp.dequantize(codes, qp32)) and torch.equal(deq[0, 1], want16.float())
+    with pytest.raises(ValueError, match="different sizes"):
+        tc._qparam_tables([qp32, (shift, 1.0, 4, torch.randn(8), torch.float32)], torch.device("cpu"))
