@@ -575,6 +575,44 @@ def main():
                       "decode_then_subtract_ms": round(ev2_ms, 4)}
         del params, pb
 
+    # the outer step over the window (src/tplr/neurons.py:309-447 with the plain SGD of neurons/trainer.py:128-130):
+    # p <- p - lr * decode(aggregate) in the launch that forms the aggregate, against the aggregate written as a
+    # dense gradient, its statistics, the isfinite test and a foreach subtraction
+    outer = None
+    if DCT and 4 <= k <= 64 and P <= 15:
+        params = [torch.zeros_like(o) for o in outs]
+        pb = tc.TensorBatch(params)
+        lr = 0.4
+        factor = (scale * lr).contiguous()
+        flags = torch.zeros(len(pb), dtype=torch.int32, device=dev)
+        pc = torch.empty((n_chunks, 2), dtype=torch.float32, device=dev)
+        pt = torch.empty((len(pb), 4), dtype=torch.float32, device=dev)
+
+        def outer_kernel():
+            _lib_mod.check(lib_c.tplr_outer_step_batch(ip_c, vp_c, factor.data_ptr(), P, k, pb.table.data_ptr(), len(pb),
+                                                       n_chunks, pc.data_ptr(), pt.data_ptr(), flags.data_ptr(), cur_stream),
+                           "tplr_outer_step_batch")
+
+        ok_ms, _ = event_ms(outer_kernel, agg_steps, 2, settle=True)
+        _, ow_wall = event_ms(lambda: tc.outer_step_batch(pb, idxs, vals, k, lr, scale=scale), agg_steps, 1)
+
+        def aggregate_then_sgd():
+            st = tc.batch_decompress_decode_batch(out_batch, idxs, vals, k, scale=scale, use_dct=DCT, stats=True)
+            if bool((st[:, 2] == 1).all()):
+                torch._foreach_sub_(params, outs, alpha=lr)
+
+        ats_ms, ats_wall = event_ms(aggregate_then_sgd, agg_steps, 1)
+        os_bytes = n_chunks * (P * 11 * k // 2 + 2 * 16384)
+        outer = {"what": f"p <- p - lr * decode(aggregate of {P} peers) for every 2-D parameter, with the gradients' norm, "
+                         "mean and all-finite flag: one launch that reads and writes every parameter once and never "
+                         "writes the gradient (bytes: payload + every chunk read and written), against the aggregate "
+                         "launch with statistics followed by torch's foreach subtraction of the dense gradients",
+                 "kernel_ms": round(ok_ms, 4), "bytes": os_bytes, "GBps": round(os_bytes / (ok_ms * 1e-3) / 1e9, 2),
+                 "frac_of_hbm_peak": round(os_bytes / (ok_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                 "call_wall_ms": round(ow_wall, 4), "aggregate_then_sgd_ms": round(ats_ms, 4),
+                 "aggregate_then_sgd_wall_ms": round(ats_wall, 4)}
+        del params, pb, pc
+
     # templar's own settings carry the values as the codes of a four-bin quantiser: the aggregate straight from
     # the codes against de-quantising every peer first (what outer_step does, src/tplr/neurons.py:325-364)
     def codes_figures(idxs_, vals_, kk):
@@ -782,6 +820,8 @@ def main():
         result["index_stats"] = stats
     if evaluation is not None:
         result["evaluation_update"] = evaluation
+    if outer is not None:
+        result["outer_step"] = outer
     if staging is not None:
         result["payload_staging"] = staging
     if not args.no_cpu_baseline:

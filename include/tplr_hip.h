@@ -321,6 +321,26 @@ int tplr_apply_decoded_batch(const uint8_t* d_idx12, const float* d_val, const f
                              const tplr_tensor_desc* d_param_desc, int n_tensors, int64_t total_chunks,
                              int use_dct, int32_t* d_nonfinite, void* stream);
 
+/* The outer step over a whole window in one launch (src/tplr/neurons.py:309-447, outer_step, with the plain SGD
+ * of neurons/trainer.py:128-130): per parameter the reference builds the dense gradient
+ * decode(batch_decompress(P peers)), takes its norm and mean, tests isfinite().all() and, if that holds, lets
+ * optimizer.step() compute p <- p - lr * grad - the dense gradient written, read three times and read again by
+ * the optimiser.  Here param <- param - decode(aggregate of the peers' payloads), every value of peer p for
+ * tensor t times d_factor[t * n_peers + p] first (pass lr * clip factor): the aggregate's fused launch whose
+ * result is subtracted from the parameter's rows instead of stored, the gradient never written.  Chunks of 64x64
+ * with the transform, k <= 64, n_peers <= 15; h_idx12, h_val as in tplr_decode_aggregate_batch.
+ * d_nonfinite (nullable, n_tensors ints zeroed by the caller): as in tplr_apply_decoded_batch, a chunk whose
+ * decoded values are not all finite is left unwritten and flags its tensor.  A caller that must leave such a
+ * parameter untouched as a whole, as the reference does, makes every factor of a tensor it cannot vouch for a NaN
+ * (then no chunk of it is written and the flag is set) and serves that tensor separately.
+ * d_chunk_stats (2 floats per chunk) and d_tensor_stats (4 floats per tensor), both or neither: the decoded
+ * values' {L2 norm, mean, 1.0 if every per-chunk figure is finite else 0.0, sum of squares} per tensor, i.e. the
+ * figures of lr * grad when the factors carry lr. */
+int tplr_outer_step_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_factor,
+                          int n_peers, int k, const tplr_tensor_desc* d_param_desc, int n_tensors,
+                          int64_t total_chunks, float* d_chunk_stats, float* d_tensor_stats, int32_t* d_nonfinite,
+                          void* stream);
+
 /* ---- validator side: checks on the packed index streams ------------------------------
  * For up to 32 peers whose flat payloads share one row layout (d_desc: n_tensors descriptors, of
  * which only chunk_begin, x_chunks and y_chunks are read; a parameter of n rows that are not

@@ -276,6 +276,26 @@ def error_feedback_step(ef, grad, decay: float, topk: int, *, use_dct: bool = Tr
     return ef, idx12, val, ef - recon
 
 
+# ---------------------------------------------------------------- outer step (src/tplr/neurons.py:341-447)
+def outer_step(param, idx_packed_list, val_list, xshape, totalk: int, lr: float, *, use_dct: bool = True):
+    """One parameter's pass through outer_step with the plain SGD the reference builds for it
+    (neurons/trainer.py:128-130: SGD(lr), no momentum, no weight decay): block norms of the peers' values (:346),
+    batch_decompress with the median clip (:355-365), decode (:367), the gradient's L2 norm and mean for the
+    fingerprint (:380-385), and - unless an element of the gradient is not finite, in which case the parameter is
+    left alone (:438-442) - p <- p - lr * grad (optimizer.step(), :446).
+    Returns (new_param, grad_norm, grad_mean, applied)."""
+    p = _c(param, np.float32)
+    vals = [_c(v, np.float32) for v in val_list]
+    norms = np.array([norm2(v) for v in vals], dtype=np.float32)                 # :346
+    grad = decode2d(batch_decompress(idx_packed_list, vals, xshape, totalk, block_norms=norms), use_dct=use_dct)
+    with np.errstate(all="ignore"):
+        g_norm = float(np.sqrt((grad.astype(np.float64) ** 2).sum()))            # :381
+        g_mean = float(grad.astype(np.float64).mean())                           # :385
+    if not np.isfinite(grad).all():                                              # :438
+        return p.copy(), g_norm, g_mean, False
+    return (p - np.float32(lr) * grad).astype(np.float32), g_norm, g_mean, True  # :446
+
+
 # ---------------------------------------------------------------- index checks
 def index_overlap(idx_list):
     """Pairwise overlap of peers' index rows, as check_uid_index_overlap computes it per

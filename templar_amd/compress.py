@@ -1259,6 +1259,78 @@ def apply_decoded_batch(params: TensorBatch, idx12: torch.Tensor, val: torch.Ten
 
 
 @torch.no_grad()
+def outer_step_batch(params: TensorBatch, idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], k: int, lr: float, *,
+                     scale: torch.Tensor | None = None, use_dct: bool = True, stats: bool = True):
+    """outer_step for every 2-D parameter of a model in one launch (src/tplr/neurons.py:309-447 with the plain
+    SGD of neurons/trainer.py:128-130): per parameter the reference forms the peers' block norms, the dense
+    gradient decode(batch_decompress(..., clip_norm=True)), its L2 norm and mean for the fingerprint (:380-385),
+    tests torch.isfinite(grad).all() (:411, :438) and lets optimizer.step() compute p <- p - lr * grad.  Here the
+    aggregate's result is subtracted from the parameters in the launch that forms it, lr and the clip factors
+    riding on the values (the transform is linear): the dense gradients are never written.
+
+    `idxs[p]`, `vals[p]`: peer p's flat payload; `scale`: ready (T, P) clip factors (PeerNorms.clip_scales), else
+    taken from the values.  Returns (stats, skipped): stats a (T, 4) tensor {grad L2 norm, grad mean, all-finite
+    flag, grad sum of squares} per parameter (None without `stats`), skipped the list of parameters left
+    untouched because their gradient holds a NaN or an infinity, as the reference leaves them.
+
+    A parameter whose peers' norms are all finite and positive under a finite median has a finite gradient (every
+    clipped value is bounded by the median, 15 of them add up per coefficient, the transform's gain is 64), so it
+    goes through the fused launch.  Any other parameter - a NaN or infinite norm, a zero factor - is kept out of
+    it (its factors become NaN: no chunk of it is written) and served the reference's way afterwards: dense
+    gradient, test, subtraction.  Reading the launch's per-parameter flags costs the one synchronisation of
+    the call.  Settings the fused launch does not serve (no transform, k > 64, more than 15 peers) take that
+    route for every parameter."""
+    lib = _lib.load()
+    P, T, n, dev = len(vals), len(params), params.total_chunks, params.device
+    if lr == 0 or lr != lr:
+        raise ValueError(f"lr must be a non-zero number, got {lr}")
+    for i, v in zip(idxs, vals):
+        if i.dtype != torch.uint8:
+            raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
+        if v.dtype != torch.float32 or v.numel() != n * k or i.numel() * 2 != n * k * 3 or not v.is_contiguous():
+            raise RuntimeError(f"flat payload mismatch: {i.numel()} index bytes / {v.numel()} values for {n} chunks, k={k}")
+    if scale is None:
+        scale = peer_clip_scales_batch(params, vals, k)
+    elif tuple(scale.shape) != (T, P) or scale.dtype != torch.float32 or not scale.is_contiguous():
+        raise ValueError(f"scale: expected a contiguous fp32 ({T}, {P}) tensor, got {tuple(scale.shape)}")
+    out = torch.zeros((T, 4), dtype=torch.float32, device=dev) if stats else None
+    fused = use_dct and 4 <= k <= _CH and P <= 15
+    flagged = list(range(T))
+    if fused:
+        sound = (torch.isfinite(scale) & (scale > 0)).all(dim=1, keepdim=True)
+        factor = torch.where(sound, scale * float(lr), torch.full_like(scale, float("nan"))).contiguous()
+        flags = torch.zeros(T, dtype=torch.int32, device=dev)
+        per_chunk = torch.empty((max(n, 1), 2), dtype=torch.float32, device=dev) if stats else None
+        ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+        vp = (C.c_void_p * P)(*[v.data_ptr() for v in vals])
+        with _on(dev):
+            st = lib.tplr_outer_step_batch(ip, vp, _ptr(factor), P, k, _ptr(params.table), T, n, _ptr(per_chunk), _ptr(out),
+                                           _ptr(flags), _stream(dev))
+        _lib.check(st, "tplr_outer_step_batch")
+        if stats:  # the launch's figures are those of lr * grad
+            out[:, 0] /= abs(float(lr))
+            out[:, 1] /= float(lr)
+            out[:, 3] /= float(lr) * float(lr)
+        flagged = torch.nonzero(flags).reshape(-1).tolist()  # the call's one synchronisation
+    skipped = []
+    for t in flagged:  # the reference's own sequence, one parameter at a time
+        y, x = params.xshape(t)[:2]
+        sl = [params.payload_slice(t, idxs[p], vals[p], k) for p in range(P)]
+        grad = _aggregate_chunks([a.contiguous() for a, _ in sl], [b.contiguous() for _, b in sl], scale[t].contiguous(),
+                                 y, x, k, normalise=False, use_dct=use_dct, rows=True)
+        finite = bool(torch.isfinite(grad).all())
+        if stats:
+            ss = (grad.double() ** 2).sum()
+            out[t] = torch.stack([ss.sqrt(), grad.double().mean(), torch.tensor(float(finite), device=dev, dtype=torch.float64),
+                                  ss]).float()
+        if finite:
+            params.tensors[t].sub_(grad, alpha=float(lr))
+        else:
+            skipped.append(t)
+    return out, skipped
+
+
+@torch.no_grad()
 def error_feedback_step_batch(ef: TensorBatch, grad: TensorBatch, decay: float, topk: int, *, use_dct: bool = True,
                               compressor: "TopKCompressor | None" = None, null_round: bool = False):
     """The miner's per-parameter loop of src/tplr/neurons.py:147-171 for a whole set of 2-D
@@ -1993,6 +2065,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "apply_decoded_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "PeerNorms", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "apply_decoded_batch", "outer_step_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "PeerNorms", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

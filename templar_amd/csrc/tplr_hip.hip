@@ -623,6 +623,20 @@ __global__ __launch_bounds__(64, 3) void k_calib_encode(const tplr_tensor_desc* 
     if (__float_as_uint(s) == 0x7fedcba9u && sink) sink[0] = s;  // (a NaN pattern no sum produces)
 }
 
+// body(Index<0>{}) ... body(Index<N - 1>{}): a loop whose counter is a constant in the body, so that
+// arrays indexed by it stay in registers whatever the optimiser thinks of unrolling
+template <int I>
+struct Index {
+    static constexpr int value = I;
+};
+template <int N, typename Body>
+__device__ __forceinline__ void static_for(Body&& body) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(body);
+        body(Index<N - 1>{});
+    }
+}
+
 // =========================================================================================
 // decode side
 // =========================================================================================
@@ -1111,14 +1125,16 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         wave_lds_fence();
         bool tripped = false;
         if constexpr (kSubtract) {
+            chunk_stats(v, g, false);
             tripped = guard_trips(v, cs.t);
             const __amdgpu_buffer_rsrc_t rs = chunk_rsrc((const void*)dst, ld);
             const int ld4 = static_cast<int>(ld) * 4;
 #pragma unroll
             for (int r = 0; r < 64; ++r)
                 v[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4, r * ld4, 0)) - v[r];
+        } else {
+            chunk_stats(v, g, false);
         }
-        chunk_stats(v, g, false);
         if (rows) {
             store_chunk_rows(v, (void*)dst, ld, lane, tripped);
         } else {
@@ -1374,8 +1390,12 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             asm volatile("" : "+v"(my_units));
             // the register with the next unit's entry, on its way from another lane
             uint32_t held = group_entry(cur[0], from4);
-            float before[kSubtract ? 64 : 1];
-            if constexpr (kSubtract)
+            // kSubtract: the destination's rows are requested here and arrive during the pass where the
+            // registers for that exist (up to 8 peers' payload in flight); with more peers they are fetched
+            // after the pass, sixteen rows at a time, two such groups in flight (kLateRows)
+            constexpr bool kLateRows = kSubtract && kUnits > 8;
+            float before[kSubtract && !kLateRows ? 64 : 1];
+            if constexpr (kSubtract && !kLateRows)
                 load_chunk_rows(before, (const void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane);
             // along b: v[k] = sum_b Z[b][lane] F[k][b]
             dct64_inv_hooked(v, [&](auto tag) {
@@ -1416,13 +1436,17 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 }
             });
             bool tripped = false;
+            // (kSubtract: the statistics are those of the decoded values, not of the difference)
+            if constexpr (kSubtract) chunk_stats(v, g, skip0);
             if constexpr (kSubtract) {
                 // (a chunk that is to be done again on the exact path holds claim marks: it is tested there)
                 if (!skip0) tripped = guard_trips(v, o0.t);
+                if constexpr (!kLateRows) {
 #pragma unroll
-                for (int r = 0; r < 64; ++r) v[r] = before[r] - v[r];
+                    for (int r = 0; r < 64; ++r) v[r] = before[r] - v[r];
+                }
             }
-            chunk_stats(v, g, skip0);
+            if constexpr (!kSubtract) chunk_stats(v, g, skip0);
             // (the loop-carried destination may have been parked in vector registers: make it
             // scalar again, or every store becomes a loop over distinct descriptors)
             const bool skip1 = g + 1 < g1 && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
@@ -1430,8 +1454,35 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             repeat = 0;
             mean_pass();
             // a chunk that is to be done again is not stored: its descriptor gets a range of zero bytes
-            store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane,
-                             skip0 || tripped);
+            if constexpr (kLateRows) {
+                void* chunk0 = (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0));
+                const int64_t ld0 = uniform64(o0.ld);
+                const __amdgpu_buffer_rsrc_t rd = chunk_rsrc(chunk0, ld0);
+                const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+                    chunk0, 0, (skip0 || tripped) ? 0 : static_cast<int>((63 * ld0 + 64) * 4), 0x00020000);
+                const int ld4 = static_cast<int>(ld0) * 4;
+                float b[2][16];
+                auto fetch = [&](auto qt) {
+                    constexpr int q = decltype(qt)::value;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        b[q & 1][i] = __builtin_bit_cast(
+                            float, __builtin_amdgcn_raw_buffer_load_b32(rd, lane * 4, (q * 16 + i) * ld4, 0));
+                };
+                fetch(Index<0>{});
+                fetch(Index<1>{});
+                static_for<4>([&](auto qt) {
+                    constexpr int q = decltype(qt)::value;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, b[q & 1][i] - v[q * 16 + i]), wr,
+                                                              lane * 4, (q * 16 + i) * ld4, 2);
+                    if constexpr (q + 2 < 4) fetch(Index<q + 2>{});
+                });
+            } else {
+                store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane,
+                                 skip0 || tripped);
+            }
             skip0 = skip1;
             o0 = o1;
             o1 = o2;
@@ -1920,19 +1971,6 @@ struct IdxPtrs {
     const uint8_t* idx[kStatPeers];
 };
 
-// body(Index<0>{}) ... body(Index<N - 1>{}): a loop whose counter is a constant in the body, so that
-// arrays indexed by it stay in registers whatever the optimiser thinks of unrolling
-template <int I>
-struct Index {
-    static constexpr int value = I;
-};
-template <int N, typename Body>
-__device__ __forceinline__ void static_for(Body&& body) {
-    if constexpr (N > 0) {
-        static_for<N - 1>(body);
-        body(Index<N - 1>{});
-    }
-}
 
 // kPerPass: peers handled by one wave instruction: 2 when k <= 32 (one peer per half of the wave), 1 when
 // k <= 64; 0 = rows of any length, entry by entry.  kPasses: wave instructions per row that the
@@ -2894,9 +2932,13 @@ __global__ __launch_bounds__(256) void k_tensor_rnorm_scales(const float* __rest
 // A chunk whose sum of squares (or sum) is not finite either holds a non-finite element or overflowed in
 // fp32: its 4096 elements are read back and examined one by one, and where they are all finite their figures
 // are formed again in double, so the flag is exact and the norm survives values near the top of the range.
+// use_dct bit 1: the tensors of `table` do not hold the values the figures are about (an update subtracted them
+// from its parameters): nothing is read back, and a figure that is not finite marks the tensor.
 __global__ __launch_bounds__(256) void k_tensor_stats(const float* __restrict__ chunk_stats,
                                                       const tplr_tensor_desc* __restrict__ table, int use_dct,
                                                       float* __restrict__ out) {
+    const bool figures_only = (use_dct & 2) != 0;
+    use_dct &= 1;
     __shared__ double part[4];
     __shared__ int bad_any;
     const tplr_tensor_desc d = table[blockIdx.x];
@@ -2909,7 +2951,9 @@ __global__ __launch_bounds__(256) void k_tensor_stats(const float* __restrict__ 
     // one chunk's figures; not finite: the chunk is read back (rare)
     auto take = [&](int64_t i, float2 got) {
         double ss = static_cast<double>(got.x), sm = static_cast<double>(got.y);
-        if (!isfinite(ss) || !isfinite(sm)) {
+        if (figures_only) {
+            if (!isfinite(ss) || !isfinite(sm)) bad = 1;
+        } else if (!isfinite(ss) || !isfinite(sm)) {
             const bool rows = use_dct || d.ld > 0;  // the (R, C) tensor itself, or chunk after chunk
             const int64_t y = i / d.x_chunks, x = i - y * d.x_chunks;
             const float* c0 = rows ? static_cast<const float*>(d.dense) + (y * 64) * d.ld + x * 64
@@ -3547,6 +3591,51 @@ int tplr_apply_decoded_batch(const uint8_t* d_idx12, const float* d_val, const f
                              int32_t* d_nonfinite, void* stream) {
     return subtract_decoded(d_idx12, d_val, d_factor, k, d_param_desc, n_tensors, total_chunks, use_dct, d_nonfinite,
                             stream);
+}
+
+int tplr_outer_step_batch(const uint8_t* const* h_idx12, const float* const* h_val, const float* d_factor, int n_peers,
+                          int k, const tplr_tensor_desc* d_param_desc, int n_tensors, int64_t total_chunks,
+                          float* d_chunk_stats, float* d_tensor_stats, int32_t* d_nonfinite, void* stream) {
+    if (!h_idx12 || !h_val || !d_param_desc || n_peers < 1 || n_tensors < 1 || total_chunks < 0 || k < 4 || (k & 1))
+        return TPLR_E_BADARG;
+    if ((d_chunk_stats == nullptr) != (d_tensor_stats == nullptr)) return TPLR_E_BADARG;
+    if (k > 64 || n_peers > 15) return TPLR_E_TOOMANY;  // the register-resident path with 4-bit counters
+    PeerPtrs pp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        pp.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
+        pp.val[p] = p < n_peers ? h_val[p] : nullptr;
+        if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
+    }
+    if (total_chunks > 0) {
+        auto apart = [](const void* a, const void* b) {
+            return static_cast<int64_t>(reinterpret_cast<intptr_t>(a) - reinterpret_cast<intptr_t>(b));
+        };
+        const int64_t si = n_peers > 1 ? apart(pp.idx[1], pp.idx[0]) : 0;
+        const int64_t sv4 = n_peers > 1 ? apart(pp.val[1], pp.val[0]) : 0;
+        bool strided = true;
+        for (int p = 1; p < n_peers; ++p)
+            strided = strided && apart(pp.idx[p], pp.idx[0]) == p * si && apart(pp.val[p], pp.val[0]) == p * sv4;
+        tplr_tensor_desc none = {};
+        const int options = d_chunk_stats ? 2 : 0;
+        int st;
+        if (n_peers <= 8 && strided)
+            st = launch_decode_as(k_decode_aggregate<true, 8, 4, true, true>, pp, d_factor, n_peers, k, d_param_desc, none,
+                                  n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats, stream, si, sv4 / 4,
+                                  nullptr, d_nonfinite);
+        else if (strided)
+            st = launch_decode_as(k_decode_aggregate<true, 16, 4, true, true>, pp, d_factor, n_peers, k, d_param_desc,
+                                  none, n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats, stream, si,
+                                  sv4 / 4, nullptr, d_nonfinite);
+        else
+            st = launch_decode_as(k_decode_aggregate<true, 16, 4, true, false>, pp, d_factor, n_peers, k, d_param_desc,
+                                  none, n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats, stream, 0, 0,
+                                  nullptr, d_nonfinite);
+        if (st) return st;
+    }
+    if (d_tensor_stats)
+        hipLaunchKernelGGL(k_tensor_stats, dim3(static_cast<unsigned>(n_tensors)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), d_chunk_stats, d_param_desc, 1 | 2, d_tensor_stats);
+    return launch_status();
 }
 
 int tplr_ef_subtract_own_batch(const uint8_t* d_idx12, const float* d_sent, const float* d_own, int k,

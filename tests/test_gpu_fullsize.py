@@ -568,3 +568,56 @@ def test_codes_aggregate_seeded_sweep(dev):
             got = ss[b0:b0 + Y * X].double()
             assert float((got - ref).abs().max()) <= 1e-5 * float(ref.max()), (draw, t)
             b0 += Y * X
+
+
+def test_full_set_outer_step_properties(dev):
+    # the 1B set, 15 peers: p <- p - lr * decode(aggregate) in one launch equals the aggregate written as dense
+    # gradients followed by the subtraction (every element, fp32 tolerance), its statistics are those of the
+    # aggregate launch, the opposite sign takes the step back, and a poisoned parameter keeps its bits while the
+    # others take their step
+    grads, k = _set("cfg3_llama1b", dev)
+    P, lr = 15, 0.4
+    batch = tc.TensorBatch(grads)
+    stage = tc.PayloadStage(batch, k, P, quantized=False)
+    idxs, vals = [], []
+    for p in range(P):
+        own = [workloads.student_t3(tuple(g.shape), 1000 * (p + 1) + j, row_scale=True, device=dev).add_(g, alpha=0.5)
+               for j, g in enumerate(grads)]
+        i12, v = stage.regions(p)
+        tc.encode_compress_batch(tc.TensorBatch(own), k, idx12=i12, val=v)
+        idxs.append(i12)
+        vals.append(v)
+        del own
+    shapes = [tuple(g.shape) for g in grads]
+    scale = tc.peer_clip_scales_batch(batch, vals, k)
+    ref_stats = tc.batch_decompress_decode_batch(batch, idxs, vals, k, scale=scale, stats=True)   # dense gradients in `grads`
+    gen = torch.Generator(device=dev).manual_seed(5)
+    params = [torch.randn(s, device=dev, generator=gen) * 0.02 for s in shapes]
+    pb = tc.TensorBatch(params)
+    start3 = params[3].clone()
+    stats, skipped = tc.outer_step_batch(pb, idxs, vals, k, lr, scale=scale)
+    assert skipped == []
+    gen = torch.Generator(device=dev).manual_seed(5)
+    worst = 0.0
+    for p, g, s in zip(params, grads, shapes):
+        want = torch.randn(s, device=dev, generator=gen) * 0.02 - lr * g
+        worst = max(worst, float((p - want).abs().max()) / float(want.abs().max()))
+    assert worst <= TOL
+    assert torch.allclose(stats[:, 0], ref_stats[:, 0], rtol=2e-5) and torch.equal(stats[:, 2], ref_stats[:, 2])
+    assert torch.allclose(stats[:, 1], ref_stats[:, 1], rtol=1e-3, atol=1e-9)
+    tc.outer_step_batch(pb, idxs, vals, k, -lr, scale=scale, stats=False)
+    gen = torch.Generator(device=dev).manual_seed(5)
+    back = 0.0
+    for p, s in zip(params, shapes):
+        p0 = torch.randn(s, device=dev, generator=gen) * 0.02
+        back = max(back, float((p - p0).abs().max()) / float(p0.abs().max()))
+    assert back <= TOL
+    # one NaN in one peer's values of parameter 3
+    keep = [p.clone() if i in (2, 3, 4) else None for i, p in enumerate(params)]
+    vals[7][batch.offsets[3] + 11, 5] = float("nan")
+    stats, skipped = tc.outer_step_batch(pb, idxs, vals, k, lr)
+    assert skipped == [3] and float(stats[3, 2]) == 0.0
+    assert torch.equal(params[3].view(torch.int32), keep[3].view(torch.int32))
+    assert not torch.equal(params[2], keep[2]) and not torch.equal(params[4], keep[4])
+    assert all(bool(torch.isfinite(p).all()) for p in params)
+    del start3

@@ -1,0 +1,161 @@
+"""The outer step over a window in one launch (tplr_outer_step_batch, outer_step_batch) against the oracle's
+restatement of src/tplr/neurons.py:341-447 with the plain SGD of neurons/trainer.py:128-130.  Needs an MI355X.
+
+Bars: updated parameters within 1e-5 of the parameter's largest magnitude (the transform and the order in which lr
+and the clip factor are applied differ in rounding), gradient norm within 1e-5, a parameter whose gradient is not
+finite left bit for bit as it was, the fused launch equal to aggregate-then-subtract on the device within the
+same tolerance.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import codec as orc  # noqa: E402  (the checker)
+import templar_amd.compress as tc  # noqa: E402
+import workloads  # noqa: E402
+
+TOL = 1e-5
+
+
+def t3(shape, seed, row_scale=False):
+    return workloads.student_t3(shape, seed, row_scale=row_scale)
+
+
+def _window(dev, shapes, k, P, use_dct=True, staged=False):
+    base = [t3(s, 400 + i, row_scale=True).to(dev) for i, s in enumerate(shapes)]
+    batch = tc.TensorBatch(base)
+    stage = tc.PayloadStage(batch, k, P, quantized=False) if staged else None
+    idxs, vals = [], []
+    for p in range(P):
+        own = [0.5 * g + t3(tuple(g.shape), 7000 + 10 * p + i, row_scale=True).to(dev) * (1 + 0.5 * p) for i, g in enumerate(base)]
+        if staged:
+            i12, v = stage.regions(p)
+            tc.encode_compress_batch(tc.TensorBatch(own), k, use_dct=use_dct, idx12=i12, val=v)
+        else:
+            i12, v = tc.encode_compress_batch(tc.TensorBatch(own), k, use_dct=use_dct)
+        idxs.append(i12)
+        vals.append(v)
+    return batch, idxs, vals, stage
+
+
+def _check_against_oracle(batch, params, start, idxs, vals, k, lr, stats, skipped, use_dct, expect_skipped=()):
+    assert sorted(skipped) == sorted(expect_skipped)
+    P = len(vals)
+    for t in range(len(batch)):
+        sl = [batch.payload_slice(t, idxs[p], vals[p], k) for p in range(P)]
+        xshape = batch.xshape(t)
+        want, g_norm, g_mean, applied = orc.outer_step(
+            start[t].cpu().numpy(), [a.cpu().numpy().reshape(xshape[0], xshape[1], -1) for a, _ in sl],
+            [b.cpu().numpy() for _, b in sl], xshape, 4096, lr, use_dct=use_dct)
+        got = params[t].cpu().numpy()
+        assert applied == (t not in expect_skipped)
+        if not applied:
+            assert np.array_equal(got.view(np.int32), start[t].cpu().numpy().view(np.int32)), f"parameter {t} was touched"
+            assert float(stats[t, 2]) == 0.0
+            continue
+        assert np.abs(got - want).max() <= TOL * np.abs(want).max(), (t, np.abs(got - want).max())
+        assert float(stats[t, 2]) == 1.0
+        assert np.isclose(float(stats[t, 0]), g_norm, rtol=2e-5), (t, float(stats[t, 0]), g_norm)
+        assert abs(float(stats[t, 1]) - g_mean) <= 2e-5 * g_norm / np.sqrt(want.size) + 1e-12
+        assert np.isclose(float(stats[t, 3]), g_norm ** 2, rtol=4e-5)
+
+
+@pytest.mark.parametrize("P,k,staged", [(15, 32, True), (15, 32, False), (8, 64, True), (3, 16, False), (1, 32, True),
+                                        (9, 4, True)])
+def test_outer_step_in_one_launch_matches_the_reference_sequence(dev, P, k, staged):
+    shapes = [(128, 192), (64, 64), (320, 128), (512, 256)]
+    batch, idxs, vals, _ = _window(dev, shapes, k, P, staged=staged)
+    gen = torch.Generator(device=dev).manual_seed(3)
+    big = torch.randn((320, 512), device=dev, generator=gen)
+    big0 = big.clone()
+    start = [torch.randn(shapes[0], device=dev, generator=gen), torch.randn(shapes[1], device=dev, generator=gen),
+             big[:, 128:256].clone(), torch.randn(shapes[3], device=dev, generator=gen)]
+    params = [start[0].clone(), start[1].clone(), big[:, 128:256], start[3].clone()]   # one parameter a strided view
+    lr = 0.4
+    stats, skipped = tc.outer_step_batch(tc.TensorBatch(params), idxs, vals, k, lr)
+    torch.cuda.synchronize()
+    _check_against_oracle(batch, params, start, idxs, vals, k, lr, stats, skipped, True)
+    assert torch.equal(big[:, :128], big0[:, :128]) and torch.equal(big[:, 256:], big0[:, 256:])  # around the view
+    # with ready clip factors (noted on arrival) the same bits
+    again = [s.clone() for s in start]
+    norms = tc.PeerNorms([batch], P)
+    for p in range(P):
+        norms.arrived(p, [vals[p]])
+    stats2, skipped2 = tc.outer_step_batch(tc.TensorBatch(again), idxs, vals, k, lr, scale=norms.clip_scales(P)[0])
+    assert skipped2 == [] and all(torch.equal(a, b) for a, b in zip(again, [p.contiguous() for p in params]))
+    assert torch.equal(stats, stats2)
+    # and the opposite sign takes the step back
+    tc.outer_step_batch(tc.TensorBatch(again), idxs, vals, k, -lr, stats=False)
+    assert max(float((a - s).abs().max()) / float(s.abs().max()) for a, s in zip(again, start)) <= TOL
+
+
+def test_outer_step_equals_aggregate_then_subtract_on_the_device(dev):
+    shapes = [(256, 256), (128, 512), (64, 64)]
+    k, P, lr = 32, 15, 0.25
+    batch, idxs, vals, _ = _window(dev, shapes, k, P, staged=True)
+    start = [torch.randn(s, device=dev) for s in shapes]
+    params = [s.clone() for s in start]
+    stats, skipped = tc.outer_step_batch(tc.TensorBatch(params), idxs, vals, k, lr)
+    dense = [torch.empty(s, device=dev) for s in shapes]
+    ref_stats = tc.batch_decompress_decode_batch(tc.TensorBatch(dense), idxs, vals, k, clip_norm=True, stats=True)
+    assert skipped == []
+    for p, s, g in zip(params, start, dense):
+        want = s - lr * g
+        assert float((p - want).abs().max()) <= TOL * float(want.abs().max())
+    assert torch.allclose(stats[:, 0], ref_stats[:, 0], rtol=2e-5) and torch.allclose(stats[:, 3], ref_stats[:, 3], rtol=4e-5)
+    assert torch.equal(stats[:, 2], ref_stats[:, 2])
+
+
+@pytest.mark.parametrize("kind", ["nan", "inf", "nan_norm_other_parameter_fine"])
+def test_a_parameter_with_a_non_finite_gradient_is_left_alone(dev, kind):
+    # src/tplr/neurons.py:438-442: `if not torch.isfinite(p.grad).all(): p.grad = None; continue` - the whole
+    # parameter keeps its bits, the others take their step
+    shapes = [(128, 192), (256, 128), (64, 64)]
+    k, P, lr = 32, 5, 0.4
+    batch, idxs, vals, _ = _window(dev, shapes, k, P, staged=True)
+    row = batch.offsets[1] + 2
+    if kind == "nan":
+        vals[3][row, 4] = float("nan")
+    elif kind == "inf":
+        vals[0][row, 0] = float("inf")
+    else:
+        vals[2][row, 9] = float("nan")
+    start = [torch.randn(s, device=dev) for s in shapes]
+    params = [s.clone() for s in start]
+    stats, skipped = tc.outer_step_batch(tc.TensorBatch(params), idxs, vals, k, lr)
+    _check_against_oracle(batch, params, start, idxs, vals, k, lr, stats, skipped, True, expect_skipped=[1])
+
+
+@pytest.mark.parametrize("P,k,use_dct", [(20, 32, True), (4, 32, False), (4, 128, True)])
+def test_settings_outside_the_fused_launch_take_the_reference_route(dev, P, k, use_dct):
+    shapes = [(128, 128), (64, 192)]
+    batch, idxs, vals, _ = _window(dev, shapes, k, P, use_dct=use_dct)
+    start = [torch.randn(s, device=dev) for s in shapes]
+    params = [s.clone() for s in start]
+    stats, skipped = tc.outer_step_batch(tc.TensorBatch(params), idxs, vals, k, 0.1, use_dct=use_dct)
+    _check_against_oracle(batch, params, start, idxs, vals, k, 0.1, stats, skipped, use_dct)
+
+
+def test_outer_step_argument_checks(dev):
+    import ctypes as C
+    from templar_amd import _lib
+    shapes = [(64, 128)]
+    batch, idxs, vals, _ = _window(dev, shapes, 32, 2)
+    params = tc.TensorBatch([torch.zeros(shapes[0], device=dev)])
+    with pytest.raises(ValueError):
+        tc.outer_step_batch(params, idxs, vals, 32, 0.0)
+    with pytest.raises(RuntimeError):
+        tc.outer_step_batch(params, idxs, [v[:1] for v in vals], 32, 0.1)
+    with pytest.raises(ValueError):
+        tc.outer_step_batch(params, idxs, vals, 32, 0.1, scale=torch.ones(3, 3, device=dev))
+    lib = _lib.load()
+    ip = (C.c_void_p * 2)(*[i.data_ptr() for i in idxs])
+    vp = (C.c_void_p * 2)(*[v.data_ptr() for v in vals])
+    t = params.table.data_ptr()
+    assert lib.tplr_outer_step_batch(ip, vp, None, 16, 32, t, 1, 2, None, None, None, None) == _lib.TPLR_E_TOOMANY
+    assert lib.tplr_outer_step_batch(ip, vp, None, 2, 128, t, 1, 2, None, None, None, None) == _lib.TPLR_E_TOOMANY
+    assert lib.tplr_outer_step_batch(ip, vp, None, 2, 2, t, 1, 2, None, None, None, None) == _lib.TPLR_E_BADARG
+    assert lib.tplr_outer_step_batch(ip, vp, None, 2, 32, t, 1, 2, vals[0].data_ptr(), None, None, None) == _lib.TPLR_E_BADARG
+    assert lib.tplr_outer_step_batch(None, vp, None, 2, 32, t, 1, 2, None, None, None, None) == _lib.TPLR_E_BADARG

@@ -507,3 +507,46 @@ def test_error_feedback_step_closed_form_against_scipy():
     # the remainder's own transform is zero at the sent coefficients
     left = scipy.fft.dctn(new.astype(np.float64).reshape(1, 64, 2, 64).transpose(0, 2, 1, 3), axes=(-2, -1), norm="ortho").reshape(-1, 4096)
     assert np.abs(np.take_along_axis(left, order, 1)).max() <= 2e-5 * np.abs(coef).max()
+
+
+# ---------------------------------------------------------------- outer step (src/tplr/neurons.py:341-447)
+@pytest.mark.parametrize("use_dct", [True, False])
+@pytest.mark.parametrize("poison", [None, "nan", "inf"])
+def test_outer_step_against_torch_sgd_on_the_torch_op_sequence(use_dct, poison):
+    # orc.outer_step against the reference's own lines replayed with torch on the CPU: block norms (:346),
+    # batch_decompress with them (:355-365), decode (:367), norm and mean (:381-385), the isfinite gate (:438-442)
+    # and torch.optim.SGD(lr).step() (:446; neurons/trainer.py:128-130)
+    torch.manual_seed(11)
+    R, Cc, k, P, lr = 128, 192, 32, 5, 0.4
+    b64 = tcp.basis(64)
+    pay = []
+    for p in range(P):
+        g = torch.distributions.StudentT(3.0).sample((R, Cc)) * 1e-3 * (1 + p)
+        pay.append(tcp.compress(tcp.encode(g, 64, 64, b64[0], b64[0], use_dct=use_dct), k))
+    idxs, vals = [a[0] for a in pay], [a[1].clone() for a in pay]
+    xshape, totalk = pay[0][2], pay[0][3]
+    if poison == "nan":
+        vals[2][0, 1, 3] = float("nan")
+    elif poison == "inf":
+        vals[4][1, 0, 0] = float("inf")
+    param = torch.nn.Parameter(torch.randn(R, Cc))
+    before = param.detach().clone()
+    opt = torch.optim.SGD([param], lr=lr)
+    norms = torch.stack([torch.norm(v, p=2) for v in vals])
+    grad = tcp.decode(tcp.batch_decompress(idxs, vals, xshape, totalk, block_norms=norms), b64[1], b64[1], use_dct=use_dct)
+    want_norm, want_mean = torch.norm(grad, p=2).item(), grad.mean().item()
+    applied = bool(torch.isfinite(grad).all())
+    if applied:
+        param.grad = grad
+        opt.step()
+    got, g_norm, g_mean, got_applied = orc.outer_step(before.numpy(), [i.numpy() for i in idxs], [v.numpy() for v in vals],
+                                                      tuple(xshape), totalk, lr, use_dct=use_dct)
+    assert got_applied == applied == (poison is None)
+    if not applied:
+        assert np.array_equal(got, before.numpy())      # the parameter keeps its bits
+        assert not np.isfinite(g_norm) or np.isnan(g_norm)
+        return
+    assert np.abs(got - param.detach().numpy()).max() <= 1e-6 * float(before.abs().max())
+    assert np.isclose(g_norm, want_norm, rtol=1e-5) and np.isclose(g_mean, want_mean, rtol=1e-3, atol=1e-9)
+    # the step really is p - lr * grad: undoing it with the gradient returns the parameter
+    assert np.abs(got + np.float32(lr) * grad.numpy() - before.numpy()).max() <= 1e-6 * float(before.abs().max())
