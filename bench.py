@@ -35,17 +35,19 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of the two whole-set kernels, from hardware counters: rocprofv3 --pmc
-# FETCH_SIZE and --pmc WRITE_SIZE runs of `bench.py --profile encode|aggregate`, each scaled by what
-# the same counter reports for the library's 1 GiB calibration copy (`--profile copy`: FETCH_SIZE
-# x 2.000, WRITE_SIZE x 1.000).  The commands and raw figures are in the rocprofv3 summaries kept
-# with the sources.  Only the configuration they were measured on has an entry.
-MEASURED_TRAFFIC = {
-    ("cfg3_llama1b", 15, "encode"): 4_871_463_995,     # 1.000 x algorithmic
-    ("cfg3_llama1b", 15, "aggregate"): 5_677_780_002,  # 1.015 x (reads 1.106 x: index groups end inside shared lines)
-    ("cfg5_72b_block", 15, "encode"): 3_586_482_621,
-    ("cfg5_72b_block", 15, "aggregate"): 4_768_937_273,
-}
+def measured_traffic(workload, k, use_dct, peers, kernel):
+    """HBM bytes per launch of a whole-set kernel from hardware counters (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+    runs of `bench.py --profile ...`, scaled by the library's calibration copy): read from profiles/traffic.json,
+    which `bench_profiles.py summarise` writes beside the summaries that give the commands.  None for a launch
+    that has no entry there."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as fh:
+            table = json.load(fh)
+    except (OSError, ValueError):
+        return None
+    from bench_profiles import traffic_key
+
+    return table.get(traffic_key(workload, k, use_dct, peers, kernel))
 
 
 def parse():
@@ -58,7 +60,7 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--topk", type=int, default=0, help="top-k per chunk instead of the workload's own (templar runs 64)")
     ap.add_argument("--no-dct", action="store_true", help="chunks are selected and scattered untransformed (templar's use_dct=false)")
-    ap.add_argument("--profile", choices=["encode", "aggregate", "miner", "copy", "calib", "fill", "read", "linfill"], default=None,
+    ap.add_argument("--profile", choices=["encode", "aggregate", "miner", "copy", "calib", "fill", "read", "linfill", "outer"], default=None,
                     help="run only that phase's batched launches --steps times (for rocprofv3) and print nothing; "
                          "'copy' runs the library's calibration copy of 1 GiB instead (counter scaling); 'calib' / 'fill' "
                          "run the memory-only form of the aggregate kernel with / without its payload loads, 'read' the "
@@ -362,7 +364,7 @@ def main():
     # held as a staged window (PayloadStage: one device buffer, the peers' payloads equally spaced), the form
     # in which a gathered window reaches the aggregate
     idxs, vals, idxs_1d, vals_1d = [], [], [], []
-    window = tc.PayloadStage(batch, k, P, quantized=False) if args.profile in (None, "aggregate", "calib", "fill") else None
+    window = tc.PayloadStage(batch, k, P, quantized=False) if args.profile in (None, "aggregate", "calib", "fill", "outer") else None
     # the peers' norms as one float per payload row, noted when a peer's payload is in place (on arrival, in a
     # gather): the window's clip factors then take two small launches and no pass over the values
     norms = tc.PeerNorms([batch] + ([rows_1d] if rows_1d is not None else []), P) if window is not None else None
@@ -472,6 +474,16 @@ def main():
         return
     if args.profile == "aggregate":
         event_ms(aggregate_pass, args.steps, args.warmup, settle=True)
+        return
+    if args.profile == "outer":
+        prm = tc.TensorBatch([torch.zeros_like(o) for o in outs])
+        fac = (scale * 0.4).contiguous()
+        flg = torch.zeros(len(prm), dtype=torch.int32, device=dev)
+        pc_ = torch.empty((n_chunks, 2), dtype=torch.float32, device=dev)
+        pt_ = torch.empty((len(prm), 4), dtype=torch.float32, device=dev)
+        event_ms(lambda: _lib_mod.check(lib_c.tplr_outer_step_batch(
+            ip_c, vp_c, fac.data_ptr(), P, k, prm.table.data_ptr(), len(prm), n_chunks, pc_.data_ptr(), pt_.data_ptr(),
+            flg.data_ptr(), cur_stream), "tplr_outer_step_batch"), args.steps, args.warmup, settle=True)
         return
     agg_steps = max(3, args.steps // 2)
     agg_ms, agg_wall = event_ms(aggregate_pass, agg_steps, 2, settle=True)
@@ -774,9 +786,9 @@ def main():
             "bound": "hbm", "kernel": "k_encode_topk_pack",
             "achieved": round(enc2d_bytes / (enc2d_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(enc2d_bytes / (enc2d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC.get((args.workload, P, "encode")),
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload kept under profiles/, "
-                              "not measured by this run; null for other workloads",
+            "traffic": measured_traffic(args.workload, k, DCT, P, "encode"),
+            "traffic_source": "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this launch "
+                              "(bench_profiles.py), not measured by this run; null for launches not profiled",
             "launches_per_step": 1, "bytes_per_launch": enc2d_bytes, "ms_per_launch": round(enc2d_ms, 4),
             "ms_per_launch_median": enc2d_spread[0], "ms_per_launch_min": enc2d_spread[1],
             "ceiling": {"read_only_ms": round(enc_read_ms, 4),
@@ -790,9 +802,9 @@ def main():
             "bound": "hbm", "kernel": "k_decode_aggregate",
             "achieved": round(agg_bytes / (aggk_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(agg_bytes / (aggk_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC.get((args.workload, P, "aggregate")),
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload kept under profiles/, "
-                              "not measured by this run; null for other workloads",
+            "traffic": measured_traffic(args.workload, k, DCT, P, "aggregate"),
+            "traffic_source": "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this launch "
+                              "(bench_profiles.py), not measured by this run; null for launches not profiled",
             "launches_per_step": 1, "bytes_per_launch": agg_bytes, "ms_per_launch": round(aggk_ms, 4),
             "ms_per_launch_median": aggk_spread[0], "ms_per_launch_min": aggk_spread[1],
             "ceiling": ceiling,
