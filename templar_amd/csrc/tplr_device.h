@@ -5,6 +5,39 @@
 // coordinate) or in an LDS tile with a row stride of 68 floats, which makes both the
 // row-per-lane 16-byte accesses and the column-per-lane 4-byte accesses bank-conflict
 // free.  The decode kernel uses the 4 padding floats of a tile row as per-lane scratch slots.
+//
+// Hand-scheduled sequences.  The compiler inserts the wait states this hardware needs between dependent
+// instructions, but it does not look into inline assembly, and the assembler adds none.  Every assembly block
+// in this file and in tplr_hip.hip therefore pads for its own hazards, inside the block and at its edges (the
+// instruction after a block is the compiler's and may be of any kind).  The hazards, the rule applied, and where:
+//
+//   hazard                                                   rule here                        sequences
+//   -------------------------------------------------------  -------------------------------  ---------------------------
+//   a vector instruction writes a scalar register pair       two other instructions (or       filter16 (compares run three
+//   (compare result, carry-out) and a later VECTOR           s_nop 1 / s_nop 0 + one          ahead of the add-with-carry
+//   instruction reads that pair as a lane mask or carry-in   instruction) between the         chain, through three pairs);
+//   (v_cndmask, v_addc_co).  A scalar instruction reading    vector write and the vector      cmp_exchange, cx32_* (compare
+//   the pair in between (s_xnor) is interlocked by the       read                             or borrow -> s_xnor -> s_nop 0
+//   hardware and counts as one of the two.                                                    -> select)
+//   a vector instruction writes a vector register and a      s_nop 1 (two wait states)        end of cmp_exchange, cx32_*,
+//   data-parallel (DPP) instruction reads it as its moved    after the write, also when the   cx32_xor4 (after its v_mov_dpp),
+//   source                                                   write is the compiler's and the  sort64_desc_u32 / sort128_*_u32
+//                                                            DPP read is in a block (a        entry and the J == 64 step
+//                                                            leading "s_nop 1" on the value)
+//   vcc written inside a block and read by the next          the blocks name vcc / scc as     all blocks that touch them
+//   instruction of the same block                            clobbers and keep their own use
+//                                                            two instructions from the write
+//   a value that must not be hoisted out of a loop or        empty asm volatile("" : "+v")    select_topk (lane-derived
+//   merged with its copies (the optimiser then keeps         on the value: an opaque copy     addresses), k_decode_aggregate
+//   dozens of loop-invariant registers alive and spills)     the optimiser cannot see         (unit counts, peer count),
+//                                                            through, no instruction          dct64_inv_hooked call-outs
+//   a 16-byte buffer store reads its data registers after    no such store is issued from     (16-byte row stores were tried
+//   issue: rewriting one in the next instruction changes     hand-written code; the           and dropped; k_row_sumsq_vec
+//   what is stored                                           compiler's own are padded by it  and the calibration fills are
+//                                                                                             compiler-scheduled)
+//
+// A new block, or a reordering of an old one, has to be checked against these rows; the select tests with ties,
+// NaNs and short keys (tests/test_gpu_kernels.py) are the ones that fail when a mask or a partner is read early.
 #pragma once
 
 #include <hip/hip_runtime.h>
