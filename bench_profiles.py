@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """rocprofv3 runs behind the summaries under profiles/, and the summaries themselves.
 
-  python bench_profiles.py run [--sets cfg3,cfg5,prod,nodct] [--phases encode,aggregate,...]
+  python bench_profiles.py run [--sets cfg3,cfg5,prod,nodct,bench] [--phases encode,aggregate,...]
       on a box with an MI355X: for every (set, phase) a kernel trace of `bench.py --profile <phase>` (50 timed
       launches after the settle phase and 10 warm-up ones), and one run each for the FETCH_SIZE, WRITE_SIZE and
       (encode, aggregate) SQ_* counters.  Raw CSVs go to gpurun_out/prof/<set>_<phase>_<what>/, trimmed to this
@@ -100,6 +100,9 @@ def _profile(tag, what, prof_args, bench_args, limit):
 def run(sets, phases):
     os.makedirs(RAW, exist_ok=True)
     for tag in sets:
+        if tag == "bench":  # the default benchmark run as a whole: every kernel of the library once
+            _profile("bench_default", "kt", ["--kernel-trace", "--stats"], ["--no-cpu-baseline"], 400)
+            continue
         S = SETS[tag]
         for ph in S["phases"]:
             if phases and ph not in phases:
@@ -486,6 +489,18 @@ From `p_kernel_trace.csv` (the last 50 launches of each kernel):
 |---|---|---|---|---|---|---|---|
 {chr(10).join(rows)}
 """)
+    if _have("bench_default"):
+        write("bench_default_cfg3_llama1b.md", f"""# bench.py (default arguments), 1B gradient set: all kernels of this library
+
+    {PRE}rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof/bench_default_kt -o p -- python3 bench.py --no-cpu-baseline
+
+`p_kernel_stats.csv`, rows of this library's kernels (the run also times the one-launch-per-tensor paths, the
+calibration launches and the settle phases, so the fused kernels appear with many launches of several sizes; their
+whole-set launches are profiled alone in k_encode_topk_pack_cfg3_llama1b.md and
+k_decode_aggregate_cfg3_llama1b_15peers.md):
+
+{_stats_table('bench_default')}
+""")
     if traffic:
         traffic["what"] = ("HBM bytes per launch of the whole-set kernels (FETCH_SIZE + WRITE_SIZE, each scaled by the calibration "
                            "copy), keyed workload/peers/kernel; written by bench_profiles.py summarise from the rocprofv3 runs whose "
@@ -499,13 +514,13 @@ From `p_kernel_trace.csv` (the last 50 launches of each kernel):
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("what", choices=["run", "summarise"])
-    ap.add_argument("--sets", default=",".join(SETS))
+    ap.add_argument("--sets", default=",".join(SETS) + ",bench")
     ap.add_argument("--phases", default="")
     ap.add_argument("--out", default=os.path.join(ROOT, "profiles"))
     args = ap.parse_args()
     sets = [s for s in args.sets.split(",") if s]
     for s in sets:
-        if s not in SETS:
+        if s not in SETS and s != "bench":
             ap.error(f"unknown set {s}")
     if args.what == "run":
         run(sets, [p for p in args.phases.split(",") if p])
