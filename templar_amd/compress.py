@@ -1554,6 +1554,35 @@ def batch_decompress_decode_rows_batch(out: RowBatch, idxs: Sequence[torch.Tenso
 
 
 @torch.no_grad()
+def outer_step_rows_batch(params: RowBatch, idxs: Sequence[torch.Tensor], vals: Sequence[torch.Tensor], k: int, lr: float, *,
+                          scale: torch.Tensor | None = None, use_dct: bool = True, stats: bool = True):
+    """outer_step_batch for the 1-D parameters (src/tplr/neurons.py:341-447 with the plain SGD of
+    neurons/trainer.py:128-130): the peers' payloads are aggregated and decoded in one launch into a scratch
+    copy of the set (a few hundred KB for a model's norm vectors), every parameter whose gradient is finite
+    takes p <- p - lr * grad, the others keep their bits.  Returns (stats, skipped) as outer_step_batch does."""
+    if lr == 0 or lr != lr:
+        raise ValueError(f"lr must be a non-zero number, got {lr}")
+    dev = params.device
+    grads = [torch.empty_like(t) for t in params.tensors]
+    batch_decompress_decode_rows_batch(RowBatch(grads), idxs, vals, k, clip_norm=scale is None, use_dct=use_dct,
+                                       validate=False, scale=scale)
+    flat = torch.cat([g.reshape(-1) for g in grads]).double()
+    sizes = torch.tensor([g.numel() for g in grads], device=dev)
+    seg = torch.repeat_interleave(torch.arange(len(grads), device=dev), sizes)
+    ss = torch.zeros(len(grads), dtype=torch.float64, device=dev).index_add_(0, seg, flat * flat)
+    sm = torch.zeros(len(grads), dtype=torch.float64, device=dev).index_add_(0, seg, flat)
+    finite = torch.isfinite(ss) & torch.isfinite(sm)  # a NaN or an infinity in a gradient shows in its sums
+    keep = finite.tolist()  # the call's one synchronisation
+    good = [i for i, ok in enumerate(keep) if ok]
+    if good:
+        torch._foreach_sub_([params.tensors[i] for i in good], [grads[i] for i in good], alpha=float(lr))
+    out = None
+    if stats:
+        out = torch.stack([ss.sqrt(), sm / sizes.double(), finite.double(), ss], dim=1).float()
+    return out, [i for i, ok in enumerate(keep) if not ok]
+
+
+@torch.no_grad()
 def error_feedback_step_rows_batch(ef: RowBatch, grad: RowBatch, decay: float, topk: int, *, use_dct: bool = True,
                                    compressor: "TopKCompressor | None" = None, null_round: bool = False):
     """error_feedback_step_batch for the 1-D parameters: the loop body of src/tplr/neurons.py:147-171
@@ -2065,6 +2094,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "apply_decoded_batch", "outer_step_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "PeerNorms", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "apply_decoded_batch", "outer_step_batch", "outer_step_rows_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "PeerNorms", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

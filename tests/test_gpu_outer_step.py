@@ -159,3 +159,42 @@ def test_outer_step_argument_checks(dev):
     assert lib.tplr_outer_step_batch(ip, vp, None, 2, 2, t, 1, 2, None, None, None, None) == _lib.TPLR_E_BADARG
     assert lib.tplr_outer_step_batch(ip, vp, None, 2, 32, t, 1, 2, vals[0].data_ptr(), None, None, None) == _lib.TPLR_E_BADARG
     assert lib.tplr_outer_step_batch(None, vp, None, 2, 32, t, 1, 2, None, None, None, None) == _lib.TPLR_E_BADARG
+
+
+@pytest.mark.parametrize("use_dct", [True, False])
+def test_outer_step_of_the_one_dimensional_parameters(dev, use_dct):
+    # the norm vectors of a model: rows of 64, the same reference lines; oracle = its batch_decompress (pinned
+    # against torch) + the 64-point inverse transform (pinned against scipy) + the SGD line
+    lengths = [64, 2048, 128, 768]
+    P, k, lr = 5, 32, 0.4
+    base = [t3((n,), 70 + i).to(dev) * (i + 1) for i, n in enumerate(lengths)]
+    rb = tc.RowBatch(base)
+    pay = []
+    for p in range(P):
+        pg = [0.5 * g + t3(tuple(g.shape), 500 + 10 * p + i).to(dev) * (1 + p) for i, g in enumerate(base)]
+        pay.append(tc.encode_compress_rows_batch(tc.RowBatch(pg), k, use_dct=use_dct))
+    idxs, vals = [a for a, _ in pay], [b.clone() for _, b in pay]
+    vals[1][rb.offsets[2], 3] = float("nan")        # parameter 2 gets a poisoned gradient
+    start = [torch.randn(n, device=dev) for n in lengths]
+    params = [s.clone() for s in start]
+    stats, skipped = tc.outer_step_rows_batch(tc.RowBatch(params), idxs, vals, k, lr, use_dct=use_dct)
+    assert skipped == [2] and float(stats[2, 2]) == 0.0
+    assert torch.equal(params[2].view(torch.int32), start[2].view(torch.int32))
+    for i, n in enumerate(lengths):
+        if i == 2:
+            continue
+        sl = [rb.payload_slice(i, idxs[p], vals[p], k) for p in range(P)]
+        ref = orc.batch_decompress([a.cpu().numpy() for a, _ in sl], [b.cpu().numpy() for _, b in sl], (n // 64, 64), 64)
+        grad = (orc.dct1d(ref, inverse=True) if use_dct else ref).reshape(-1)
+        want = start[i].cpu().numpy() - np.float32(lr) * grad
+        assert np.abs(params[i].cpu().numpy() - want).max() <= TOL * np.abs(want).max()
+        assert np.isclose(float(stats[i, 0]), np.sqrt((grad.astype(np.float64) ** 2).sum()), rtol=2e-5)
+        assert abs(float(stats[i, 1]) - grad.astype(np.float64).mean()) <= 2e-5 * np.abs(grad).max()
+        assert float(stats[i, 2]) == 1.0
+    # ready clip factors give the same bits
+    again = [s.clone() for s in start]
+    norms = tc.PeerNorms([rb], P)
+    for p in range(P):
+        norms.arrived(p, [vals[p]])
+    tc.outer_step_rows_batch(tc.RowBatch(again), idxs, vals, k, lr, use_dct=use_dct, scale=norms.clip_scales(P)[0], stats=False)
+    assert all(torch.equal(a.view(torch.int32), b.view(torch.int32)) for a, b in zip(again, params))
