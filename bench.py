@@ -654,6 +654,22 @@ def main():
 
         c_ms, c_wall = event_ms(from_codes, agg_steps, 2, settle=True)
         d_ms, d_wall = event_ms(dequantise_first, agg_steps, 2)
+        # the outer step from the same codes: p <- p - lr * aggregate in the launch that forms it, against the
+        # aggregate from codes with statistics followed by a foreach subtraction of the dense gradients
+        prm = [torch.zeros_like(o) for o in outs]
+        pbt = tc.TensorBatch(prm)
+        o_ms, o_wall = event_ms(lambda: tc.outer_step_codes_batch(pbt, idxs_, codes, None, kk, 0.4, tables=q_tables,
+                                                                  validate=False), agg_steps, 2)
+
+        def codes_then_sgd():
+            st = tc.batch_decompress_decode_codes_batch(out_batch, idxs_, codes, qps, kk, validate=False, tables=q_tables,
+                                                        stats=True)
+            if bool((st[:, 2] == 1).all()):
+                torch._foreach_sub_(prm, outs, alpha=0.4)
+
+        s_ms, s_wall = event_ms(codes_then_sgd, agg_steps, 1)
+        del prm, pbt
+        outer_bytes = n_chunks * (PP * (kk + kk // 2 + kk) + 2 * 16384)
         code_bytes = n_chunks * (PP * (kk + kk // 2 + kk) + 16384)
         return {"what": f"aggregate of the 2-D set from 4-bin codes, {PP} peers, k = {kk}, chunks not transformed (index "
                         "bytes + one byte per value read, dense written; norms from counts; no fp32 copy of the payload) "
@@ -662,7 +678,15 @@ def main():
                 "dequantise_first_ms": round(d_ms, 4), "dequantise_first_wall_ms": round(d_wall, 4),
                 "from_codes_bytes": code_bytes,
                 "from_codes_GBps": round(code_bytes / (c_ms * 1e-3) / 1e9, 2),
-                "from_codes_frac_of_hbm_peak": round(code_bytes / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                "from_codes_frac_of_hbm_peak": round(code_bytes / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                "outer_step_from_codes_ms": round(o_ms, 4), "outer_step_from_codes_wall_ms": round(o_wall, 4),
+                "outer_step_from_codes_bytes": outer_bytes,
+                "outer_step_from_codes_GBps": round(outer_bytes / (o_ms * 1e-3) / 1e9, 2),
+                "outer_step_what": "p <- p - lr * aggregate for every 2-D parameter straight from the codes (norms from "
+                                   "counts, clip factors, one fused launch, per-parameter statistics and non-finite "
+                                   "flags read back: the whole call with its one synchronisation), against the "
+                                   "aggregate from codes with statistics followed by a foreach subtraction",
+                "aggregate_from_codes_then_sgd_ms": round(s_ms, 4), "aggregate_from_codes_then_sgd_wall_ms": round(s_wall, 4)}
 
     codes_path = None
     if not DCT and k <= 64 and P <= 24 and args.profile is None:

@@ -341,6 +341,16 @@ int tplr_outer_step_batch(const uint8_t* const* h_idx12, const float* const* h_v
                           int64_t total_chunks, float* d_chunk_stats, float* d_tensor_stats, int32_t* d_nonfinite,
                           void* stream);
 
+/* The same outer step straight from quantised payloads at templar's own settings (4-bin codes, chunks not
+ * transformed, hparams/hparams.json): h_codes, d_deq as in tplr_decode_aggregate_codes_batch, d_factor[t * n_peers + p]
+ * multiplies peer p's de-quantised values for tensor t (pass lr * clip factor).  The peers' payloads must be equally
+ * spaced in memory and four-byte aligned, as a staged window lays them out (else TPLR_E_SHAPE); k = 32 or 64;
+ * n_peers <= 24.  d_chunk_stats, d_tensor_stats, d_nonfinite as in tplr_outer_step_batch. */
+int tplr_outer_step_codes_batch(const uint8_t* const* h_idx12, const uint8_t* const* h_codes, const float* d_deq,
+                                const float* d_factor, int n_peers, int k, const tplr_tensor_desc* d_param_desc,
+                                int n_tensors, int64_t total_chunks, float* d_chunk_stats, float* d_tensor_stats,
+                                int32_t* d_nonfinite, void* stream);
+
 /* ---- validator side: checks on the packed index streams ------------------------------
  * For up to 32 peers whose flat payloads share one row layout (d_desc: n_tensors descriptors, of
  * which only chunk_begin, x_chunks and y_chunks are read; a parameter of n rows that are not

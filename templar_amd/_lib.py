@@ -60,6 +60,7 @@ SIGNATURES = {
     "tplr_ef_encode_topk_pack_batch": (_i32, [_vp, _vp, _i32, _i64, C.c_float, _i32, _i32, _vp, _vp, _vp]),
     "tplr_ef_subtract_batch": (_i32, [_vp, _vp, _i32, _vp, _i32, _i64, _i32, _vp]),
     "tplr_apply_decoded_batch": (_i32, [_vp, _vp, _vp, _i32, _vp, _i32, _i64, _i32, _vp, _vp]),
+    "tplr_outer_step_codes_batch": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp, _vp, _vp]),
     "tplr_outer_step_batch": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp, _vp, _vp]),
     "tplr_ef_step_batch": (_i32, [_vp, _vp, _i32, _i64, C.c_float, _i32, _vp, _vp, _vp]),
     "tplr_ef_subtract_own_batch": (_i32, [_vp, _vp, _vp, _i32, _vp, _i32, _i64, _vp]),

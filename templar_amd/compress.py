@@ -1847,6 +1847,92 @@ def batch_decompress_decode_codes_batch(out: TensorBatch, idxs: Sequence[torch.T
     return None
 
 
+@torch.no_grad()
+def outer_step_codes_batch(params: TensorBatch, idxs: Sequence[torch.Tensor], codes: Sequence[torch.Tensor],
+                           quant_params: "Sequence[Sequence[QuantParamsT]] | None", k: int, lr: float, *,
+                           tables: "tuple[torch.Tensor, int] | None" = None, stats: bool = True, validate: bool = True):
+    """outer_step_batch at templar's own settings (hparams/hparams.json: 4-bin quantiser, chunks not transformed,
+    top-k 64, 20 peers): maybe_dequantize_values, block norms, batch_decompress, decode, the gradient's norm, mean and
+    isfinite test and SGD's p <- p - lr * grad (src/tplr/neurons.py:325-447, neurons/trainer.py:128-130) for every
+    2-D parameter in one launch straight from the codes - no fp32 copy of the payload, no dense gradient.
+    codes[p], quant_params[i][p] / `tables` as in batch_decompress_decode_codes_batch; the payloads must be a staged
+    window (PayloadStage.load(..., expand=False)).  Returns (stats, skipped) as outer_step_batch does.  A parameter the
+    fused launch cannot vouch for, and settings it does not serve (more than four bins, k other than 32 or 64, more
+    than 24 peers, payloads not equally spaced), take the reference's route on de-quantised values inside the call.
+    `validate` raises IndexError on a code the quantiser cannot have produced, before anything is written."""
+    lib = _lib.load()
+    P, T, n, dev = len(codes), len(params), params.total_chunks, params.device
+    if lr == 0 or lr != lr:
+        raise ValueError(f"lr must be a non-zero number, got {lr}")
+    if tables is None and (quant_params is None or len(quant_params) != T or any(len(q) != P for q in quant_params)):
+        raise IndexError("quant_params must hold one entry per parameter and peer")
+    for i, c in zip(idxs, codes):
+        if i.dtype != torch.uint8:
+            raise ValueError(f"Expected uint8 for 12-bit packed indices, got {i.dtype}")
+        if c.dtype != torch.uint8 or c.numel() != n * k or i.numel() * 2 != n * k * 3 or not c.is_contiguous():
+            raise RuntimeError(f"flat payload mismatch: {i.numel()} index bytes / {c.numel()} codes for {n} chunks, k={k}")
+    deq, n_bins = tables if tables is not None else dequantised_tables(quant_params, dev)
+
+    def dequantised(t=None):
+        """fp32 values behind the codes: of parameter t per peer ((rows, k) each), or of everything per peer."""
+        if t is None:
+            seg = torch.repeat_interleave(torch.arange(T, device=dev),
+                                          torch.tensor([params.payload_rows(i) for i in range(T)], device=dev))
+            return [deq[seg, p].gather(1, codes[p].view(n, k).long()) for p in range(P)]
+        b, rows = params.offsets[t], params.payload_rows(t)
+        return [deq[t, p][codes[p].view(n, k)[b:b + rows].long()] for p in range(P)]
+
+    if n_bins > 4 or k not in (32, 64) or P > 24 or deq.shape != (T, P, 4):
+        return outer_step_batch(params, idxs, dequantised(), k, lr, use_dct=False, stats=stats)
+    ip = (C.c_void_p * P)(*[i.data_ptr() for i in idxs])
+    cp = (C.c_void_p * P)(*[c.data_ptr() for c in codes])
+    slices = max(1, min(64, 8192 // (T * P)))
+    ss = torch.empty((T, P, slices), dtype=torch.float32, device=dev)
+    scale = torch.empty((T, P), dtype=torch.float32, device=dev)
+    bad = torch.zeros(1, dtype=torch.int32, device=dev)
+    with _on(dev):
+        _lib.check(lib.tplr_code_sumsq(cp, P, k, _ptr(params.table), T, slices, n_bins, _ptr(deq), _ptr(ss), _ptr(bad),
+                                       _stream(dev)), "tplr_code_sumsq")
+        _lib.check(lib.tplr_clip_scales_batch(_ptr(ss), T, P, slices, _ptr(scale), None, _stream(dev)),
+                   "tplr_clip_scales_batch")
+    if validate:
+        worst = int(bad.item())
+        if worst:
+            raise IndexError(f"index {worst} is out of bounds for dimension 0 with size {n_bins}")
+    sound = (torch.isfinite(scale) & (scale > 0)).all(dim=1, keepdim=True)
+    factor = torch.where(sound, scale * float(lr), torch.full_like(scale, float("nan"))).contiguous()
+    flags = torch.zeros(T, dtype=torch.int32, device=dev)
+    out = torch.zeros((T, 4), dtype=torch.float32, device=dev) if stats else None
+    per_chunk = torch.empty((max(n, 1), 2), dtype=torch.float32, device=dev) if stats else None
+    with _on(dev):
+        st = lib.tplr_outer_step_codes_batch(ip, cp, _ptr(deq), _ptr(factor), P, k, _ptr(params.table), T, n,
+                                             _ptr(per_chunk), _ptr(out), _ptr(flags), _stream(dev))
+    if st == _lib.TPLR_E_SHAPE:  # the payloads are not a staged window
+        return outer_step_batch(params, idxs, dequantised(), k, lr, use_dct=False, stats=stats)
+    _lib.check(st, "tplr_outer_step_codes_batch")
+    if stats:  # the launch's figures are those of lr * grad
+        out[:, 0] /= abs(float(lr))
+        out[:, 1] /= float(lr)
+        out[:, 3] /= float(lr) * float(lr)
+    skipped = []
+    for t in torch.nonzero(flags).reshape(-1).tolist():  # the reference's own sequence, one parameter at a time
+        y, x = params.xshape(t)[:2]
+        b, rows = params.offsets[t], params.payload_rows(t)
+        ti = [i[b * (k // 2) * 3:(b + rows) * (k // 2) * 3].contiguous() for i in idxs]
+        grad = _aggregate_chunks(ti, [v.contiguous() for v in dequantised(t)], scale[t].contiguous(), y, x, k,
+                                 normalise=False, use_dct=False, rows=True)
+        finite = bool(torch.isfinite(grad).all())
+        if stats:
+            s2 = (grad.double() ** 2).sum()
+            out[t] = torch.stack([s2.sqrt(), grad.double().mean(), torch.tensor(float(finite), device=dev, dtype=torch.float64),
+                                  s2]).float()
+        if finite:
+            params.tensors[t].sub_(grad, alpha=float(lr))
+        else:
+            skipped.append(t)
+    return out, skipped
+
+
 class PayloadStage:
     """One window's payloads of all peers as flat buffers in the layout the batch kernels read.
 
@@ -2094,6 +2180,6 @@ CompressDCT = TopKCompressor
 __all__ = [
     "pack_12bit_indices", "unpack_12bit_indices", "ChunkingTransformer", "TopKCompressor", "TransformDCT",
     "CompressDCT", "encode_compress", "batch_decompress_decode", "LazyAggregate", "TensorBatch",
-    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "apply_decoded_batch", "outer_step_batch", "outer_step_rows_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "PeerNorms", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
+    "encode_compress_batch", "batch_decompress_decode_batch", "aggregate_mean_normalised_batch", "apply_decoded_batch", "outer_step_batch", "outer_step_rows_batch", "outer_step_codes_batch", "batch_decompress_decode_codes_batch", "dequantised_tables", "peer_clip_scales_batch", "error_feedback_step_batch", "index_stats_batch", "overlap_fractions", "dequantize_batch", "quantize_batch", "PayloadStage", "PeerNorms", "RowBatch", "encode_compress_rows_batch", "batch_decompress_decode_rows_batch", "error_feedback_step_rows_batch", "check_compressed_indices", "ShapeT", "Shape4D", "TotK",
     "IdxT", "ValT", "QuantParamsT", "_dct", "_idct", "_get_smaller_split", "_get_divisors", "_get_prime_divisors",
 ]

@@ -715,7 +715,8 @@ struct Counters {
 // Generic path (kUnits == 0): any k and peer count, entries loaded where they are used.
 // kSubtract (fast path with the transform only): the destination receives destination - result
 // instead of the result (the error-feedback update of src/tplr/neurons.py:171); its rows are
-// requested before the second pass and arrive during it.  With `guard` (one int per tensor, zeroed by the
+// requested before the second pass and arrive during it (without the transform, codes through wide loads:
+// requested when the chunk leaves the tile, before it is read out).  With `guard` (one int per tensor, zeroed by the
 // caller) a chunk whose result holds a NaN or an infinity is not subtracted - its destination keeps its
 // bits - and guard[tensor] becomes 1: the validator's check of the decoded gradient before
 // p.data.sub_ (neurons/validator.py:3646-3660).
@@ -746,7 +747,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                                                             int64_t stride_idx, int64_t stride_val,
                                                             const float* __restrict__ deq,
                                                             int32_t* __restrict__ guard) {
-    static_assert(!kCodes || (kUnits > 0 && !kUseDct && !kSubtract), "codes are served by the fast path without the transform");
+    static_assert(!kCodes || (kUnits > 0 && !kUseDct), "codes are served by the fast path without the transform");
+    static_assert(!(kCodes && kSubtract) || kWideK > 0, "the subtraction from codes: the wide-load pipeline only");
     static_assert(kWideK == 0 || (kCodes && kStrided && (kWideK == 32 || kWideK == 64)), "wide loads: codes, equally spaced payloads");
     // this launch covers the chunks first .. first + total - 1 of the batch
     // options: bit 0 = per-peer, per-chunk normalisation (generic instantiation); bit 1 = `sumsq` takes two
@@ -1649,7 +1651,12 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 int lane = threadIdx.x;
                 asm volatile("" : "+v"(lane));
                 float v[64];
-                if (out_cur.ld > 0) {  // wave-uniform
+                gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0));
+                // kSubtract: the destination is a (R, C) tensor; its rows are requested first and arrive while
+                // the tile is read out
+                float before[kSubtract ? 64 : 1];
+                if constexpr (kSubtract) load_chunk_rows(before, (const void*)dst, uniform64(out_cur.ld), lane);
+                if (kSubtract || out_cur.ld > 0) {  // wave-uniform
                     tile_cols_to_regs(v, tile, lane);
                 } else {
 #pragma unroll
@@ -1661,9 +1668,14 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 }
                 wave_lds_fence();
                 chunk_stats(v, g, skip_cur);
-                gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0));
-                if (out_cur.ld > 0) {
-                    store_chunk_rows(v, (void*)dst, uniform64(out_cur.ld), lane, skip_cur);
+                bool tripped = false;
+                if constexpr (kSubtract) {
+                    if (!skip_cur) tripped = guard_trips(v, out_cur.t);
+#pragma unroll
+                    for (int r = 0; r < 64; ++r) v[r] = before[r] - v[r];
+                }
+                if (kSubtract || out_cur.ld > 0) {
+                    store_chunk_rows(v, (void*)dst, uniform64(out_cur.ld), lane, skip_cur || tripped);
                 } else if (!skip_cur) {
 #pragma unroll
                     for (int q0 = 0; q0 < 16; ++q0)
@@ -3635,6 +3647,56 @@ int tplr_outer_step_batch(const uint8_t* const* h_idx12, const float* const* h_v
     if (d_tensor_stats)
         hipLaunchKernelGGL(k_tensor_stats, dim3(static_cast<unsigned>(n_tensors)), dim3(256), 0,
                            static_cast<hipStream_t>(stream), d_chunk_stats, d_param_desc, 1 | 2, d_tensor_stats);
+    return launch_status();
+}
+
+int tplr_outer_step_codes_batch(const uint8_t* const* h_idx12, const uint8_t* const* h_codes, const float* d_deq,
+                                const float* d_factor, int n_peers, int k, const tplr_tensor_desc* d_param_desc,
+                                int n_tensors, int64_t total_chunks, float* d_chunk_stats, float* d_tensor_stats,
+                                int32_t* d_nonfinite, void* stream) {
+    if (!h_idx12 || !h_codes || !d_deq || !d_param_desc || n_peers < 1 || n_tensors < 1 || total_chunks < 0)
+        return TPLR_E_BADARG;
+    if ((d_chunk_stats == nullptr) != (d_tensor_stats == nullptr)) return TPLR_E_BADARG;
+    if (k != 32 && k != 64) return TPLR_E_BADARG;   // the wide-load pipeline's two row lengths
+    if (n_peers > 24) return TPLR_E_TOOMANY;
+    PeerPtrs pp;
+    for (int p = 0; p < TPLR_MAX_PEERS; ++p) {
+        pp.idx[p] = p < n_peers ? h_idx12[p] : nullptr;
+        pp.val[p] = p < n_peers ? reinterpret_cast<const float*>(h_codes[p]) : nullptr;
+        if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
+    }
+    auto apart = [](const void* a, const void* b) {
+        return static_cast<int64_t>(reinterpret_cast<intptr_t>(a) - reinterpret_cast<intptr_t>(b));
+    };
+    const int64_t si = n_peers > 1 ? apart(pp.idx[1], pp.idx[0]) : 0;
+    const int64_t sv = n_peers > 1 ? apart(pp.val[1], pp.val[0]) : 0;
+    bool wide = (reinterpret_cast<uintptr_t>(pp.val[0]) & 3) == 0 && (sv & 3) == 0 && sv >= 0 && si >= 0 &&
+                (reinterpret_cast<uintptr_t>(pp.idx[0]) & 3) == 0 && (si & 3) == 0 && sv * n_peers < (int64_t{1} << 32) &&
+                si * n_peers < (int64_t{1} << 32);
+    for (int p = 1; p < n_peers; ++p)
+        wide = wide && apart(pp.idx[p], pp.idx[0]) == p * si && apart(pp.val[p], pp.val[0]) == p * sv;
+    if (!wide) return TPLR_E_SHAPE;  // the peers' payloads must be equally spaced, four-byte aligned (a staged window)
+    if (total_chunks > 0) {
+        tplr_tensor_desc none = {};
+        const int options = d_chunk_stats ? 2 : 0;
+        int st;
+#define TPLR_OUTER_CODES(U, BITS)                                                                                       \
+    (k == 64 ? launch_decode_as(k_decode_aggregate<false, U, BITS, true, true, true, 64>, pp, d_factor, n_peers, k,      \
+                                d_param_desc, none, n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats,  \
+                                stream, si, sv, d_deq, d_nonfinite)                                                     \
+             : launch_decode_as(k_decode_aggregate<false, U, BITS, true, true, true, 32>, pp, d_factor, n_peers, k,      \
+                                d_param_desc, none, n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats,  \
+                                stream, si, sv, d_deq, d_nonfinite))
+        if (n_peers <= 15)
+            st = TPLR_OUTER_CODES(16, 4);
+        else
+            st = TPLR_OUTER_CODES(24, 5);
+#undef TPLR_OUTER_CODES
+        if (st) return st;
+    }
+    if (d_tensor_stats)
+        hipLaunchKernelGGL(k_tensor_stats, dim3(static_cast<unsigned>(n_tensors)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), d_chunk_stats, d_param_desc, 2, d_tensor_stats);
     return launch_status();
 }
 

@@ -198,3 +198,74 @@ def test_outer_step_of_the_one_dimensional_parameters(dev, use_dct):
         norms.arrived(p, [vals[p]])
     tc.outer_step_rows_batch(tc.RowBatch(again), idxs, vals, k, lr, use_dct=use_dct, scale=norms.clip_scales(P)[0], stats=False)
     assert all(torch.equal(a.view(torch.int32), b.view(torch.int32)) for a, b in zip(again, params))
+
+
+def _codes_window(dev, shapes, k, P, bins=4):
+    """P peers' staged 4-bin payloads of untransformed chunks: (batch, idxs, codes, quant_params, fp32 values)."""
+    base = [t3(s, 300 + i, row_scale=True).to(dev) for i, s in enumerate(shapes)]
+    batch = tc.TensorBatch(base)
+    T, n = len(shapes), batch.total_chunks
+    stage = tc.PayloadStage(batch, k, P, quantized=True)
+    idxs, codes, qps, fp32 = [], [], [[None] * P for _ in range(T)], []
+    for p in range(P):
+        own = [0.5 * g + t3(tuple(g.shape), 6000 + 10 * p + i, row_scale=True).to(dev) * (1 + 0.3 * p) for i, g in enumerate(base)]
+        i12, c = stage.regions(p)
+        idx_p, val_p = tc.encode_compress_batch(tc.TensorBatch(own), k, use_dct=False)
+        cc, shift, scale, lookup = tc.quantize_batch(batch, val_p, k, bins, 6.0)
+        i12.copy_(idx_p)
+        c.copy_(cc)
+        for i in range(T):
+            qps[i][p] = (shift[i].clone(), float(scale[i]), bins // 2, lookup[i].clone(), torch.float32)
+        idxs.append(i12)
+        codes.append(c)
+        fp32.append(tc.dequantize_batch(batch, c.reshape(-1), [qps[i][p] for i in range(T)], k))
+    return batch, idxs, codes, qps, fp32
+
+
+@pytest.mark.parametrize("P,k", [(20, 64), (15, 32), (4, 64), (24, 32)])
+def test_outer_step_straight_from_four_bin_codes(dev, P, k):
+    # templar's own settings (hparams.json: 4-bin quantiser, use_dct false, top-k 64, 20 peers): against the oracle's
+    # outer step on the de-quantised values, and against the same call's reference route on the device
+    shapes = [(128, 192), (64, 64), (256, 256), (192, 128)]
+    batch, idxs, codes, qps, fp32 = _codes_window(dev, shapes, k, P)
+    start = [torch.randn(s, device=dev) for s in shapes]
+    params = [s.clone() for s in start]
+    lr = 0.4
+    stats, skipped = tc.outer_step_codes_batch(tc.TensorBatch(params), idxs, codes, qps, k, lr)
+    _check_against_oracle(batch, params, start, idxs, fp32, k, lr, stats, skipped, False)
+    # the reference route on the de-quantised values: the same tensors within rounding of the clip factors
+    other = [s.clone() for s in start]
+    stats2, skipped2 = tc.outer_step_batch(tc.TensorBatch(other), idxs, fp32, k, lr, use_dct=False)
+    assert skipped2 == []
+    for a, b in zip(params, other):
+        assert float((a - b).abs().max()) <= 1e-6 * float(b.abs().max())
+    assert torch.allclose(stats[:, 0], stats2[:, 0], rtol=2e-5)
+    # payloads that are not a staged window take the other route inside the call: same result
+    loose = [s.clone() for s in start]
+    tc.outer_step_codes_batch(tc.TensorBatch(loose), [i.clone() for i in idxs], [c.clone() for c in codes], qps, k, lr, stats=False)
+    for a, b in zip(loose, other):
+        assert float((a - b).abs().max()) <= 1e-6 * float(b.abs().max())
+
+
+def test_outer_step_from_codes_leaves_a_poisoned_parameter_alone(dev):
+    shapes = [(128, 192), (256, 128), (64, 64)]
+    k, P, lr = 64, 6, 0.3
+    batch, idxs, codes, qps, fp32 = _codes_window(dev, shapes, k, P)
+    # peer 2's table for parameter 1 carries an infinity (a corrupt quant_params tuple)
+    sh, sc, off, lut, dt = qps[1][2]
+    lut = lut.clone()
+    lut[1] = float("inf")
+    qps[1][2] = (sh, sc, off, lut, dt)
+    fp32[2] = tc.dequantize_batch(batch, codes[2].reshape(-1), [qps[i][2] for i in range(len(shapes))], k)
+    start = [torch.randn(s, device=dev) for s in shapes]
+    params = [s.clone() for s in start]
+    stats, skipped = tc.outer_step_codes_batch(tc.TensorBatch(params), idxs, codes, qps, k, lr)
+    _check_against_oracle(batch, params, start, idxs, fp32, k, lr, stats, skipped, False, expect_skipped=[1])
+    # a code past the quantiser's bins raises before anything is written
+    spoiled = [c.clone() for c in codes]
+    params = [s.clone() for s in start]
+    stage = torch.stack([c.reshape(-1) for c in spoiled])
+    stage[3, 17] = 9
+    with pytest.raises(IndexError):
+        tc.outer_step_codes_batch(tc.TensorBatch(params), idxs, [stage[p].view(-1, k) for p in range(P)], qps, k, lr)
+    assert all(torch.equal(a, b) for a, b in zip(params, start))
