@@ -269,3 +269,23 @@ def test_outer_step_from_codes_leaves_a_poisoned_parameter_alone(dev):
     with pytest.raises(IndexError):
         tc.outer_step_codes_batch(tc.TensorBatch(params), idxs, [stage[p].view(-1, k) for p in range(P)], qps, k, lr)
     assert all(torch.equal(a, b) for a, b in zip(params, start))
+
+
+def test_outer_step_seeded_sweep(dev):
+    # twenty draws of shapes, peer counts, k, learning rates and layouts, each against the oracle
+    rng = np.random.default_rng(2024)
+    for draw in range(20):
+        T = int(rng.integers(1, 5))
+        shapes = [(64 * int(rng.integers(1, 5)), 64 * int(rng.integers(1, 5))) for _ in range(T)]
+        P = int(rng.integers(1, 16))
+        k = int(rng.choice([4, 8, 16, 32, 64]))
+        lr = float(rng.choice([-1.0, 1.0]) * rng.uniform(0.01, 2.0))
+        staged = bool(rng.integers(0, 2))
+        batch, idxs, vals, _ = _window(dev, shapes, k, P, staged=staged)
+        start = [torch.randn(s, device=dev) * float(rng.uniform(0.01, 10.0)) for s in shapes]
+        params = [s.clone() for s in start]
+        stats, skipped = tc.outer_step_batch(tc.TensorBatch(params), idxs, vals, k, lr)
+        try:
+            _check_against_oracle(batch, params, start, idxs, vals, k, lr, stats, skipped, True)
+        except AssertionError as e:
+            raise AssertionError(f"draw {draw}: shapes {shapes}, P {P}, k {k}, lr {lr}, staged {staged}: {e}") from e

@@ -176,3 +176,50 @@ def test_staged_window_leaves_the_row_figures(dev):
         assert torch.equal(s1, tc.peer_clip_scales_batch(b1, [v for _, v in pay1], k))
     with pytest.raises(ValueError):
         tc.PayloadStage(b2, k, P, quantized=False, norms=tc.PeerNorms([b1, b2], max_peers=P))
+
+
+def test_peer_norms_seeded_sweep(dev):
+    # thirty draws of row counts, row lengths, peer counts and alignments: the row figures bit for bit against the
+    # replay of their order, the factors against the oracle's on norms taken in double
+    rng = np.random.default_rng(77)
+    lib = _lib.load()
+    for draw in range(30):
+        k = int(rng.choice([2, 4, 6, 8, 12, 16, 24, 32, 40, 64]))
+        P = int(rng.integers(1, 9))
+        rows = [int(rng.integers(1, 40)) for _ in range(int(rng.integers(1, 6)))]
+        n = sum(rows)
+        off = int(rng.integers(0, 4))  # floats past a 16-byte boundary
+        vals = [t3((n, k), 1000 * draw + p, row_scale=True) * float(10.0 ** rng.uniform(-6, 3)) for p in range(P)]
+        bufs = [torch.empty(n * k + off, device=dev) for _ in range(P)]
+        d_vals = []
+        for b, v in zip(bufs, vals):
+            b[off:].copy_(v.reshape(-1))
+            d_vals.append(b[off:].view(n, k))
+        outs = [torch.empty(n, device=dev) for _ in range(P)]
+        vp = (C.c_void_p * P)(*[v.data_ptr() for v in d_vals])
+        op = (C.c_void_p * P)(*[o.data_ptr() for o in outs])
+        assert lib.tplr_row_sumsq(vp, P, k, n, op, None) == 0
+        for v, o in zip(vals, outs):
+            assert np.array_equal(o.cpu().numpy(), tree_rows(v.numpy())), (draw, k, off)
+        # clip factors of a row list cut into `rows`
+        import numpy as _np
+        desc = _np.zeros(len(rows), dtype=_np.dtype([("dense", "<u8"), ("ld", "<i8"), ("chunk_begin", "<i8"),
+                                                     ("x_chunks", "<i4"), ("y_chunks", "<i4")]))
+        begin = 0
+        for i, r in enumerate(rows):
+            desc[i] = (0, 64, begin, r, 1)
+            begin += r
+        table = torch.from_numpy(desc.view(_np.uint8).copy()).to(dev)
+        S = int(rng.integers(1, 5))
+        partial = torch.empty(len(rows) * P * S, dtype=torch.float64, device=dev)
+        scale = torch.empty((len(rows), P), device=dev)
+        med = torch.empty(len(rows), device=dev)
+        assert lib.tplr_clip_scales_rows(op, P, table.data_ptr(), len(rows), S, partial.data_ptr(), scale.data_ptr(),
+                                         med.data_ptr(), None) == 0
+        begin = 0
+        for i, r in enumerate(rows):
+            nr = np.array([np.sqrt((v.numpy()[begin:begin + r].astype(np.float64) ** 2).sum()) for v in vals], np.float32)
+            want_med, want = orc.clip_scales(nr)
+            assert np.allclose(scale[i].cpu().numpy(), want, rtol=3e-6), (draw, i)
+            assert np.isclose(float(med[i]), want_med, rtol=3e-6)
+            begin += r
