@@ -161,7 +161,7 @@ __device__ __forceinline__ void tile_to_flat(const float* tile, float* __restric
 // element i < 64 in lane i (idx0/val0), element 64 + i in lane i (idx1/val1, only for k > 64).
 //
 // Method: a cheap lower bound T0 for the k-th largest magnitude comes from per-lane maxima
-// (k <= 32) or per-lane top-2 (k <= 128): the k-th largest of those is met by at least k
+// (k <= 32) or the maxima of each lane's two half rows (k <= 128): the k-th largest of those is met by at least k
 // elements, and so are its leading bits with the rest cleared, which is as far as the search
 // goes.  Everything >= T0 (typically 1.1-1.5 k elements) is compacted into 8-byte candidate
 // slots - (magnitude bits, 4095 - index, sign) - in index order and bitonic-sorted, on 32-bit
@@ -177,18 +177,36 @@ struct Selected {
     float val0, val1;
 };
 
+// max(|a|, |b|, |c|) in one instruction (a quiet NaN loses against a number)
+__device__ __forceinline__ float max3_abs(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, |%1|, |%2|, |%3|" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// largest magnitude among v[kFrom .. kFrom + kCount - 1]: kCount / 2 instructions
+template <int kFrom, int kCount>
+__device__ __forceinline__ float max_abs_of(const float (&v)[64]) {
+    static_assert(kCount >= 4 && kCount % 2 == 0, "a first triple, then pairs, then the last one");
+    float m = max3_abs(v[kFrom], v[kFrom + 1], v[kFrom + 2]);
+#pragma unroll
+    for (int d = 3; d + 1 < kCount; d += 2) m = max3_abs(m, v[kFrom + d], v[kFrom + d + 1]);
+    return max3_abs(m, v[kFrom + kCount - 1], v[kFrom + kCount - 1]);
+}
+
+// The statistics the threshold is taken from: magnitudes of distinct elements of the lane's row, one (the largest)
+// or two (the largest of each half of the row).  The k-th largest of the wave's statistics is met by at least k
+// elements of the chunk, whichever elements they are, and the halves' maxima cost a quarter of the instructions of
+// the row's two largest while passing as few candidates.
 template <bool kTwo>
 __device__ __forceinline__ void lane_stats(const float (&v)[64], uint32_t& b1, uint32_t& b2) {
-    float m1 = __builtin_fabsf(v[0]);
-    float m2 = 0.0f;
-#pragma unroll
-    for (int d = 1; d < 64; ++d) {
-        const float a = __builtin_fabsf(v[d]);
-        if (kTwo) m2 = __builtin_amdgcn_fmed3f(m1, m2, a);
-        m1 = __builtin_fmaxf(m1, a);
+    if (kTwo) {
+        b1 = __float_as_uint(max_abs_of<0, 32>(v));
+        b2 = __float_as_uint(max_abs_of<32, 32>(v));
+    } else {
+        b1 = __float_as_uint(max_abs_of<0, 64>(v));
+        b2 = 0;
     }
-    b1 = __float_as_uint(m1);
-    b2 = __float_as_uint(m2);
 }
 
 // The search for the k-th largest lane statistic is a chain of dependent steps (vector compare, scalar count,
@@ -570,7 +588,7 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
 
         if (total > static_cast<uint32_t>(kCandCap) || total < static_cast<uint32_t>(k)) {
             // Exact search for the k-th largest key, from the bits t0 and the maximum share.
-            const uint32_t vmax = wave_max_u32(mag_key(b1));
+            const uint32_t vmax = wave_max_u32(kTwo ? (mag_key(b1) > mag_key(b2) ? mag_key(b1) : mag_key(b2)) : mag_key(b1));
             uint32_t t = mag_key(t0);
             uint32_t n_ge = count_ge(w, t);
             if (n_ge > static_cast<uint32_t>(kCandCap)) {
@@ -633,12 +651,21 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
             uint32_t at = upper ? h.z + __popc(h.x) : h.z;
             const uint32_t ix0 = h.w * 64 + (upper ? 32u : 0u);
             row += upper ? 32 : 0;
+            // two candidates per trip: their reads are in flight together, and the trip's round trip through the
+            // LDS, which is what the loop waits for, is paid half as often
+            auto slot_of = [&](uint32_t bits, uint32_t ix) {
+                return (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - ix) << 1) | (bits >> 31);
+            };
             while (m) {
-                const int z = __builtin_clz(m);
-                m &= ~(0x80000000u >> z);
-                const uint32_t bits = __float_as_uint(row[z]);
-                const uint32_t ix = ix0 + z;
-                cand[at++] = (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - ix) << 1) | (bits >> 31);
+                const int z0 = __builtin_clz(m);
+                m &= ~(0x80000000u >> z0);
+                const bool two = m != 0;
+                const int z1 = two ? __builtin_clz(m) : z0;
+                m &= ~(0x80000000u >> z1);
+                const uint32_t bits0 = __float_as_uint(row[z0]), bits1 = __float_as_uint(row[z1]);
+                cand[at] = slot_of(bits0, ix0 + z0);
+                if (two) cand[at + 1] = slot_of(bits1, ix0 + z1);
+                at += two ? 2u : 1u;
             }
         }
     };
@@ -673,7 +700,7 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
     int slot_of_lane = lane;
     asm volatile("" : "+v"(slot_of_lane));
     if (total <= 64) {
-        const bool mine = lane < static_cast<int>(total);
+        const bool mine = slot_of_lane < static_cast<int>(total);
         e0 = mine ? cand[slot_of_lane] : 0ull;
         // Slots were filled in index order, so (magnitude, 63 - slot) orders the candidates as the 64-bit keys
         // do; with the magnitudes taken from the floor it fits 32 bits while they span less than 2^26 (eight
@@ -687,7 +714,7 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
             sort64_desc(e0, lane);
         }
     } else {
-        const bool mine = lane + 64 < static_cast<int>(total);
+        const bool mine = slot_of_lane + 64 < static_cast<int>(total);
         e0 = cand[slot_of_lane];
         e1 = mine ? cand[slot_of_lane + 64] : 0ull;
         // the same with seven bits of slot and magnitudes that span less than 2^25 (four binades)
