@@ -610,7 +610,14 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
             exact_masks(w, t, ghi, glo, ehi, elo);
             if (n_ge > static_cast<uint32_t>(kCandCap)) {
                 // more ties at the threshold than slots: take the lowest-index ties only
-                const uint32_t g = wave_sum_u32(__popc(ghi) + __popc(glo));
+                uint32_t g = wave_sum_u32(__popc(ghi) + __popc(glo));
+                if (g >= static_cast<uint32_t>(k)) {
+                    // k or more keys above the largest statistic: NaNs, which the statistics leave out (a maximum
+                    // drops a quiet NaN) and which share the top key - they are the selection, lowest index first
+                    t = 0x7fffffffu;
+                    exact_masks(w, t, ghi, glo, ehi, elo);
+                    g = 0;
+                }
                 const uint32_t ties = __popc(ehi) + __popc(elo);
                 const uint32_t tincl = wave_incl_scan_u32(ties);
                 const int need = k - static_cast<int>(g);

@@ -265,6 +265,33 @@ def test_topk_candidates_at_the_limits_of_the_short_sort_keys(dev, k):
     check_topk(rows, k, dev)
 
 
+@pytest.mark.parametrize("k", [2, 32, 64, 100, 128])
+def test_topk_more_nans_than_candidate_slots(dev, k):
+    # NaNs rank first (all of them tie, lowest index first) and a lane's maximum drops them, so the threshold
+    # statistics do not see them: rows with more NaNs than the select has candidate slots (128), spread over the
+    # lanes, in a few lanes only, positive and negative, with infinities and large values beside them.
+    rng = np.random.default_rng(77 + k)
+    rows = (rng.standard_normal((8, 4096)) * 1e-3).astype(np.float32)
+    rows[0, rng.choice(4096, 129, replace=False)] = np.nan
+    rows[1, rng.choice(4096, 300, replace=False)] = np.nan
+    rows[2, rng.choice(4096, 1000, replace=False)] = np.nan
+    rows[2, rng.choice(4096, 50, replace=False)] = np.inf
+    rows[3, 64 * 5:64 * 9] = np.nan                                   # four lanes' rows entirely
+    rows[4, rng.choice(4096, 200, replace=False)] = -np.nan
+    rows[4, rng.choice(4096, 200, replace=False)] = np.nan
+    rows[5, rng.choice(4096, 127, replace=False)] = np.nan            # one short of the slots
+    rows[6, ::2] = np.nan
+    rows[6, 1::2] = np.float32(3e38)
+    rows[7, rng.choice(4096, 4000, replace=False)] = np.nan
+    check_topk(rows, k, dev)
+    # the fused encode without the transform takes the same select
+    x = torch.from_numpy(rows.reshape(8, 64, 64).transpose(1, 0, 2).reshape(64, 8 * 64).copy()).to(dev)
+    idx, val, _, _ = tc.encode_compress(x, k, use_dct=False)
+    want_i, want_v = orc.topk_rows(rows, k)
+    assert np.array_equal(tc.unpack_12bit_indices(idx, val.shape).cpu().numpy().reshape(-1, k), want_i)
+    assert np.array_equal(val.cpu().numpy().reshape(-1, k).view(np.uint32), want_v.view(np.uint32))
+
+
 @pytest.mark.parametrize("n,k", [(64, 32), (64, 64), (100, 10), (37, 6), (4095, 32), (2048, 128), (2, 2), (2048, 512),
                                  (300, 300), (4095, 4094)])
 def test_topk_generic_rows(dev, n, k):
