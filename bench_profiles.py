@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """rocprofv3 runs behind the summaries under profiles/, and the summaries themselves.
 
-  python bench_profiles.py run [--sets cfg3,cfg5,prod,nodct,bench] [--phases encode,aggregate,...]
+  python bench_profiles.py run [--sets cfg3,cfg5,prod,nodct,bench,matrix] [--phases encode,aggregate,...]
       on a box with an MI355X: for every (set, phase) a kernel trace of `bench.py --profile <phase>` (50 timed
       launches after the settle phase and 10 warm-up ones), and one run each for the FETCH_SIZE, WRITE_SIZE and
       (encode, aggregate) SQ_* counters.  Raw CSVs go to gpurun_out/prof/<set>_<phase>_<what>/, trimmed to this
@@ -55,6 +55,10 @@ SETS = {
 }
 COUNTED = {"copy", "encode", "aggregate", "calib", "outer"}   # phases whose HBM traffic is counted
 WITH_SQ = {"encode", "aggregate"}
+# the measurement build with half of the forward transform on the matrix cores (`TPLR_BUILD_MATRIX_VARIANT=1` makes
+# __graft_entry__.build() write it beside the product library): the set `matrix` profiles its encode launch
+MATRIX_LIB = os.path.join(ROOT, "templar_amd", "libtplr_hip_matrix_variant.so")
+MFMA = "SQ_INSTS_VALU_MFMA_MOPS_F32 SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES GRBM_GUI_ACTIVE".split()
 
 
 # ------------------------------------------------------------------------------------------------ run
@@ -80,12 +84,14 @@ def _trim(directory):
                 fh.writelines([lines[0]] + keep)
 
 
-def _profile(tag, what, prof_args, bench_args, limit):
+def _profile(tag, what, prof_args, bench_args, limit, lib=None):
     out = os.path.join(RAW, f"{tag}_{what}")
     cmd = ["rocprofv3", *prof_args, "--output-format", "csv", "-d", out, "-o", "p", "--", "python3",
            os.path.join(ROOT, "bench.py"), *bench_args]
     print("==", tag, what, flush=True)
     env = dict(os.environ, TMPDIR="/tmp")
+    if lib:
+        env["TPLR_HIP_LIB"] = lib
     with open(out + ".log", "w") as log:
         try:
             rc = subprocess.run(cmd, cwd="/tmp", env=env, stdout=log, stderr=subprocess.STDOUT, timeout=limit).returncode
@@ -102,6 +108,16 @@ def run(sets, phases):
     for tag in sets:
         if tag == "bench":  # the default benchmark run as a whole: every kernel of the library once
             _profile("bench_default", "kt", ["--kernel-trace", "--stats"], ["--no-cpu-baseline"], 400)
+            continue
+        if tag == "matrix":
+            if not os.path.exists(MATRIX_LIB):
+                sys.exit(f"{MATRIX_LIB} is not built: TPLR_BUILD_MATRIX_VARIANT=1 python -c 'import __graft_entry__ as g; g.build()'")
+            base = ["--profile", "encode"]
+            _profile("matrix_encode", "kt", ["--kernel-trace", "--stats"], base + ["--steps", "50", "--warmup", "10"], 300, MATRIX_LIB)
+            for what, counters in (("SQ", SQ), ("MFMA", MFMA)):
+                _profile("matrix_encode", what, ["--kernel-include-regex", "tplr", "--pmc", *counters],
+                         base + ["--steps", "3", "--warmup", "1"], 240, MATRIX_LIB)
+            _profile("cfg3_encode", "MFMA", ["--kernel-include-regex", "tplr", "--pmc", *MFMA], base + ["--steps", "3", "--warmup", "1"], 240)
             continue
         S = SETS[tag]
         for ph in S["phases"]:
@@ -501,6 +517,84 @@ k_decode_aggregate_cfg3_llama1b_15peers.md):
 
 {_stats_table('bench_default')}
 """)
+    # ---------------- the measurement build with half of the forward transform on the matrix cores
+    if _have("matrix_encode") and _have("matrix_encode", "MFMA") and _have("cfg3_encode", "MFMA") and _have("cfg3_encode"):
+        kern = "k_encode_topk_pack<false, true, false>"
+        n = SETS["cfg3"]["chunks"]
+        alg = n * 16384 + n * 11 * 32 // 2
+        tr, dur = _trace("matrix_encode", kern)
+        avg = sum(dur[-50:]) / 50
+        _, dur0 = _trace("cfg3_encode", kern)
+        avg0 = sum(dur0[-50:]) / 50
+
+        def mfma(tag):
+            acc = collections.defaultdict(list)
+            for r in csv.DictReader(open(_csv(tag, "MFMA", "*counter_collection.csv"))):
+                if kern in r["Kernel_Name"]:
+                    acc[r["Counter_Name"]].append(float(r["Counter_Value"]))
+            return {k_: sum(v) / len(v) for k_, v in acc.items()}
+
+        m1, m0 = mfma("matrix_encode"), mfma("cfg3_encode")
+        mops, busy = m1.get("SQ_INSTS_VALU_MFMA_MOPS_F32", 0), m1.get("SQ_VALU_MFMA_BUSY_CYCLES", 0)
+        n_mfma, simds, cyc = mops / 8, 1024, m1.get("GRBM_GUI_ACTIVE", 8) / 8   # (a 32x32x2 instruction is 4 096 operations)
+        m_sq = collections.defaultdict(list)
+        for r in csv.DictReader(open(_csv("matrix_encode", "SQ", "*counter_collection.csv"))):
+            if kern in r["Kernel_Name"]:
+                m_sq[r["Counter_Name"]].append(float(r["Counter_Value"]))
+        m_sq = {k_: sum(v) / len(v) for k_, v in m_sq.items()}
+        m_sq0 = 0.0
+        if _have("cfg3_encode", "SQ"):
+            v0 = [float(r["Counter_Value"]) for r in csv.DictReader(open(_csv("cfg3_encode", "SQ", "*counter_collection.csv")))
+                  if kern in r["Kernel_Name"] and r["Counter_Name"] == "SQ_INSTS_VALU"]
+            m_sq0 = sum(v0) / len(v0) / n
+        rows = ["| counter | vector code (the product) | odd half on the matrix cores |", "|---|---|---|"]
+        rows += [f"| {c} | {m0.get(c, 0):,.0f} | {m1.get(c, 0):,.0f} |" for c in MFMA]
+        pre = PRE + "TPLR_HIP_LIB=templar_amd/libtplr_hip_matrix_variant.so "
+        write("k_encode_topk_pack_cfg3_llama1b_matrix_cores.md", f"""# The forward transform's odd half on the matrix cores against the generated vector code: encode launch of the 1B set
+
+The product computes the 64-point transform as factorised vector code (535 instructions per 64-vector).  A
+measurement build of the same sources (`-DTPLR_DCT_MATRIX_CORES=1`, `templar_amd/csrc/tplr_device.h`:
+`dct64_fwd_matrix`) computes the odd half of the forward transform - a 32-point DCT-IV, 250 of those instructions -
+as a dense 32x32x64 product with 32 `v_mfma_f32_32x32x2_f32` per pass, operands formed with `v_permlane32_swap`, and
+keeps everything else.  Built beside the product library by
+
+    TPLR_BUILD_MATRIX_VARIANT=1 python -c 'import __graft_entry__ as g; g.build()'
+
+and profiled with the commands below (`python bench_profiles.py run --sets matrix` runs all of them).
+
+## Kernel trace
+
+    {pre}rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof/matrix_encode_kt -o p -- python3 bench.py --profile encode --steps 50 --warmup 10
+
+{_stats_table('matrix_encode')}
+
+Launch geometry: {_geometry(tr[-1])}.
+
+The 50 timed launches average **{avg:.1f} us** against **{avg0:.1f} us** for the product's vector code
+(k_encode_topk_pack_cfg3_llama1b.md): {alg / avg / 1e3:.0f} GB/s = {alg / avg / 1e3 / 80:.1f} % of 8 TB/s against
+{alg / avg0 / 1e3:.0f} GB/s = {alg / avg0 / 1e3 / 80:.1f} %.
+
+## Matrix-core and vector-ALU activity (hardware counters)
+
+    {pre}rocprofv3 --kernel-include-regex tplr --pmc {' '.join(MFMA)} --output-format csv -d gpurun_out/prof/matrix_encode_MFMA -o p -- python3 bench.py --profile encode --steps 3 --warmup 1
+    {PRE}rocprofv3 --kernel-include-regex tplr --pmc {' '.join(MFMA)} --output-format csv -d gpurun_out/prof/cfg3_encode_MFMA -o p -- python3 bench.py --profile encode --steps 3 --warmup 1
+
+{chr(10).join(rows)}
+
+`SQ_INSTS_VALU_MFMA_MOPS_F32` counts 512 floating-point operations each: {mops * 512 / n:,.0f} per chunk (two passes of
+a dense 32x32x64 product are 262 144), in {n_mfma / n:.0f} matrix instructions per chunk.  `SQ_VALU_MFMA_BUSY_CYCLES` is
+{busy / n_mfma:.1f} cycles per instruction: the matrix pipelines of the {simds} SIMDs are busy {busy / simds / cyc * 100:.0f} % of the
+launch's {cyc / 1e6:.2f} M cycles (`GRBM_GUI_ACTIVE` over 8 XCDs) - far from saturated - and yet the launch takes
+{avg / avg0:.2f} x as long as with vector code although it issues {m_sq['SQ_INSTS_VALU'] / n:.0f} vector instructions per chunk instead of
+{m_sq0:.0f}: the vector ALU is active {m_sq['SQ_ACTIVE_INST_VALU'] / m_sq['SQ_WAVE_CYCLES'] * 100:.0f} % of a wave's time (31 % in the product) and the waves wait
+for an issue slot {m_sq['SQ_WAIT_INST_ANY'] / m_sq['SQ_WAVE_CYCLES'] * 100:.0f} % of it.  A SIMD that is working on a matrix instruction issues next to nothing
+else here, so the 64 cycles of each instruction come on top of the vector work instead of beside it - 4 096
+cycles per chunk against the 1 000 the factorised odd half takes.  The transform stays vector code.
+
+    {pre}rocprofv3 --kernel-include-regex tplr --pmc {' '.join(SQ)} --output-format csv -d gpurun_out/prof/matrix_encode_SQ -o p -- python3 bench.py --profile encode --steps 3 --warmup 1
+
+{_sq('matrix_encode', kern, n, 3, 'Here the transform is half vector code, half matrix-core instructions.')}
+""")
     if traffic:
         traffic["what"] = ("HBM bytes per launch of the whole-set kernels (FETCH_SIZE + WRITE_SIZE, each scaled by the calibration "
                            "copy), keyed workload/peers/kernel; written by bench_profiles.py summarise from the rocprofv3 runs whose "
@@ -520,7 +614,7 @@ def main():
     args = ap.parse_args()
     sets = [s for s in args.sets.split(",") if s]
     for s in sets:
-        if s not in SETS and s != "bench":
+        if s not in SETS and s not in ("bench", "matrix"):
             ap.error(f"unknown set {s}")
     if args.what == "run":
         run(sets, [p for p in args.phases.split(",") if p])

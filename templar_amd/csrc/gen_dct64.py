@@ -31,7 +31,9 @@ The inverse transform is the transposed flow graph run backwards.
 Functions written: dct64_fwd_head (the 32 input butterflies, from a separate
 input array),
 dct64_fwd_tail, dct64_fwd (both), dct64_inv, and dct64_inv_hooked (dct64_inv
-with call-outs to a caller-supplied functor between its instructions).  Run as a build step
+with call-outs to a caller-supplied functor between its instructions); and, under TPLR_DCT_MATRIX_CORES, the
+pieces of a measurement variant that computes the odd half of the forward transform (a 32-point DCT-IV, 47 % of
+the operations) as a dense product on the matrix cores: dct64_fwd_even and the matrix kDct4Lane.  Run as a build step
 (`python gen_dct64.py`); `--check` only verifies and prints op counts.
 """
 from __future__ import annotations
@@ -95,7 +97,20 @@ def build_forward():
             out[2 * j - 1] = q[half - j]
         return out
 
-    out_slots = c2(list(range(N)), True)
+    # top level by hand so that the op list splits into head | even half | odd half
+    h = N // 2
+    slots = list(range(N))
+    for t in range(h):
+        ops.append(("bfly", slots[t], slots[N - 1 - t]))
+    n_head = len(ops)
+    even = c2([slots[t] for t in range(h)], True)
+    n_even_end = len(ops)
+    odd = c4([slots[N - 1 - t] for t in range(h)])
+    out_slots = [None] * N
+    for m in range(h):
+        out_slots[2 * m] = even[m]
+        out_slots[2 * m + 1] = odd[m]
+    build_forward.split = (n_head, n_even_end)
     return ops, out_slots
 
 
@@ -259,13 +274,42 @@ def emit_split_forward(ops, out_slots, n_head):
     return head, tail, em.nops, em2.nops, negs
 
 
+def emit_matrix_variant(fwd, out_slots, n_head, n_even_end):
+    """Pieces for the measurement variant whose odd half (the 32-point DCT-IV of the differences) is a dense
+    32x32 product on the matrix cores: the even half of the forward transform and the DCT-IV matrix."""
+    h = N // 2
+    # forward even half: slots 0..31 hold the sums after the head; even outputs are out[2m]
+    em = Emitter("t")
+    var = {s_: f"v[{s_}]" for s_ in range(h)}
+    sign = {s_: 1.0 for s_ in range(h)}
+    emit_ops(em, fwd[n_head:n_even_end], var, sign)
+    lines = list(em.lines)
+    for m in range(h):
+        s_ = out_slots[2 * m]
+        lines.append(f"    out[{2 * m}] = {'-' if sign[s_] < 0 else ''}{var[s_]};")
+    f_even = ("__device__ __forceinline__ void dct64_fwd_even(const float (&v)[64], float (&out)[64]) {\n"
+              + "\n".join(lines) + "\n}\n")
+    # DCT-IV matrix C4[m][n] = cos(pi (2n+1)(2m+1) / (4*32)), symmetric.  Stored the way the
+    # 32x32x2 matrix instruction wants its A operand: for K-step s, lane l supplies
+    # A[i = l % 32][k = l / 32] = C4[l % 32][2 s + l / 32]; one row of 16 floats per lane.
+    rows = []
+    for l in range(64):
+        m = l % 32
+        rows.append("    {" + ", ".join(
+            lit(math.cos(math.pi * (2 * (2 * s_ + l // 32) + 1) * (2 * m + 1) / (4 * h))) for s_ in range(16)) + "},")
+    table = ("// 32-point DCT-IV C4[m][n] = cos(pi (2n+1)(2m+1) / 128), the odd half of the transform,\n"
+             "// as A operands of v_mfma_f32_32x32x2_f32: kDct4Lane[l][s] = C4[l % 32][2 s + l / 32]\n"
+             "__device__ const float kDct4Lane[64][16] = {\n" + "\n".join(rows) + "\n};\n")
+    return f_even, table, em.nops
+
+
 def main():
     check_only = "--check" in sys.argv
     fwd, out_slots = build_forward()
     inv = transpose_ops(fwd)
     ident = list(range(N))
-    n_head = N // 2
-    assert all(op[0] == "bfly" for op in fwd[:n_head])
+    n_head, n_even_end = build_forward.split
+    assert n_head == N // 2 and all(op[0] == "bfly" for op in fwd[:n_head])
 
     f = dense_dct()
     for lifting in (False, True):
@@ -290,10 +334,25 @@ def main():
     back = run_ops(inv, st2, np.float32, lifting=True)[ident].astype(np.float64) / (GAIN * GAIN)
     rel_rt = np.abs(back - x).max() / np.abs(x).max()
 
+    # matrix-core variant of the forward transform: head butterflies, even half by the op list, odd half as
+    # a dense 32-point DCT-IV of d[n] = slot[63 - n]
+    h = N // 2
+    c4 = np.cos(np.pi * np.outer(2 * np.arange(h) + 1, 2 * np.arange(h) + 1) / (4 * h))
+    st = np.zeros((N, 4096))
+    st[ident] = x
+    st = run_ops(fwd[:n_even_end], st, np.float64, lifting=True)
+    y_mm = np.zeros((N, 4096))
+    y_mm[0::2] = st[[out_slots[2 * m] for m in range(h)]]
+    y_mm[1::2] = c4 @ st[[N - 1 - n for n in range(h)]]
+    err_mm_f = np.abs(y_mm / GAIN - y64).max() / np.abs(y64).max()
+    assert err_mm_f < 1e-12, err_mm_f
+
     head, tail, n_h, n_t, neg_f = emit_split_forward(fwd, out_slots, n_head)
     t_inv, n_inv, neg_i = emit_function("dct64_inv", inv, out_slots, ident)
     t_inv_hooked, _, _ = emit_function("dct64_inv_hooked", inv, out_slots, ident, hooks=N_HOOKS)
+    f_even, table, n_fe = emit_matrix_variant(fwd, out_slots, n_head, n_even_end)
     print(f"dct64_fwd: {n_h} + {n_t} ops (+{neg_f} negations), dct64_inv: {n_inv} ops (+{neg_i} negations)")
+    print(f"matrix-core variant of dct64_fwd: 64 butterflies, even half {n_fe} ops, odd half = 32x32 DCT-IV")
     print(f"fp64 matrix error fwd {err_f:.2e} inv {err_i:.2e}; fp32 forward err / max|y| = {rel:.2e}, "
           f"round trip err / max|x| = {rel_rt:.2e}")
     if check_only:
@@ -321,6 +380,9 @@ def main():
                  "template <int I>\nstruct DctHook {\n    static constexpr int value = I;\n};\n"
                  f"constexpr int kDctHooks = {N_HOOKS};\n\n")
         fh.write(t_inv_hooked)
+        fh.write("\n// Measurement variant (TPLR_DCT_MATRIX_CORES): the odd half of dct64_fwd as a dense product on the\n"
+                 "// matrix cores; see dct64_fwd_matrix in tplr_device.h.\n#if TPLR_DCT_MATRIX_CORES\n")
+        fh.write(table + "\n" + f_even + "#endif\n")
 
 
 if __name__ == "__main__":

@@ -43,6 +43,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#ifndef TPLR_DCT_MATRIX_CORES
+#define TPLR_DCT_MATRIX_CORES 0  // 1: a measurement build, see dct64_fwd_matrix below
+#endif
 #include "dct64_gen.h"
 
 namespace tplr {
@@ -61,6 +64,80 @@ __device__ __forceinline__ int64_t xcd_contiguous(int64_t bid, int64_t grid) {
     const int64_t per = grid >> 3;
     return (bid & 7) * per + (bid >> 3);
 }
+
+// -----------------------------------------------------------------------------------------
+// Measurement variant (TPLR_DCT_MATRIX_CORES=1, off in the product): the forward 64-point transform with its
+// odd half on the matrix cores.
+//
+// After the 32 input butterflies the odd-indexed outputs are a 32-point DCT-IV of the differences
+// d[n] = x[n] - x[63-n]: 250 of the 535 vector instructions of the factorised transform.  Here that half is the
+// dense product Y = C4 D (32x32 times 32x64: one column per lane) with 32 v_mfma_f32_32x32x2_f32, which run
+// beside the vector ALU work of the other resident waves (and beside this wave's even half).
+//
+// Operand layout of the instruction (wave64): A: lane l holds A[l%32][l/32]; B: lane l holds B[l/32][l%32];
+// D: lane l, register r holds D[8(r/4) + 4(l/32) + r%4][l%32].  Lanes 0..31 and 32..63 form two column groups
+// with one accumulator each.  v_permlane32_swap(a, b) exchanges the upper half of a with the lower half of b,
+// which turns the register pair (d[2s], d[2s+1]) of every lane into the B operands of both groups for K-step s,
+// and turns the two accumulators back into one result pair per lane.
+//
+// It exists to put a number on the choice of vector code for the transform: the encode launch of the 1B set takes
+// 1.68 ms this way against 0.94 ms.  Each 32x32x2 fp32 instruction holds the matrix pipeline of its SIMD for 64
+// cycles, 4 096 cycles per chunk, and the SIMD issues next to no vector instruction meanwhile: the matrix work comes
+// on top of the vector work, not beside it, and the factorised odd half costs the vector ALU 1 000 cycles.  Its
+// coefficients differ from dct64_fwd's in the last bits, so a build with it selects other elements on near-ties than
+// the stand-alone transform kernels, which keep the vector code.
+// -----------------------------------------------------------------------------------------
+#if TPLR_DCT_MATRIX_CORES
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// y = C4_32 d for the 64 lanes' vectors; ca = this lane's row of kDct4Lane
+__device__ __forceinline__ void dct4_32_matrix(const float (&d)[32], float (&y)[32], const float (&ca)[16]) {
+    v16f acc_lo = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    v16f acc_hi = acc_lo;
+    // (the exchange as an assembly statement with both registers read and written: through the compiler's
+    // builtin the second accumulator chain was seen to be dropped; the wait states keep a matrix instruction
+    // from reading a register the exchange has just written)
+    auto swap_halves = [](float& a, float& b) { asm volatile("v_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b)); };
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        float b0 = d[2 * s], b1 = d[2 * s + 1];
+        swap_halves(b0, b1);
+        acc_lo = __builtin_amdgcn_mfma_f32_32x32x2f32(ca[s], b0, acc_lo, 0, 0, 0);
+        acc_hi = __builtin_amdgcn_mfma_f32_32x32x2f32(ca[s], b1, acc_hi, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        float q0 = acc_lo[r], q1 = acc_hi[r];
+        swap_halves(q0, q1);
+        const int i = 8 * (r >> 2) + (r & 3);
+        y[i] = q0;
+        y[i + 4] = q1;
+    }
+}
+
+__device__ __forceinline__ void load_dct4_operand(float (&ca)[16], int lane) {
+    const float4* row = reinterpret_cast<const float4*>(&kDct4Lane[lane][0]);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const float4 t = row[q];
+        ca[4 * q] = t.x, ca[4 * q + 1] = t.y, ca[4 * q + 2] = t.z, ca[4 * q + 3] = t.w;
+    }
+}
+
+// v <- sqrt(32) * DCT-II(v) (orthonormal), one 64-vector per lane; all 64 lanes must be active.
+// `ca` is the lane's row of kDct4Lane (load_dct4_operand), kept by the caller across its loop.
+__device__ __forceinline__ void dct64_fwd_matrix(float (&v)[64], const float (&ca)[16]) {
+    float t[64];
+    dct64_fwd_head(v, t);
+    float d[32], y[32];
+#pragma unroll
+    for (int n = 0; n < 32; ++n) d[n] = t[63 - n];
+    dct4_32_matrix(d, y, ca);
+    dct64_fwd_even(t, v);
+#pragma unroll
+    for (int m = 0; m < 32; ++m) v[2 * m + 1] = y[m];
+}
+#endif
 
 // One wavefront per workgroup: LDS instructions of a wave execute in order, so lanes only need
 // the compiler to keep program order.  (A workgroup barrier would also drain the vector-memory
@@ -658,21 +735,12 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
             uint32_t at = upper ? h.z + __popc(h.x) : h.z;
             const uint32_t ix0 = h.w * 64 + (upper ? 32u : 0u);
             row += upper ? 32 : 0;
-            // two candidates per trip: their reads are in flight together, and the trip's round trip through the
-            // LDS, which is what the loop waits for, is paid half as often
-            auto slot_of = [&](uint32_t bits, uint32_t ix) {
-                return (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - ix) << 1) | (bits >> 31);
-            };
             while (m) {
-                const int z0 = __builtin_clz(m);
-                m &= ~(0x80000000u >> z0);
-                const bool two = m != 0;
-                const int z1 = two ? __builtin_clz(m) : z0;
-                m &= ~(0x80000000u >> z1);
-                const uint32_t bits0 = __float_as_uint(row[z0]), bits1 = __float_as_uint(row[z1]);
-                cand[at] = slot_of(bits0, ix0 + z0);
-                if (two) cand[at + 1] = slot_of(bits1, ix0 + z1);
-                at += two ? 2u : 1u;
+                const int z = __builtin_clz(m);
+                m &= ~(0x80000000u >> z);
+                const uint32_t bits = __float_as_uint(row[z]);
+                const uint32_t ix = ix0 + z;
+                cand[at++] = (static_cast<uint64_t>(mag_key(bits)) << 32) | ((4095u - ix) << 1) | (bits >> 31);
             }
         }
     };

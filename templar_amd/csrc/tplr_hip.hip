@@ -575,6 +575,10 @@ __global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_de
     Cursor c, cg;
     cursor_seek(c, table, single, n_tensors, g0);
     if (kEf) cursor_seek(cg, grad_table, single, n_tensors, g0);
+#if TPLR_DCT_MATRIX_CORES
+    float ca[16] = {};
+    if (kUseDct) load_dct4_operand(ca, lane);
+#endif
     for (int64_t g = g0; g < g1; ++g) {
         float v[64], w[64];
         load_chunk_cols(v, c, lane);
@@ -594,7 +598,13 @@ __global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_de
         // the transform are mixed across both and one direction is as good as two.)
         uint32_t c1 = 0, c2 = 0;
         if (!kUseDct) lane_stats<kTwo>(v, c1, c2);
+#if TPLR_DCT_MATRIX_CORES
+        if (kUseDct) dct64_fwd_matrix(v, ca);
+        transpose_via_half(v, w, buf, lane);
+        if (kUseDct) dct64_fwd_matrix(w, ca);
+#else
         chunk_forward<kUseDct>(v, w, buf, lane);
+#endif
         const Selected s =
             select_topk<kTwo, !kUseDct>(w, buf, cand, lane, k, kUseDct ? kDctPow2Scale : 1.0f, c1, c2);
         emit_selected<kTwo>(s, lane, k, g, idx12, val);
