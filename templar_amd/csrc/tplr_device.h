@@ -663,7 +663,9 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
         incl = wave_incl_scan_u32(cnt);
         total = __builtin_amdgcn_readlane(incl, 63);
 
-        if (total > static_cast<uint32_t>(kCandCap) || total < static_cast<uint32_t>(k)) {
+        // (the rare paths below are marked as such: code the compiler lays out of line costs the common path
+        // neither taken branches nor instruction fetches)
+        if (__builtin_expect(total > static_cast<uint32_t>(kCandCap) || total < static_cast<uint32_t>(k), 0)) {
             // Exact search for the k-th largest key, from the bits t0 and the maximum share.
             const uint32_t vmax = wave_max_u32(kTwo ? (mag_key(b1) > mag_key(b2) ? mag_key(b1) : mag_key(b2)) : mag_key(b1));
             uint32_t t = mag_key(t0);
@@ -781,7 +783,7 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
         // do; with the magnitudes taken from the floor it fits 32 bits while they span less than 2^26 (eight
         // binades), and the sort costs a third.  The winner's slot comes back out of the key.
         const uint32_t above = static_cast<uint32_t>(e0 >> 32) - floor_key;
-        if (__ballot(mine && above >= (1u << 26)) == 0) {  // wave-uniform
+        if (__builtin_expect(__ballot(mine && above >= (1u << 26)) == 0, 1)) {  // wave-uniform
             uint32_t key = mine ? (above << 6) | (63u - static_cast<uint32_t>(slot_of_lane)) : 0u;
             sort64_desc_u32(key);
             e0 = cand[63u - (key & 63u)];
@@ -795,7 +797,7 @@ __device__ __forceinline__ Selected select_topk(const float (&w)[64], float* buf
         // the same with seven bits of slot and magnitudes that span less than 2^25 (four binades)
         const uint32_t above0 = static_cast<uint32_t>(e0 >> 32) - floor_key;
         const uint32_t above1 = static_cast<uint32_t>(e1 >> 32) - floor_key;
-        if (__ballot(above0 >= (1u << 25) || (mine && above1 >= (1u << 25))) == 0) {  // wave-uniform
+        if (__builtin_expect(__ballot(above0 >= (1u << 25) || (mine && above1 >= (1u << 25))) == 0, 1)) {  // wave-uniform
             uint32_t key0 = (above0 << 7) | (127u - static_cast<uint32_t>(slot_of_lane));
             uint32_t key1 = mine ? (above1 << 7) | (63u - static_cast<uint32_t>(slot_of_lane)) : 0u;
             sort128_desc_u32(key0, key1);
