@@ -1025,6 +1025,42 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         wave_lds_fence();
     };
 
+    // The same pass in pieces, for the pipeline with the transform: a chunk's 64 row stores are issued at the pace
+    // the memory system takes them, and the wave would stand at them with nothing else to do - so the LDS round
+    // trips of this pass (on the next chunk's tile) run between groups of those stores.  mean_begin scans the row's
+    // counters, mean_trip divides one coefficient in every lane that still has one, mean_finish does the rest.
+    struct MeanState {
+        uint32_t todo, word, m;
+        int q;
+    };
+    auto mean_begin = [&](MeanState& ms) {
+        wave_lds_fence();
+        ms.todo = 0, ms.word = 0, ms.m = 0, ms.q = 0;
+        if (reduce_mode != TPLR_REDUCE_MEAN) return;
+        const uint32_t* crow = cnt + lane * Cnt::kRowWords;
+#pragma unroll
+        for (int q = 0; q < Cnt::kRowWords; ++q) ms.todo |= ((crow[q] & Cnt::kMulti) ? 1u : 0u) << q;
+    };
+    auto mean_trip = [&](MeanState& ms) {
+        if (ms.todo | ms.m) {
+            if (ms.m == 0) {
+                ms.q = __builtin_ctz(ms.todo);
+                ms.todo &= ms.todo - 1;
+                ms.word = cnt[lane * Cnt::kRowWords + ms.q];
+                ms.m = ms.word & Cnt::kMulti;
+            }
+            const int slot = __builtin_ctz(ms.m) / kCntBits;
+            const uint32_t n = (ms.word >> (slot * kCntBits)) & Cnt::kMask;
+            ms.m &= ~(Cnt::kMask << (slot * kCntBits));
+            float* t = &tile[lane * kLd + ms.q * Cnt::kPerWord + slot];
+            *t = *t / static_cast<float>(n);
+        }
+    };
+    auto mean_finish = [&](MeanState& ms) {
+        while (ms.todo | ms.m) mean_trip(ms);
+        wave_lds_fence();
+    };
+
     // ---- exact path for a chunk with repeated indices inside one peer's row (no top-k produces
     // them; the reference sums every entry and divides by the number of entries,
     // src/tplr/compress.py:472-474).  Entries are added in source order - peer by peer, and inside
@@ -1464,7 +1500,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             const bool skip1 = g + 1 < g1 && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
             if (skip1) mark_redo(g + 1);
             repeat = 0;
-            mean_pass();
+            // the mean of the next chunk's tile, its trips between the groups of this chunk's stores
+            MeanState ms;
+            mean_begin(ms);
             // a chunk that is to be done again is not stored: its descriptor gets a range of zero bytes
             if constexpr (kLateRows) {
                 void* chunk0 = (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0));
@@ -1490,11 +1528,23 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, b[q & 1][i] - v[q * 16 + i]), wr,
                                                               lane * 4, (q * 16 + i) * ld4, 2);
                     if constexpr (q + 2 < 4) fetch(Index<q + 2>{});
+                    mean_trip(ms);
                 });
             } else {
-                store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), uniform64(o0.ld), lane,
-                                 skip0 || tripped);
+                const int64_t ld0 = uniform64(o0.ld);
+                const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+                    (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), 0,
+                    (skip0 || tripped) ? 0 : static_cast<int>((63 * ld0 + 64) * 4), 0x00020000);
+                const int ld4 = static_cast<int>(ld0) * 4;
+                static_for<8>([&](auto qt) {
+                    constexpr int q = decltype(qt)::value;
+#pragma unroll
+                    for (int r = q * 8; r < (q + 1) * 8; ++r)
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v[r]), wr, lane * 4, r * ld4, 2);
+                    mean_trip(ms);
+                });
             }
+            mean_finish(ms);
             skip0 = skip1;
             o0 = o1;
             o1 = o2;
