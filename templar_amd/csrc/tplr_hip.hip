@@ -949,12 +949,13 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         const uint32_t was = atomicAdd(cw, 1u << sh);
         if ((((seen ^ was) >> sh) & Cnt::kMask) != 0u || ((was >> sh) & Cnt::kMask) == Cnt::kMask) repeat = kClaimMark;
     };
-    auto scatter = [&](int64_t g, int t_now) {
+    // (unit_lo, unit_hi: the fast path's units to run, for a caller that threads them between other work)
+    auto scatter = [&](int64_t g, int t_now, int unit_lo = 0, int unit_hi = 1 << 20) {
         if (fast) {
             if (lane_on) {
 #pragma unroll
                 for (int i = 0; i < kRegs; ++i) {
-                    if (i < P) {  // wave-uniform
+                    if (i >= unit_lo && i < unit_hi && i < P) {  // wave-uniform
                         const uint32_t e = (lane & 1) ? (ix[i] >> 4) : (ix[i] & 0xfffu);
                         const float x = kCodes ? code_value(__builtin_bit_cast(uint32_t, a[i]), i)
                                                : a[i] * __builtin_bit_cast(float, __builtin_amdgcn_readlane(
@@ -1818,7 +1819,41 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         const bool more = g + 1 < g1;
         Out out_after = out_next;
         int t_after = t_next;
-        if (more) {
+        // Without the transform chunk g is complete here: its 64 row stores go out first - the wave stands at
+        // them at the pace the memory system takes them - and, where the registers allow it (up to 16 peers), the
+        // next chunk's scatter, a chain of LDS round trips, runs between groups of them.
+        bool stored = false;
+        if (!kUseDct && fast && more && out_cur.ld > 0) {  // wave-uniform
+            chunk_stats(v, g, skip_cur);
+            const int64_t ld_s = uniform64(out_cur.ld);
+            const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+                (void*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0)), 0,
+                skip_cur ? 0 : static_cast<int>((63 * ld_s + 64) * 4), 0x00020000);
+            const int ld4 = static_cast<int>(ld_s) * 4;
+            zero_tile();
+            if constexpr (kUnits <= 16) {
+                constexpr int kGroups = 4, kPerGroup = (kRegs + kGroups - 1) / kGroups;
+                static_for<kGroups>([&](auto qt) {
+                    constexpr int q = decltype(qt)::value;
+#pragma unroll
+                    for (int r = q * 16; r < (q + 1) * 16; ++r)
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v[r]), wr, lane * 4, r * ld4, 2);
+                    scatter(g + 1, t_next, q * kPerGroup, (q + 1) * kPerGroup);
+                });
+            } else {
+#pragma unroll
+                for (int r = 0; r < 64; ++r)
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v[r]), wr, lane * 4, r * ld4, 2);
+                scatter(g + 1, t_next);
+            }
+            if (g + 2 < g1) {
+                cursor_next(c, g + 2);
+                out_after = out_of(c, g + 2);
+                t_after = c.t;
+                load_payload(g + 2, c.t);
+            }
+            stored = true;
+        } else if (more) {
             zero_tile();
             scatter(g + 1, t_next);
             if (g + 2 < g1) {
@@ -1830,7 +1865,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
         // ---- second half of chunk g, in registers
         if (kUseDct) dct64_inv(v);  // along b: v[k] = sum_b Z[b][lane] F[k][b]
-        chunk_stats(v, g, skip_cur);
+        if (!stored) chunk_stats(v, g, skip_cur);
         const bool skip_next = more && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
         if (skip_next) mark_redo(g + 1);
         repeat = 0;
@@ -1839,7 +1874,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         // (the loop-carried destination may have been parked in vector registers: make it scalar
         // again, or every store becomes a loop over distinct descriptors)
         gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0));
-        if (kUseDct || out_cur.ld > 0) {
+        if (stored) {
+            // (written above)
+        } else if (kUseDct || out_cur.ld > 0) {
             store_chunk_rows(v, (void*)dst, uniform64(out_cur.ld), lane, skip_cur);
         } else if (!skip_cur) {
 #pragma unroll
