@@ -552,10 +552,23 @@ __global__ __launch_bounds__(64) void k_encode_rows(const tplr_tensor_desc* __re
     }
 }
 
+// the wave's issue priority (0 .. 3; the instruction takes an immediate, hence the ladder); `level` is wave-uniform
+__device__ __forceinline__ void set_wave_priority(int level) {
+    if (level == 0) __builtin_amdgcn_s_setprio(0);
+    else if (level == 1) __builtin_amdgcn_s_setprio(1);
+    else if (level == 2) __builtin_amdgcn_s_setprio(2);
+    else __builtin_amdgcn_s_setprio(3);
+}
+
 // Persistent fused encode: every wave walks its slice of the chunk list.  The kernel is bound by
 // vector-ALU issue and by the latencies between its phases, so it is shaped for residency -
 // 8.5 KB + 1 KB of LDS and a register budget that admits three to four waves per SIMD - and
 // leaves the overlap of one wave's row loads with the other waves' arithmetic to the hardware.
+// The three waves of a SIMD pass its issue slots round: the arbiter alone serves the oldest wave first, so
+// that the workgroups dispatched last run behind all the way and the launch waits for them.  Each wave
+// therefore steps through the priority levels 0, 1, 2 chunk by chunk, the three dispatch layers of a full
+// grid one step apart, and changes level once its rows are requested (4 % off the launch; the level
+// values, the direction and a change at another phase or every other chunk matter less than 1 %).
 // kEf: the miner's momentum update rides on the load (src/tplr/neurons.py:151-152): the chunk of
 // the error-feedback tensor becomes ef * decay + grad (two roundings, as mul_ then add_), is
 // written back in place and is what gets encoded.
@@ -579,6 +592,7 @@ __global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_de
     float ca[16] = {};
     if (kUseDct) load_dct4_operand(ca, lane);
 #endif
+    int turn = static_cast<int>(blockIdx.x * 3u / gridDim.x);  // the dispatch layer of a full grid; wave-uniform
     for (int64_t g = g0; g < g1; ++g) {
         float v[64], w[64];
         load_chunk_cols(v, c, lane);
@@ -596,6 +610,8 @@ __global__ __launch_bounds__(64, 3) void k_encode_topk_pack(const tplr_tensor_de
         // Untransformed gradients often differ in scale from row to row or column to column;
         // the select's threshold statistic is then taken in both directions.  (Coefficients of
         // the transform are mixed across both and one direction is as good as two.)
+        set_wave_priority(turn);
+        turn = turn == 2 ? 0 : turn + 1;
         uint32_t c1 = 0, c2 = 0;
         if (!kUseDct) lane_stats<kTwo>(v, c1, c2);
 #if TPLR_DCT_MATRIX_CORES
@@ -1392,7 +1408,17 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         const int dummy_pos = kPark ? kTileFloats + lane : lane * kLd + kChunk;
         const uint32_t park = 4096u + lane;  // (kPark) maps to tile[kTileFloats + lane] and cnt[512 + lane / 8]
         // one chunk: `st` holds chunk g + 1 and is refilled with chunk g + 3
+        // The two waves that share a SIMD are served oldest first, and on that rule alone the wave of the later
+        // workgroup layer falls behind and finishes last.  The waves take turns instead: on every other chunk a
+        // wave runs two priority levels up, on opposite chunks in the two layers.  A wave changes level where its
+        // own chunk begins, so the turns overlap; one more level while it stores settles those overlaps for the
+        // wave that is about to finish a chunk.  (Measured on fifteen peers: 3 % off the launch; raising other
+        // phases, other hand-over points or a permanent edge for the late layer gain less or nothing.)
+        // (a full grid is two layers of one workgroup per SIMD; on a smaller grid the halves need not share SIMDs,
+        // and two waves that happen to hold the same turn are simply served oldest first again)
+        const bool late_layer = blockIdx.x * 2 >= gridDim.x;  // wave-uniform
         auto step = [&](int64_t g, Set& st, auto odd) {
+            const int turn = decltype(odd)::value != late_layer ? 2 : 0;
             uint32_t from4 = 0;  // four times the lane that holds this lane's entry of chunk g + 1
             {
                 const int j = static_cast<int>(g - g0);  // the chunk scattered below is number j + 1 of the range
@@ -1407,6 +1433,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
                 from4 = pair_lane4 + static_cast<uint32_t>(((j + 1) & (G - 1)) * 2 * k);
             }
             float v[64];
+            set_wave_priority(turn);  // (the payload requests above still go out at the last chunk's level)
             tile_rows_to_regs(v, tile, lane);
             dct64_inv(v);  // along d: v[l] = sum_d Y[lane][d] F[l][d]
             wave_lds_fence();
@@ -1502,6 +1529,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             if (skip1) mark_redo(g + 1);
             repeat = 0;
             // the mean of the next chunk's tile, its trips between the groups of this chunk's stores
+            set_wave_priority(turn + 1);
             MeanState ms;
             mean_begin(ms);
             // a chunk that is to be done again is not stored: its descriptor gets a range of zero bytes
