@@ -1733,7 +1733,9 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
         // one chunk: `st` holds chunk g + 1 and is refilled with chunk g + 3.  Chunk g is stored as soon as it has
         // left the tile, so that its 64 registers are free while the next chunk is scattered
-        auto step = [&](int64_t g, WSet& st) {
+        const bool late_layer = blockIdx.x * 2 >= gridDim.x;  // wave-uniform
+        auto step = [&](int64_t g, WSet& st, bool odd) {
+            set_wave_priority(odd != late_layer ? 2 : 0);  // the two waves of a SIMD take turns, as above
             {
                 // (tile and destination addresses are formed per chunk from an opaque copy of the lane id: hoisted
                 // out of the loop they take a hundred registers)
@@ -1794,8 +1796,8 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             out_after = out3;
         };
         for (int64_t g = g0; g < g1; g += 2) {
-            step(g, s1);
-            if (g + 1 < g1) step(g + 1, s0);
+            step(g, s1, false);
+            if (g + 1 < g1) step(g + 1, s0, true);
         }
         redo_marked();
         return;
@@ -1821,8 +1823,10 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         t_next = c.t;
         if (fast) load_payload(g0 + 1, c.t);
     }
+    const bool late_layer = blockIdx.x * 2 >= gridDim.x;  // wave-uniform
     for (int64_t g = g0; g < g1; ++g) {
         float v[64];
+        set_wave_priority((((g - g0) & 1) != 0) != late_layer ? 2 : 0);  // the two waves of a SIMD take turns, as above
         // ---- first half: everything that needs chunk g's coefficients in the tile
         if (kUseDct) {
             tile_rows_to_regs(v, tile, lane);
