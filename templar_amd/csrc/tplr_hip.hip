@@ -1966,6 +1966,11 @@ __global__ __launch_bounds__(64, 2) void k_ef_step(const tplr_tensor_desc* __res
             cursor_next(cg, g + 1);
             cursor_next(c, g + 1);
         }
+        // the two waves of a SIMD take turns chunk by chunk, as in the aggregate: two priority levels up on every
+        // other chunk, opposite chunks in the two dispatch layers, one more level from the stores to the next
+        // chunk's requests (3 % off the launch)
+        const int turn = (((g - g0) & 1) != 0) != (blockIdx.x * 2 >= gridDim.x) ? 2 : 0;  // wave-uniform
+        set_wave_priority(turn);
         chunk_forward<true>(v, w, tile, lane);
         const Selected s = select_topk<kTwo, false>(w, tile, cand, lane, k, kDctPow2Scale, 0, 0);
         emit_selected<kTwo>(s, lane, k, g, idx12, val);
@@ -1983,6 +1988,7 @@ __global__ __launch_bounds__(64, 2) void k_ef_step(const tplr_tensor_desc* __res
         wave_lds_fence();
 #pragma unroll
         for (int r = 0; r < 64; ++r) v[r] = e[r] - v[r];
+        set_wave_priority(turn + 1);
         store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(dst)), uniform64(ld), lane);
     }
 }
