@@ -763,9 +763,18 @@ struct Counters {
 // lane fetches its own entry from the lane that holds it with lane permutes when the entry is scattered.
 // 8 load instructions per chunk instead of 40 for 20 peers at k = 64, and two register sets of 15
 // registers: the payload is requested two chunks ahead, as in the pipeline with the transform.
+// kTeam (the pipeline with the transform): workgroups of kTeam waves.  A team owns a contiguous range of chunks and
+// deals them out one by one - wave w takes chunks w, w + kTeam, w + 2 kTeam, ... of it - and meets at a barrier
+// before every chunk's row stores, so that the team writes kTeam neighbouring chunks, rows of kTeam * 256
+// contiguous bytes, at the same moment.  (Persistent waves on ranges of their own write each 2 KB of a tensor row in
+// eight visits microseconds apart, and the memory system serves such stores at 5 TB/s where it takes 6-7 TB/s of
+// stores that arrive together.)  Each wave keeps its own tile, counters and marks.
+template <bool kUseDct, int kUnits>
+constexpr int aggregate_team() { return (kUseDct && kUnits > 0 && kUnits <= 16) ? 4 : 1; }  // (24 units: no registers to spare)
+
 template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false, bool kStrided = false, bool kCodes = false,
           int kWideK = 0>
-__global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
+__global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits>()), 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
                                                             int64_t first, int64_t total, int reduce_mode,
@@ -785,7 +794,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     // again on the exact path writes them there
     auto chunk_stats = [&](const float (&v)[64], int64_t g, bool skip) {
         if (!sumsq) return;  // wave-uniform
-        const int lane_ = threadIdx.x;
+        const int lane_ = threadIdx.x & 63;
         float ss = 0.f;
 #pragma unroll
         for (int r = 0; r < 64; ++r) ss = __builtin_fmaf(v[r], v[r], ss);
@@ -811,7 +820,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
 #pragma unroll
         for (int r = 0; r < 64; ++r) z = __builtin_fmaf(v[r], 0.0f, z);
         const bool bad = __ballot(z != z) != 0;
-        if (bad && threadIdx.x == 0) guard[t] = 1;
+        if (bad && (threadIdx.x & 63) == 0) guard[t] = 1;
         return bad;
     };
     using Cnt = Counters<kCntBits>;
@@ -819,23 +828,39 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     // arithmetic of real coefficients maps to 64 tile slots and 8 counter words past the chunk's own
     // (one select per step instead of three); 4-bit counters only: a row of them is 8 whole words
     constexpr bool kPark = kUnits > 0 && kUseDct && kCntBits == 4;
-    __shared__ __align__(16) float tile[kTileFloats + (kPark ? 64 : 0)];
-    __shared__ __align__(16) uint32_t cnt[Cnt::kAlloc + (kPark ? 8 : 0)];
+    constexpr int kTeam = aggregate_team<kUseDct, kUnits>();
+    const int wv = kTeam > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)) : 0;  // wave of the team
+    __shared__ __align__(16) float tile_all[kTeam][kTileFloats + (kPark ? 64 : 0)];
+    __shared__ __align__(16) uint32_t cnt_all[kTeam][Cnt::kAlloc + (kPark ? 8 : 0)];
+    float* const tile = tile_all[wv];
+    uint32_t* const cnt = cnt_all[wv];
     // the marks live in the counters' rounding slack where there is enough of it (5-bit counters:
     // the kernel then still fits eight times into a compute unit's LDS), else in words of their own
     constexpr bool kMarksInSlack = Cnt::kAlloc - Cnt::kWords >= kMarkWords;
-    __shared__ uint32_t own_marks[kMarksInSlack ? 1 : kMarkWords];
-    uint32_t* const marks = kMarksInSlack ? cnt + Cnt::kWords : own_marks;
+    __shared__ uint32_t own_marks[kTeam][kMarksInSlack ? 1 : kMarkWords];
+    uint32_t* const marks = kMarksInSlack ? cnt + Cnt::kWords : own_marks[wv];
     constexpr bool kFast = kUnits > 0;
     constexpr int kRegs = kFast ? kUnits : 1;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63;
     int64_t g0, g1;
-    // (the pipeline with the transform fetches packed indices per group of four or two chunks: slices that
-    // begin on a multiple of that keep every group inside two 128-byte lines)
-    my_range(total, g0, g1, kUnits > 0 && kUseDct ? (k <= 32 ? 4 : 2) : 1, first);
+    // (a team's range begins on a multiple of kTeam chunks of the batch: its waves' rows line up)
+    my_range(total, g0, g1, kTeam, first);
     if (g0 >= g1) return;
     g0 += first;
     g1 += first;
+    // kTeam > 1: [g0, g1) becomes this wave's share, every kTeam-th chunk from g0; `team_steps` is the longest
+    // share of the team (every wave of it has to arrive at that many barriers)
+    constexpr int T = kTeam;
+    const int64_t team_steps = (g1 - g0 + T - 1) / T;
+    g0 += wv;
+    const int64_t my_steps = g0 < g1 ? (g1 - 1 - g0) / T + 1 : 0;
+    if constexpr (kTeam > 1) {
+        if (my_steps == 0) {  // wave-uniform: a team with fewer chunks than waves
+            for (int64_t i = 0; i < team_steps; ++i) __builtin_amdgcn_s_barrier();
+            return;
+        }
+    }
+    const int64_t g_last = g0 + (my_steps - 1) * T;  // this wave's last chunk
 
     const int64_t idx_stride = k + (k >> 1);
     // the inverse transform below is 32x the orthonormal one: its input carries the exact 2^-5
@@ -949,8 +974,13 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
     // Chunks found that way are not stored; they are marked - bit i of `marks` for the i-th chunk of
     // the wave's range - and done again after the main loop.
     marks[lane] = 0;
+    // The slots that lanes and units without an entry scatter to (a row's padding, the words past the tile) are never
+    // cleared with the tile, and LDS keeps what the last kernel on this compute unit left there: a bit pattern that
+    // reads as a claim mark would send every chunk to the exact path.
+    *reinterpret_cast<float4*>(tile + lane * kLd + kChunk) = make_float4(0.f, 0.f, 0.f, 0.f);
+    if constexpr (kPark) tile[kTileFloats + lane] = 0.f;
     auto mark_redo = [&](int64_t g) {  // wave-uniform call, rare
-        const int i = static_cast<int>(g - g0);
+        const int i = static_cast<int>((g - g0) / T);
         if (lane == 0) marks[i >> 5] |= 1u << (i & 31);
     };
     auto add_entry = [&](uint32_t ixe, float val) {
@@ -1218,7 +1248,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             uint32_t m = __builtin_amdgcn_readlane(static_cast<int>(mine), l);
 #pragma unroll 1
             while (m) {
-                redo_chunk(g0 + (l * 32 + __builtin_ctz(m)));
+                redo_chunk(g0 + static_cast<int64_t>(l * 32 + __builtin_ctz(m)) * T);
                 m &= m - 1;
             }
         }
@@ -1276,34 +1306,39 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             }
             st.a[i] = __builtin_nontemporal_load(vrow + le);  // streaming: 7 % faster than cached here
         };
-        // The packed indices come in once per group of G chunks instead of once per chunk.  A chunk's
+        // The packed indices come in once per group of G of the wave's chunks instead of once per chunk.  A chunk's
         // index row is 1.5 k bytes, so neighbouring rows share 128-byte lines, and a streaming load per chunk
-        // fetches those lines from memory again and again (3.3 x the index bytes at k = 32).  Here lane l takes
-        // the four bytes at 3 l of the group - the entries 2 l and 2 l + 1 of its G k entries, whatever k - with
-        // one load per peer and group, and entry j of the group's chunk c is fetched from lane (c k + j) / 2 with
-        // a lane permute when it is scattered.  `cur` is the group being scattered, `nxt` the one on its way:
+        // fetches those lines from memory again and again (3.3 x the index bytes at k = 32).  Here the lanes
+        // c k/2 .. (c + 1) k/2 - 1 take the row of the group's chunk c, four bytes at 3 (l mod k/2) each - two
+        // entries and a byte of the next pair - with one load per peer and group, and entry j of the group's chunk c
+        // is fetched from lane (c k + j) / 2 with a lane permute when it is scattered.  The wave's chunks are T
+        // apart, so the group's rows are T rows apart; the rows between them are those of the team's other waves,
+        // which ask for them at the same moment.  `cur` is the group being scattered, `nxt` the one on its way:
         // requested two chunks before its first use and moved to `cur` at that use.  A lane whose four bytes would
         // end past the rows this launch may read starts one byte earlier and shifts that byte out on arrival.
         const int G = k <= 32 ? 4 : 2;
         const int64_t piece_end = first + total;
+        const int64_t idx_end = piece_end * idx_stride;  // bytes of a peer's index rows that this launch may read
         uint32_t cur[kRegs], nxt[kRegs];
         uint32_t nxt_fix = 0;  // bits to shift out of `nxt` when it becomes `cur`
-        const bool tiny = piece_end * idx_stride < 4;  // one row of two entries is all there is: three bytes
+        const bool tiny = idx_end < 4;  // one row of two entries is all there is: three bytes
+        // where this lane's four bytes begin, counted from the group's first row (lanes past the group's last pair
+        // repeat it)
+        int lane_goff;
+        {
+            const int half_k = k >> 1;
+            int c = lane / half_k, q = lane - c * half_k;
+            if (c >= G) c = G - 1, q = half_k - 1;
+            lane_goff = c * T * static_cast<int>(idx_stride) + 3 * q;
+        }
         auto group_load = [&](uint32_t (&dst)[kRegs], int64_t gs, auto first_call) -> uint32_t {
             if (gs >= piece_end) gs = piece_end - 1;  // (a group nobody will scatter)
-            // bytes to read from: the group, or what is left of the rows of this launch.  The group's last pair
-            // is its last three bytes, and a fourth byte behind them would be the first of another 128-byte line
-            // every other group
-            const int64_t room64 = (piece_end - gs) * idx_stride;
-            const int group_bytes = G * static_cast<int>(idx_stride);
-            const int room = room64 < group_bytes ? static_cast<int>(room64) : group_bytes;
-            // the last pair starts at room - 3: that lane and those past it read the last four bytes instead
-            // (when a row is three bytes, that begins in the row before: `tiny` is the case without one)
-            const int want = 3 * lane;
-            const int from = want < room - 4 ? want : room - 4;
-            const uint32_t fix = want == room - 3 ? 8u : 0u;
-            const uint32_t off = static_cast<uint32_t>(from + 1);
-            const gbyte* grow = (const gbyte*)pp.idx[0] + uniform64(gs * idx_stride - 1);
+            // the last pair of the last row starts at idx_end - 3: that lane reads the last four bytes instead, and
+            // so does every lane whose row lies past the end (a group's later chunks when the range ends inside it)
+            const int64_t want = gs * idx_stride + lane_goff;
+            const int64_t from = want < idx_end - 4 ? want : idx_end - 4;
+            const uint32_t fix = want == idx_end - 3 ? 8u : 0u;
+            const gbyte* grow = (const gbyte*)pp.idx[0];
             if constexpr (kStrided) asm volatile("" : "+s"(walk_peers));
             if constexpr (decltype(first_call)::value) {
                 // (k = 2 makes groups of four rows and a launch of one row has one chunk: no other call is reached)
@@ -1320,9 +1355,13 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             for (int i = 0; i < kRegs; ++i) {
                 if constexpr (!kStrided) {
                     const int u = i < P ? i : P - 1;
-                    grow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u)) + (gs * idx_stride - 1);
+                    grow = reinterpret_cast<const gbyte*>(lane_bcast64(my_idx, u));
                 }
-                dst[i] = __builtin_nontemporal_load((const gu32*)(grow + off));
+                // (a team's other waves read the rest of these lines at the same moment: cached, not streaming)
+                if constexpr (kTeam > 1)
+                    dst[i] = *(const gu32*)(grow + from);
+                else
+                    dst[i] = __builtin_nontemporal_load((const gu32*)(grow + from));
                 if constexpr (kStrided) {
                     if (i + 1 < walk_peers) grow += stride_idx;
                 }
@@ -1354,8 +1393,13 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             const uint32_t fix = group_load(cur, g0, std::true_type{});
 #pragma unroll
             for (int i = 0; i < kRegs; ++i) cur[i] >>= fix;
-            if (G == 2) nxt_fix = group_load(nxt, g0 + 2, std::false_type{});
+            if (G == 2) nxt_fix = group_load(nxt, g0 + 2 * T, std::false_type{});
         }
+        // the cursor from chunk g - T to chunk g
+        auto cursor_to = [&](Cursor& cu, int64_t g) {
+#pragma unroll
+            for (int s = T - 1; s >= 0; --s) cursor_next(cu, g - s);
+        };
         zero_tile();
         {
 #pragma unroll
@@ -1376,15 +1420,15 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         if (skip0) mark_redo(g0);
         repeat = 0;
         mean_pass();
-        if (g0 + 1 < g1) {
-            cursor_next(c, g0 + 1);
-            o1 = out_of(c, g0 + 1);
-            set_load(s1, g0 + 1, c.t);
+        if (g0 + T < g1) {
+            cursor_to(c, g0 + T);
+            o1 = out_of(c, g0 + T);
+            set_load(s1, g0 + T, c.t);
         }
-        if (g0 + 2 < g1) {
-            cursor_next(c, g0 + 2);
-            o2 = out_of(c, g0 + 2);
-            set_load(s0, g0 + 2, c.t);
+        if (g0 + 2 * T < g1) {
+            cursor_to(c, g0 + 2 * T);
+            o2 = out_of(c, g0 + 2 * T);
+            set_load(s0, g0 + 2 * T, c.t);
         }
         {
             // The memory counter completes in order, and the compiler sizes every wait for the
@@ -1403,7 +1447,7 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
         }
 
         // (kStrided) where the chunk loaded last sits in a payload; the loop's loads advance chunk by chunk
-        const int64_t loaded_last = g0 + 2 < g1 ? g0 + 2 : g1 - 1;
+        const int64_t loaded_last = g0 + 2 * T < g1 ? g0 + 2 * T : g_last;
         int64_t last_v = uniform64(loaded_last * k);
         const int dummy_pos = kPark ? kTileFloats + lane : lane * kLd + kChunk;
         const uint32_t park = 4096u + lane;  // (kPark) maps to tile[kTileFloats + lane] and cnt[512 + lane / 8]
@@ -1421,14 +1465,15 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             const int turn = decltype(odd)::value != late_layer ? 2 : 0;
             uint32_t from4 = 0;  // four times the lane that holds this lane's entry of chunk g + 1
             {
-                const int j = static_cast<int>(g - g0);  // the chunk scattered below is number j + 1 of the range
+                const int j = static_cast<int>((g - g0) / T);  // the chunk scattered below is number j + 1 of the wave's
                 if constexpr (decltype(odd)::value) {
                     // groups begin at odd steps: G = 4 alternates "request" and "take over", G = 2 does both
                     if (G == 2 || (j & 2)) {
 #pragma unroll
                         for (int i = 0; i < kRegs; ++i) cur[i] = nxt[i] >> nxt_fix;
                     }
-                    if (G == 2 || !(j & 2)) nxt_fix = group_load(nxt, g0 + ((j + 3) & ~(G - 1)), std::false_type{});
+                    if (G == 2 || !(j & 2))
+                        nxt_fix = group_load(nxt, g0 + static_cast<int64_t>((j + 3) & ~(G - 1)) * T, std::false_type{});
                 }
                 from4 = pair_lane4 + static_cast<uint32_t>(((j + 1) & (G - 1)) * 2 * k);
             }
@@ -1444,16 +1489,16 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
 
             zero_tile();
             const float sc_now = st.sc;
-            const bool more3 = g + 3 < g1;
+            const bool more3 = g + 3 * T < g1;
             Out o3 = o2;
             if (more3) {
-                cursor_next(c, g + 3);
-                o3 = out_of(c, g + 3);
+                cursor_to(c, g + 3 * T);
+                o3 = out_of(c, g + 3 * T);
                 set_scale(st, c.t);
             }
-            const int64_t g_load = more3 ? g + 3 : g1 - 1;
+            const int64_t g_load = more3 ? g + 3 * T : g_last;
             if constexpr (kStrided) {
-                if (more3) last_v += k;
+                if (more3) last_v += T * k;
                 set_walk(last_v);
             }
             constexpr int kSteps = kUnits + 1;
@@ -1525,9 +1570,11 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             if constexpr (!kSubtract) chunk_stats(v, g, skip0);
             // (the loop-carried destination may have been parked in vector registers: make it
             // scalar again, or every store becomes a loop over distinct descriptors)
-            const bool skip1 = g + 1 < g1 && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
-            if (skip1) mark_redo(g + 1);
+            const bool skip1 = g + T < g1 && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
+            if (skip1) mark_redo(g + T);
             repeat = 0;
+            // the team stores together (a bare barrier: nothing is handed over, no memory operation is waited for)
+            if constexpr (kTeam > 1) __builtin_amdgcn_s_barrier();
             // the mean of the next chunk's tile, its trips between the groups of this chunk's stores
             set_wave_priority(turn + 1);
             MeanState ms;
@@ -1579,9 +1626,12 @@ __global__ __launch_bounds__(64, 2) void k_decode_aggregate(const PeerPtrs pp, c
             o1 = o2;
             o2 = o3;
         };
-        for (int64_t g = g0; g < g1; g += 2) {
+        for (int64_t g = g0; g < g1; g += 2 * T) {
             step(g, s1, std::false_type{});
-            if (g + 1 < g1) step(g + 1, s0, std::true_type{});
+            if (g + T < g1) step(g + T, s0, std::true_type{});
+        }
+        if constexpr (kTeam > 1) {
+            for (int64_t i = my_steps; i < team_steps; ++i) __builtin_amdgcn_s_barrier();
         }
         redo_marked();
         return;
@@ -3445,12 +3495,13 @@ static inline unsigned grid8(int64_t n) { return static_cast<unsigned>(((n + 7) 
 // calculator reports it for the kernel at hand (registers or LDS bound it); a larger grid
 // would leave a second, mostly empty round
 template <typename Kernel>
-static int persistent_grid(Kernel kernel, int64_t total) {
+static int persistent_grid(Kernel kernel, int64_t total, int threads = 64) {
     int n_cu = 256, per_cu = 0, dev = 0, v = 0;
     if (hipGetDevice(&dev) == hipSuccess &&
         hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
         n_cu = v;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 64, 0) != hipSuccess || per_cu < 1) per_cu = 4;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1)
+        per_cu = threads > 64 ? 2 : 4;
     int64_t g = static_cast<int64_t>(n_cu) * per_cu;
     g = g < 8 ? 8 : (g / 8) * 8;
     const int64_t need = ((total + 7) / 8) * 8;
@@ -3470,22 +3521,23 @@ static int launch_encode_as(Kernel kernel, const tplr_tensor_desc* d_desc, const
     return launch_status();
 }
 
-template <typename Kernel>
+// kTeam: waves per workgroup of the kernel (aggregate_team<> of its instantiation)
+template <int kTeam = 1, typename Kernel>
 static int launch_decode_as(Kernel kernel, const PeerPtrs& pp, const float* d_scale, int n_peers, int k,
                             const tplr_tensor_desc* d_desc, const tplr_tensor_desc& single, int n_tensors,
                             int64_t total, int reduce_mode, int normalise, float* d_sumsq, void* stream,
                             int64_t stride_idx = 0, int64_t stride_val = 0, const float* d_deq = nullptr,
                             int32_t* d_guard = nullptr) {
-    static int resident = 0;  // per kernel variant
-    if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40);
+    static int resident = 0;  // workgroups; per kernel variant
+    if (resident == 0) resident = persistent_grid(kernel, int64_t{1} << 40, 64 * kTeam);
     // a wave keeps one mark per chunk of its range (chunks to be done again on the exact path), so
     // one launch takes at most kMaxChunksPerWave chunks per wave: 68 GB of output on a whole device
-    // (the margin covers the rounding of the slices and their alignment to index groups)
-    const int64_t piece = static_cast<int64_t>(resident) * (kMaxChunksPerWave - 8);
+    // (the margin covers the rounding of the slices and their alignment)
+    const int64_t piece = static_cast<int64_t>(resident) * kTeam * (kMaxChunksPerWave - 8);
     for (int64_t first = 0; first < total; first += piece) {
         const int64_t count = total - first < piece ? total - first : piece;
-        const int64_t need = ((count + 7) / 8) * 8;
-        const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64);
+        const int64_t need = (((count + kTeam - 1) / kTeam + 7) / 8) * 8;  // workgroups that have a chunk each, in eights
+        const dim3 grid(static_cast<unsigned>(need < resident ? need : resident)), block(64 * kTeam);
         hipLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), pp, d_scale, n_peers, k, d_desc,
                            single, n_tensors, first, count, reduce_mode, normalise, d_sumsq, stride_idx, stride_val, d_deq,
                            d_guard);
@@ -3724,7 +3776,7 @@ static int subtract_decoded(const uint8_t* d_idx12, const float* d_val, const fl
     pp.idx[0] = d_idx12;
     pp.val[0] = d_val;
     // (one peer: the factor table (n_tensors, 1) is the aggregate's clip-factor table)
-    return launch_decode_as(k_decode_aggregate<true, 8, 4, true, true>, pp, d_factor, 1, k, d_desc, none, n_tensors,
+    return launch_decode_as<4>(k_decode_aggregate<true, 8, 4, true, true>, pp, d_factor, 1, k, d_desc, none, n_tensors,
                             total_chunks, TPLR_REDUCE_MEAN, 0, nullptr, stream, 0, 0, nullptr, d_guard);
 }
 
@@ -3766,15 +3818,15 @@ int tplr_outer_step_batch(const uint8_t* const* h_idx12, const float* const* h_v
         const int options = d_chunk_stats ? 2 : 0;
         int st;
         if (n_peers <= 8 && strided)
-            st = launch_decode_as(k_decode_aggregate<true, 8, 4, true, true>, pp, d_factor, n_peers, k, d_param_desc, none,
+            st = launch_decode_as<4>(k_decode_aggregate<true, 8, 4, true, true>, pp, d_factor, n_peers, k, d_param_desc, none,
                                   n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats, stream, si, sv4 / 4,
                                   nullptr, d_nonfinite);
         else if (strided)
-            st = launch_decode_as(k_decode_aggregate<true, 16, 4, true, true>, pp, d_factor, n_peers, k, d_param_desc,
+            st = launch_decode_as<4>(k_decode_aggregate<true, 16, 4, true, true>, pp, d_factor, n_peers, k, d_param_desc,
                                   none, n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats, stream, si,
                                   sv4 / 4, nullptr, d_nonfinite);
         else
-            st = launch_decode_as(k_decode_aggregate<true, 16, 4, true, false>, pp, d_factor, n_peers, k, d_param_desc,
+            st = launch_decode_as<4>(k_decode_aggregate<true, 16, 4, true, false>, pp, d_factor, n_peers, k, d_param_desc,
                                   none, n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats, stream, 0, 0,
                                   nullptr, d_nonfinite);
         if (st) return st;
@@ -3908,13 +3960,13 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
 #define TPLR_DECODE_CASE(U, BITS)                                                                                   \
     case U:                                                                                                         \
         if (strided)                                                                                                \
-            return use_dct ? launch_decode_as(k_decode_aggregate<true, U, BITS, false, true>, pp, d_scale, n_peers,   \
+            return use_dct ? launch_decode_as<aggregate_team<true, U>()>(k_decode_aggregate<true, U, BITS, false, true>, pp, d_scale, n_peers,\
                                               k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq,  \
                                               stream, si, sv)                                                        \
                            : launch_decode_as(k_decode_aggregate<false, U, BITS, false, true>, pp, d_scale, n_peers,  \
                                               k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq,  \
                                               stream, si, sv);                                                       \
-        return use_dct ? launch_decode_as(k_decode_aggregate<true, U, BITS>, pp, d_scale, n_peers, k, d_desc,         \
+        return use_dct ? launch_decode_as<aggregate_team<true, U>()>(k_decode_aggregate<true, U, BITS>, pp, d_scale, n_peers, k, d_desc,\
                                           single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream)         \
                        : launch_decode_as(k_decode_aggregate<false, U, BITS>, pp, d_scale, n_peers, k, d_desc,        \
                                           single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream);
@@ -4538,7 +4590,7 @@ int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_va
         if (p < n_peers && (!pp.idx[p] || !pp.val[p])) return TPLR_E_BADARG;
     }
     static int resident = 0;
-    if (resident == 0) resident = persistent_grid(k_decode_aggregate<true, 16, 4>, int64_t{1} << 40);  // the grid it stands in for
+    if (resident == 0) resident = 4 * persistent_grid(k_decode_aggregate<true, 16, 4>, int64_t{1} << 40, 256);  // as many waves as the launch it stands in for
     const int64_t need = ((total_chunks + 7) / 8) * 8;
     const dim3 grid(static_cast<unsigned>(need < resident ? need : resident));
     const hipStream_t on = static_cast<hipStream_t>(stream);
