@@ -422,7 +422,8 @@ Total HBM traffic per launch {fb + wb:,.0f} B = {(fb + wb) / alg:.3f} x the algo
                 text += f"""
 ## What the memory system alone needs: the kernel's loads and stores without the scatter and the transform
 
-`k_calib_aggregate` (`tplr_calib_aggregate`) runs the same grid over the same chunk ranges and issues the same streaming
+`k_calib_aggregate` (`tplr_calib_aggregate`) runs the same grid over the same chunk ranges (teams of four waves that
+meet at a barrier before their stores where the launch itself runs them: `k_calib_aggregate_team`) and issues the same
 payload loads and the same 64 row stores per chunk, and nothing else; with no peers it is the pure fill of the outputs.
 
 {_cmd(tag, 'calib', 'kt', a)}

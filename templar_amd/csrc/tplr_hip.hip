@@ -3477,6 +3477,81 @@ __global__ __launch_bounds__(64, 2) void k_calib_aggregate(const PeerPtrs pp, in
     }
 }
 
+// The same for the pipeline with the transform up to 16 peers, whose workgroups are teams of four waves: wave w
+// takes chunks w, w + 4, ... of the team's range, a group's index rows are four rows apart (lanes c k/2 .. take the
+// row of the group's chunk c; cached loads), and the team meets at a barrier before every chunk's stores.
+template <int kGroup>
+__global__ __launch_bounds__(256, 2) void k_calib_aggregate_team(const PeerPtrs pp, int P, int k,
+                                                                 const tplr_tensor_desc* __restrict__ table,
+                                                                 int n_tensors, int64_t total) {
+    constexpr int T = 4;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+    int64_t t0, t1;
+    my_range(total, t0, t1, T);
+    if (t0 >= t1) return;
+    const int64_t idx_stride = k + (k >> 1), idx_end = total * idx_stride;
+    const int le = lane < k ? lane : 0;
+    int lane_goff;
+    {
+        const int half_k = k >> 1;
+        int c = lane / half_k, q = lane - c * half_k;
+        if (c >= kGroup) c = kGroup - 1, q = half_k - 1;
+        lane_goff = c * T * static_cast<int>(idx_stride) + 3 * q;
+    }
+    constexpr int kU = 16;
+    uint32_t ix[kU];
+    float a[2][kU];
+#pragma unroll
+    for (int i = 0; i < kU; ++i) ix[i] = 0, a[0][i] = 0.f, a[1][i] = 0.f;
+    const int64_t steps = (t1 - t0 + T - 1) / T;  // of the team; a wave past the end repeats its last chunk and stores nothing
+    auto clampg = [&](int64_t g) { return g < t1 ? g : t1 - 1; };
+    auto load_group = [&](int64_t g) {
+        const int64_t want = clampg(g) * idx_stride + lane_goff;
+        const int64_t from = want < idx_end - 4 ? want : idx_end - 4;
+#pragma unroll
+        for (int i = 0; i < kU; ++i)
+            if (i < P) ix[i] = *(const gu32*)((const gbyte*)pp.idx[i] + from);
+    };
+    auto load_vals = [&](auto st, int64_t g) {
+        constexpr int s = decltype(st)::value;
+#pragma unroll
+        for (int i = 0; i < kU; ++i)
+            if (i < P) a[s][i] = __builtin_nontemporal_load((const gfloat*)pp.val[i] + clampg(g) * k + le);
+    };
+    Cursor c;
+    tplr_tensor_desc none = {};
+    cursor_seek(c, table, none, n_tensors, clampg(t0 + w));
+    load_group(t0 + w);
+    load_vals(Index<0>{}, t0 + w);
+    load_vals(Index<1>{}, t0 + w + T);
+    auto body = [&](int64_t gb, auto st, bool with_group) {
+        const int64_t g = gb + w;
+        float x = 0.f;
+#pragma unroll
+        for (int i = 0; i < kU; ++i) x += a[decltype(st)::value][i] + __builtin_bit_cast(float, ix[i]);
+        if (with_group) load_group(g + 2 * T);
+        load_vals(st, g + 2 * T);
+        float v[64];
+#pragma unroll
+        for (int r = 0; r < 64; ++r) v[r] = x + static_cast<float>(r);
+        __builtin_amdgcn_s_barrier();
+        if (g < t1) store_chunk_cols(v, (float*)c.base, c.ld, c.y, c.xc, lane);
+#pragma unroll
+        for (int j = 1; j <= T; ++j)
+            if (g + j < t1) cursor_next(c, g + j);
+    };
+    // (every wave of the team runs the same number of steps, and with them of barriers)
+    for (int64_t s = 0; s < steps; s += kGroup) {
+        const int64_t gb = t0 + s * T;
+        body(gb, Index<0>{}, false);
+        if (s + 1 < steps) body(gb + T, Index<1>{}, kGroup == 2);
+        if constexpr (kGroup == 4) {
+            if (s + 2 < steps) body(gb + 2 * T, Index<0>{}, true);
+            if (s + 3 < steps) body(gb + 3 * T, Index<1>{}, false);
+        }
+    }
+}
+
 }  // namespace tplr
 
 // =========================================================================================
@@ -4594,6 +4669,16 @@ int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_va
     const int64_t need = ((total_chunks + 7) / 8) * 8;
     const dim3 grid(static_cast<unsigned>(need < resident ? need : resident));
     const hipStream_t on = static_cast<hipStream_t>(stream);
+    if (use_dct && n_peers <= 16) {
+        // (the launch it stands for runs teams of four waves)
+        const int64_t teams = (((total_chunks + 3) / 4 + 7) / 8) * 8;
+        const dim3 tgrid(static_cast<unsigned>(teams < resident / 4 ? teams : resident / 4));
+        if (k <= 32)
+            hipLaunchKernelGGL(k_calib_aggregate_team<4>, tgrid, dim3(256), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
+        else
+            hipLaunchKernelGGL(k_calib_aggregate_team<2>, tgrid, dim3(256), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
+        return launch_status();
+    }
     if (!use_dct)
         hipLaunchKernelGGL(k_calib_aggregate<0>, grid, dim3(64), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
     else if (k <= 32)
