@@ -769,12 +769,15 @@ struct Counters {
 // contiguous bytes, at the same moment.  (Persistent waves on ranges of their own write each 2 KB of a tensor row in
 // eight visits microseconds apart, and the memory system serves such stores at 5 TB/s where it takes 6-7 TB/s of
 // stores that arrive together.)  Each wave keeps its own tile, counters and marks.
-template <bool kUseDct, int kUnits>
-constexpr int aggregate_team() { return (kUseDct && kUnits > 0 && kUnits <= 16) ? 4 : 1; }  // (24 units: no registers to spare)
+template <bool kUseDct, int kUnits, int kWideK = 0>
+constexpr int aggregate_team() {
+    // the pipeline with the transform up to 16 units (with 24 there are no registers to spare) and the one from codes
+    return ((kUseDct && kUnits > 0 && kUnits <= 16) || kWideK > 0) ? 4 : 1;
+}
 
 template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false, bool kStrided = false, bool kCodes = false,
           int kWideK = 0>
-__global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits>()), 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
+__global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK>()), 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
                                                             int64_t first, int64_t total, int reduce_mode,
@@ -828,7 +831,7 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits>()), 2) void k
     // arithmetic of real coefficients maps to 64 tile slots and 8 counter words past the chunk's own
     // (one select per step instead of three); 4-bit counters only: a row of them is 8 whole words
     constexpr bool kPark = kUnits > 0 && kUseDct && kCntBits == 4;
-    constexpr int kTeam = aggregate_team<kUseDct, kUnits>();
+    constexpr int kTeam = aggregate_team<kUseDct, kUnits, kWideK>();
     const int wv = kTeam > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)) : 0;  // wave of the team
     __shared__ __align__(16) float tile_all[kTeam][kTileFloats + (kPark ? 64 : 0)];
     __shared__ __align__(16) uint32_t cnt_all[kTeam][Cnt::kAlloc + (kPark ? 8 : 0)];
@@ -1195,6 +1198,12 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits>()), 2) void k
                    cu.ld, cu.t};
     };
 
+    // the cursor from chunk g - T, the wave's last one, to chunk g
+    auto cursor_to = [&](Cursor& cu, int64_t g) {
+#pragma unroll
+        for (int s = T - 1; s >= 0; --s) cursor_next(cu, g - s);
+    };
+
     // ---- the chunks marked for the exact path, one at a time, after the wave's main loop
     auto redo_chunk = [&](int64_t g) {
         Cursor cs;
@@ -1395,11 +1404,6 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits>()), 2) void k
             for (int i = 0; i < kRegs; ++i) cur[i] >>= fix;
             if (G == 2) nxt_fix = group_load(nxt, g0 + 2 * T, std::false_type{});
         }
-        // the cursor from chunk g - T to chunk g
-        auto cursor_to = [&](Cursor& cu, int64_t g) {
-#pragma unroll
-            for (int s = T - 1; s >= 0; --s) cursor_next(cu, g - s);
-        };
         zero_tile();
         {
 #pragma unroll
@@ -1771,25 +1775,27 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits>()), 2) void k
         if (skip_cur) mark_redo(g0);
         repeat = 0;
         mean_pass();
-        if (g0 + 1 < g1) {
-            cursor_next(c, g0 + 1);
-            out_next = out_of(c, g0 + 1);
-            wset_load(s1, g0 + 1, c.t);
+        if (g0 + T < g1) {
+            cursor_to(c, g0 + T);
+            out_next = out_of(c, g0 + T);
+            wset_load(s1, g0 + T, c.t);
         }
-        if (g0 + 2 < g1) {
-            cursor_next(c, g0 + 2);
-            out_after = out_of(c, g0 + 2);
-            wset_load(s0, g0 + 2, c.t);
+        if (g0 + 2 * T < g1) {
+            cursor_to(c, g0 + 2 * T);
+            out_after = out_of(c, g0 + 2 * T);
+            wset_load(s0, g0 + 2 * T, c.t);
         }
+        // (the chunks of a wave are T apart: g + 1 below stands for the wave's next chunk)
         // one chunk: `st` holds chunk g + 1 and is refilled with chunk g + 3.  Chunk g is stored as soon as it has
         // left the tile, so that its 64 registers are free while the next chunk is scattered
         const bool late_layer = blockIdx.x * 2 >= gridDim.x;  // wave-uniform
         auto step = [&](int64_t g, WSet& st, bool odd) {
-            set_wave_priority(odd != late_layer ? 2 : 0);  // the two waves of a SIMD take turns, as above
+            const int turn = odd != late_layer ? 2 : 0;
+            set_wave_priority(turn);  // the two waves of a SIMD take turns, as above
             {
                 // (tile and destination addresses are formed per chunk from an opaque copy of the lane id: hoisted
                 // out of the loop they take a hundred registers)
-                int lane = threadIdx.x;
+                int lane = threadIdx.x & 63;
                 asm volatile("" : "+v"(lane));
                 float v[64];
                 gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0));
@@ -1815,6 +1821,11 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits>()), 2) void k
 #pragma unroll
                     for (int r = 0; r < 64; ++r) v[r] = before[r] - v[r];
                 }
+                // the team stores together, one priority level up (as in the pipeline with the transform)
+                if constexpr (kTeam > 1) {
+                    __builtin_amdgcn_s_barrier();
+                    set_wave_priority(turn + 1);
+                }
                 if (kSubtract || out_cur.ld > 0) {
                     store_chunk_rows(v, (void*)dst, uniform64(out_cur.ld), lane, skip_cur || tripped);
                 } else if (!skip_cur) {
@@ -1823,20 +1834,21 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits>()), 2) void k
                         reinterpret_cast<float4*>((float*)dst)[q0 * 64 + lane] =
                             make_float4(v[4 * q0], v[4 * q0 + 1], v[4 * q0 + 2], v[4 * q0 + 3]);
                 }
+                if constexpr (kTeam > 1) set_wave_priority(turn);
             }
-            const bool more = g + 1 < g1;
+            const bool more = g + T < g1;
             Out out3 = out_after;
             bool skip_next = false;
             if (more) {
                 zero_tile();
                 wset_scatter(st);
-                if (g + 3 < g1) {
-                    cursor_next(c, g + 3);
-                    out3 = out_of(c, g + 3);
-                    wset_load(st, g + 3, c.t);
+                if (g + 3 * T < g1) {
+                    cursor_to(c, g + 3 * T);
+                    out3 = out_of(c, g + 3 * T);
+                    wset_load(st, g + 3 * T, c.t);
                 }
                 skip_next = __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
-                if (skip_next) mark_redo(g + 1);
+                if (skip_next) mark_redo(g + T);
                 repeat = 0;
                 mean_pass();
             }
@@ -1845,9 +1857,12 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits>()), 2) void k
             out_next = out_after;
             out_after = out3;
         };
-        for (int64_t g = g0; g < g1; g += 2) {
+        for (int64_t g = g0; g < g1; g += 2 * T) {
             step(g, s1, false);
-            if (g + 1 < g1) step(g + 1, s0, true);
+            if (g + T < g1) step(g + T, s0, true);
+        }
+        if constexpr (kTeam > 1) {
+            for (int64_t i = my_steps; i < team_steps; ++i) __builtin_amdgcn_s_barrier();
         }
         redo_marked();
         return;
@@ -3943,10 +3958,10 @@ int tplr_outer_step_codes_batch(const uint8_t* const* h_idx12, const uint8_t* co
         const int options = d_chunk_stats ? 2 : 0;
         int st;
 #define TPLR_OUTER_CODES(U, BITS)                                                                                       \
-    (k == 64 ? launch_decode_as(k_decode_aggregate<false, U, BITS, true, true, true, 64>, pp, d_factor, n_peers, k,      \
+    (k == 64 ? launch_decode_as<4>(k_decode_aggregate<false, U, BITS, true, true, true, 64>, pp, d_factor, n_peers, k,      \
                                 d_param_desc, none, n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats,  \
                                 stream, si, sv, d_deq, d_nonfinite)                                                     \
-             : launch_decode_as(k_decode_aggregate<false, U, BITS, true, true, true, 32>, pp, d_factor, n_peers, k,      \
+             : launch_decode_as<4>(k_decode_aggregate<false, U, BITS, true, true, true, 32>, pp, d_factor, n_peers, k,      \
                                 d_param_desc, none, n_tensors, total_chunks, TPLR_REDUCE_MEAN, options, d_chunk_stats,  \
                                 stream, si, sv, d_deq, d_nonfinite))
         if (n_peers <= 15)
@@ -4010,11 +4025,11 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
 #define TPLR_CODES_CASE(U, BITS)                                                                                    \
     case U:                                                                                                         \
         if (strided && wide_ok && k == 64)                                                                          \
-            return launch_decode_as(k_decode_aggregate<false, U, BITS, false, true, true, 64>, pp, d_scale, n_peers,  \
+            return launch_decode_as<4>(k_decode_aggregate<false, U, BITS, false, true, true, 64>, pp, d_scale, n_peers,  \
                                     k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream, si, \
                                     sv4, d_deq);                                                                    \
         if (strided && wide_ok && k == 32)                                                                          \
-            return launch_decode_as(k_decode_aggregate<false, U, BITS, false, true, true, 32>, pp, d_scale, n_peers,  \
+            return launch_decode_as<4>(k_decode_aggregate<false, U, BITS, false, true, true, 32>, pp, d_scale, n_peers,  \
                                     k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream, si, \
                                     sv4, d_deq);                                                                    \
         if (strided)                                                                                                \
