@@ -1997,24 +1997,42 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK>()), 2
 // the k selected values go back into a cleared tile exactly as the one-peer decode adds them (0 + value * 2^-5),
 // through the inverse transform, and the difference is stored.  Two waves per SIMD (a whole tile, 64 more
 // registers): the launch moves 14 GB and is bound by that.
+// Workgroups are teams of four waves, as in the aggregate: wave w takes every fourth chunk of the team's range, the
+// team reads rows of 1 KB at the same moment and meets at a barrier before it stores them (6 % off the launch).
+// (k <= 32 only: at k = 64 the team form is 2 % slower than single waves)
 template <bool kTwo>
-__global__ __launch_bounds__(64, 2) void k_ef_step(const tplr_tensor_desc* __restrict__ table,
+constexpr int ef_team() { return kTwo ? 1 : 4; }
+template <bool kTwo>
+__global__ __launch_bounds__(64 * ef_team<kTwo>(), 2) void k_ef_step(const tplr_tensor_desc* __restrict__ table,
                                                    const tplr_tensor_desc* __restrict__ grad_table, int n_tensors,
                                                    int64_t total, int k, float decay, uint8_t* __restrict__ idx12,
                                                    float* __restrict__ val) {
-    __shared__ __align__(16) float tile[kTileFloats];
-    __shared__ uint64_t cand[kCandCap];
+    constexpr int T = ef_team<kTwo>();
+    __shared__ __align__(16) float tile_all[T][kTileFloats];
+    __shared__ uint64_t cand_all[T][kCandCap];
+    const int wv = T > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)) : 0;
+    float* const tile = tile_all[wv];
+    uint64_t* const cand = cand_all[wv];
     int64_t g0, g1;
-    my_range(total, g0, g1);
+    my_range(total, g0, g1, T);
     if (g0 >= g1) return;
+    const int64_t team_steps = (g1 - g0 + T - 1) / T;
+    g0 += wv;
+    const int64_t my_steps = g0 < g1 ? (g1 - 1 - g0) / T + 1 : 0;
+    if (my_steps == 0) {  // wave-uniform: a team with fewer chunks than waves
+        if constexpr (T > 1) {
+            for (int64_t i = 0; i < team_steps; ++i) __builtin_amdgcn_s_barrier();
+        }
+        return;
+    }
     Cursor c, cg;
     tplr_tensor_desc none = {};
     cursor_seek(c, table, none, n_tensors, g0);
     cursor_seek(cg, grad_table, none, n_tensors, g0);
-    for (int64_t g = g0; g < g1; ++g) {
+    for (int64_t g = g0; g < g1; g += T) {
         // (lane-derived addresses are formed per chunk from a copy of the lane id the optimiser cannot see
         // through: hoisted out of the loop they would be spilled)
-        int lane = threadIdx.x;
+        int lane = threadIdx.x & 63;
         asm volatile("" : "+v"(lane));
         float e[64], v[64], w[64];
         load_chunk_cols(e, c, lane);
@@ -2027,14 +2045,17 @@ __global__ __launch_bounds__(64, 2) void k_ef_step(const tplr_tensor_desc* __res
         }
         gfloat* const dst = c.base + (c.y * 64) * c.ld + static_cast<int64_t>(c.xc) * 64;
         const int64_t ld = c.ld;
-        if (g + 1 < g1) {
-            cursor_next(cg, g + 1);
-            cursor_next(c, g + 1);
+        if (g + T < g1) {
+#pragma unroll
+            for (int s = 1; s <= T; ++s) {
+                cursor_next(cg, g + s);
+                cursor_next(c, g + s);
+            }
         }
         // the two waves of a SIMD take turns chunk by chunk, as in the aggregate: two priority levels up on every
         // other chunk, opposite chunks in the two dispatch layers, one more level from the stores to the next
         // chunk's requests (3 % off the launch)
-        const int turn = (((g - g0) & 1) != 0) != (blockIdx.x * 2 >= gridDim.x) ? 2 : 0;  // wave-uniform
+        const int turn = ((((g - g0) / T) & 1) != 0) != (blockIdx.x * 2 >= gridDim.x) ? 2 : 0;  // wave-uniform
         set_wave_priority(turn);
         chunk_forward<true>(v, w, tile, lane);
         const Selected s = select_topk<kTwo, false>(w, tile, cand, lane, k, kDctPow2Scale, 0, 0);
@@ -2053,8 +2074,12 @@ __global__ __launch_bounds__(64, 2) void k_ef_step(const tplr_tensor_desc* __res
         wave_lds_fence();
 #pragma unroll
         for (int r = 0; r < 64; ++r) v[r] = e[r] - v[r];
+        if constexpr (T > 1) __builtin_amdgcn_s_barrier();  // the team stores together
         set_wave_priority(turn + 1);
         store_chunk_rows(v, (void*)uniform64(reinterpret_cast<int64_t>(dst)), uniform64(ld), lane);
+    }
+    if constexpr (T > 1) {
+        for (int64_t i = my_steps; i < team_steps; ++i) __builtin_amdgcn_s_barrier();
     }
 }
 
@@ -3827,17 +3852,20 @@ int tplr_ef_step_batch(const tplr_tensor_desc* d_ef_desc, const tplr_tensor_desc
         return TPLR_E_BADARG;
     if (k > 64) return TPLR_E_TOOMANY;
     if (total_chunks == 0) return 0;
-    const int64_t need = ((total_chunks + 7) / 8) * 8;
     if (k > 32) {
+        constexpr int kT = ef_team<true>();
+        const int64_t teams = (((total_chunks + kT - 1) / kT + 7) / 8) * 8;  // workgroups that have a chunk each, in eights
         static int resident = 0;
-        if (resident == 0) resident = persistent_grid(k_ef_step<true>, int64_t{1} << 40);
-        hipLaunchKernelGGL(k_ef_step<true>, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+        if (resident == 0) resident = persistent_grid(k_ef_step<true>, int64_t{1} << 40, 64 * kT);
+        hipLaunchKernelGGL(k_ef_step<true>, dim3(static_cast<unsigned>(teams < resident ? teams : resident)), dim3(64 * kT), 0,
                            static_cast<hipStream_t>(stream), d_ef_desc, d_grad_desc, n_tensors, total_chunks, k, decay,
                            d_idx12, d_val);
     } else {
         static int resident = 0;
-        if (resident == 0) resident = persistent_grid(k_ef_step<false>, int64_t{1} << 40);
-        hipLaunchKernelGGL(k_ef_step<false>, dim3(static_cast<unsigned>(need < resident ? need : resident)), dim3(64), 0,
+        constexpr int kT = ef_team<false>();
+        const int64_t teams = (((total_chunks + kT - 1) / kT + 7) / 8) * 8;
+        if (resident == 0) resident = persistent_grid(k_ef_step<false>, int64_t{1} << 40, 64 * kT);
+        hipLaunchKernelGGL(k_ef_step<false>, dim3(static_cast<unsigned>(teams < resident ? teams : resident)), dim3(64 * kT), 0,
                            static_cast<hipStream_t>(stream), d_ef_desc, d_grad_desc, n_tensors, total_chunks, k, decay,
                            d_idx12, d_val);
     }
