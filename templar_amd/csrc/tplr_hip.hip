@@ -800,15 +800,16 @@ struct Counters {
 // contiguous bytes, at the same moment.  (Persistent waves on ranges of their own write each 2 KB of a tensor row in
 // eight visits microseconds apart, and the memory system serves such stores at 5 TB/s where it takes 6-7 TB/s of
 // stores that arrive together.)  Each wave keeps its own tile, counters and marks.
-template <bool kUseDct, int kUnits, int kWideK = 0>
+template <bool kUseDct, int kUnits, int kWideK = 0, bool kPlain = false>
 constexpr int aggregate_team() {
-    // the pipeline with the transform up to 16 units (with 24 there are no registers to spare) and the one from codes
-    return ((kUseDct && kUnits > 0 && kUnits <= 16) || kWideK > 0) ? 4 : 1;
+    // the pipeline with the transform up to 16 units (with 24 there are no registers to spare), the one from codes,
+    // and (kPlain: fp32 values, no subtraction) the fast path without the transform
+    return ((kUseDct && kUnits > 0 && kUnits <= 16) || kWideK > 0 || (kPlain && !kUseDct && kUnits > 0)) ? 4 : 1;
 }
 
 template <bool kUseDct, int kUnits, int kCntBits, bool kSubtract = false, bool kStrided = false, bool kCodes = false,
           int kWideK = 0>
-__global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK>()), 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
+__global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK, !kCodes && !kSubtract>()), 2) void k_decode_aggregate(const PeerPtrs pp, const float* __restrict__ scale, int P,
                                                             int k, const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
                                                             int64_t first, int64_t total, int reduce_mode,
@@ -862,7 +863,7 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK>()), 2
     // arithmetic of real coefficients maps to 64 tile slots and 8 counter words past the chunk's own
     // (one select per step instead of three); 4-bit counters only: a row of them is 8 whole words
     constexpr bool kPark = kUnits > 0 && kUseDct && kCntBits == 4;
-    constexpr int kTeam = aggregate_team<kUseDct, kUnits, kWideK>();
+    constexpr int kTeam = aggregate_team<kUseDct, kUnits, kWideK, !kCodes && !kSubtract>();
     const int wv = kTeam > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)) : 0;  // wave of the team
     __shared__ __align__(16) float tile_all[kTeam][kTileFloats + (kPark ? 64 : 0)];
     __shared__ __align__(16) uint32_t cnt_all[kTeam][Cnt::kAlloc + (kPark ? 8 : 0)];
@@ -1913,16 +1914,18 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK>()), 2
     if (skip_cur) mark_redo(g0);
     repeat = 0;
     mean_pass();
-    if (g0 + 1 < g1) {
-        cursor_next(c, g0 + 1);
-        out_next = out_of(c, g0 + 1);
+    // (the chunks of a wave are T apart: "g + 1" in the comments below stands for the wave's next chunk)
+    if (g0 + T < g1) {
+        cursor_to(c, g0 + T);
+        out_next = out_of(c, g0 + T);
         t_next = c.t;
-        if (fast) load_payload(g0 + 1, c.t);
+        if (fast) load_payload(g0 + T, c.t);
     }
     const bool late_layer = blockIdx.x * 2 >= gridDim.x;  // wave-uniform
-    for (int64_t g = g0; g < g1; ++g) {
+    for (int64_t g = g0; g < g1; g += T) {
         float v[64];
-        set_wave_priority((((g - g0) & 1) != 0) != late_layer ? 2 : 0);  // the two waves of a SIMD take turns, as above
+        const int turn = ((((g - g0) / T) & 1) != 0) != late_layer ? 2 : 0;
+        set_wave_priority(turn);  // the two waves of a SIMD take turns, as above
         // ---- first half: everything that needs chunk g's coefficients in the tile
         if (kUseDct) {
             tile_rows_to_regs(v, tile, lane);
@@ -1944,7 +1947,7 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK>()), 2
         wave_lds_fence();
 
         // ---- the tile is free: chunk g + 1 moves in, chunk g + 2 is requested
-        const bool more = g + 1 < g1;
+        const bool more = g + T < g1;
         Out out_after = out_next;
         int t_after = t_next;
         // Without the transform chunk g is complete here: its 64 row stores go out first - the wave stands at
@@ -1959,6 +1962,10 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK>()), 2
                 skip_cur ? 0 : static_cast<int>((63 * ld_s + 64) * 4), 0x00020000);
             const int ld4 = static_cast<int>(ld_s) * 4;
             zero_tile();
+            if constexpr (kTeam > 1) {  // the team stores together, one priority level up
+                __builtin_amdgcn_s_barrier();
+                set_wave_priority(turn + 1);
+            }
             if constexpr (kUnits <= 16) {
                 constexpr int kGroups = 4, kPerGroup = (kRegs + kGroups - 1) / kGroups;
                 static_for<kGroups>([&](auto qt) {
@@ -1966,42 +1973,46 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK>()), 2
 #pragma unroll
                     for (int r = q * 16; r < (q + 1) * 16; ++r)
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v[r]), wr, lane * 4, r * ld4, 2);
-                    scatter(g + 1, t_next, q * kPerGroup, (q + 1) * kPerGroup);
+                    scatter(g + T, t_next, q * kPerGroup, (q + 1) * kPerGroup);
                 });
             } else {
 #pragma unroll
                 for (int r = 0; r < 64; ++r)
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v[r]), wr, lane * 4, r * ld4, 2);
-                scatter(g + 1, t_next);
+                scatter(g + T, t_next);
             }
-            if (g + 2 < g1) {
-                cursor_next(c, g + 2);
-                out_after = out_of(c, g + 2);
+            if constexpr (kTeam > 1) set_wave_priority(turn);
+            if (g + 2 * T < g1) {
+                cursor_to(c, g + 2 * T);
+                out_after = out_of(c, g + 2 * T);
                 t_after = c.t;
-                load_payload(g + 2, c.t);
+                load_payload(g + 2 * T, c.t);
             }
             stored = true;
         } else if (more) {
             zero_tile();
-            scatter(g + 1, t_next);
-            if (g + 2 < g1) {
-                cursor_next(c, g + 2);
-                out_after = out_of(c, g + 2);
+            scatter(g + T, t_next);
+            if (g + 2 * T < g1) {
+                cursor_to(c, g + 2 * T);
+                out_after = out_of(c, g + 2 * T);
                 t_after = c.t;
-                if (fast) load_payload(g + 2, c.t);
+                if (fast) load_payload(g + 2 * T, c.t);
             }
         }
         // ---- second half of chunk g, in registers
         if (kUseDct) dct64_inv(v);  // along b: v[k] = sum_b Z[b][lane] F[k][b]
         if (!stored) chunk_stats(v, g, skip_cur);
         const bool skip_next = more && __ballot(repeat == kClaimMark) != 0;  // wave-uniform, false for top-k payloads
-        if (skip_next) mark_redo(g + 1);
+        if (skip_next) mark_redo(g + T);
         repeat = 0;
         if (more) mean_pass();
 
         // (the loop-carried destination may have been parked in vector registers: make it scalar
         // again, or every store becomes a loop over distinct descriptors)
         gfloat* const dst = (gfloat*)uniform64(reinterpret_cast<int64_t>(out_cur.chunk0));
+        if constexpr (kTeam > 1) {
+            if (!stored) __builtin_amdgcn_s_barrier();  // (every wave of the team: one barrier per chunk, here or above)
+        }
         if (stored) {
             // (written above)
         } else if (kUseDct || out_cur.ld > 0) {
@@ -2016,6 +2027,9 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK>()), 2
         out_cur = out_next;
         out_next = out_after;
         t_next = t_after;
+    }
+    if constexpr (kTeam > 1) {
+        for (int64_t i = my_steps; i < team_steps; ++i) __builtin_amdgcn_s_barrier();
     }
     redo_marked();
 }
@@ -3548,9 +3562,10 @@ __global__ __launch_bounds__(64, 2) void k_calib_aggregate(const PeerPtrs pp, in
     }
 }
 
-// The same for the pipeline with the transform up to 16 peers, whose workgroups are teams of four waves: wave w
-// takes chunks w, w + 4, ... of the team's range, a group's index rows are four rows apart (lanes c k/2 .. take the
-// row of the group's chunk c; cached loads), and the team meets at a barrier before every chunk's stores.
+// The same for the launches whose workgroups are teams of four waves: wave w takes chunks w, w + 4, ... of the
+// team's range and the team meets at a barrier before every chunk's stores.  kGroup = 4 or 2 (with the transform):
+// a group's index rows are four rows apart (lanes c k/2 .. take the row of the group's chunk c; cached loads);
+// kGroup = 0 (without it): one two-byte index load per peer and chunk.
 template <int kGroup>
 __global__ __launch_bounds__(256, 2) void k_calib_aggregate_team(const PeerPtrs pp, int P, int k,
                                                                  const tplr_tensor_desc* __restrict__ table,
@@ -3562,18 +3577,22 @@ __global__ __launch_bounds__(256, 2) void k_calib_aggregate_team(const PeerPtrs 
     if (t0 >= t1) return;
     const int64_t idx_stride = k + (k >> 1), idx_end = total * idx_stride;
     const int le = lane < k ? lane : 0;
-    int lane_goff;
-    {
+    const uint32_t lane_ioff = 3u * (static_cast<uint32_t>(le) >> 1) + (le & 1);
+    int lane_goff = 0;
+    if constexpr (kGroup > 0) {
         const int half_k = k >> 1;
         int c = lane / half_k, q = lane - c * half_k;
         if (c >= kGroup) c = kGroup - 1, q = half_k - 1;
         lane_goff = c * T * static_cast<int>(idx_stride) + 3 * q;
     }
-    constexpr int kU = 16;
-    uint32_t ix[kU];
+    constexpr int kU = kGroup > 0 ? 16 : 24;
+    uint32_t ix[kU], ix2[2][kGroup > 0 ? 1 : kU];
     float a[2][kU];
 #pragma unroll
-    for (int i = 0; i < kU; ++i) ix[i] = 0, a[0][i] = 0.f, a[1][i] = 0.f;
+    for (int i = 0; i < kU; ++i) {
+        ix[i] = 0, a[0][i] = 0.f, a[1][i] = 0.f;
+        if constexpr (kGroup == 0) ix2[0][i] = ix2[1][i] = 0;
+    }
     const int64_t steps = (t1 - t0 + T - 1) / T;  // of the team; a wave past the end repeats its last chunk and stores nothing
     auto clampg = [&](int64_t g) { return g < t1 ? g : t1 - 1; };
     auto load_group = [&](int64_t g) {
@@ -3587,20 +3606,31 @@ __global__ __launch_bounds__(256, 2) void k_calib_aggregate_team(const PeerPtrs 
         constexpr int s = decltype(st)::value;
 #pragma unroll
         for (int i = 0; i < kU; ++i)
-            if (i < P) a[s][i] = __builtin_nontemporal_load((const gfloat*)pp.val[i] + clampg(g) * k + le);
+            if (i < P) {
+                if constexpr (kGroup > 0) {
+                    a[s][i] = __builtin_nontemporal_load((const gfloat*)pp.val[i] + clampg(g) * k + le);
+                } else {  // (as the kernel without the transform loads them: cached, two bytes of indices per chunk)
+                    ix2[s][i] = *(const gu16*)((const gbyte*)pp.idx[i] + clampg(g) * idx_stride + lane_ioff);
+                    a[s][i] = ((const gfloat*)pp.val[i] + clampg(g) * k)[le];
+                }
+            }
     };
     Cursor c;
     tplr_tensor_desc none = {};
     cursor_seek(c, table, none, n_tensors, clampg(t0 + w));
-    load_group(t0 + w);
+    if constexpr (kGroup > 0) load_group(t0 + w);
     load_vals(Index<0>{}, t0 + w);
     load_vals(Index<1>{}, t0 + w + T);
     auto body = [&](int64_t gb, auto st, bool with_group) {
         const int64_t g = gb + w;
         float x = 0.f;
 #pragma unroll
-        for (int i = 0; i < kU; ++i) x += a[decltype(st)::value][i] + __builtin_bit_cast(float, ix[i]);
-        if (with_group) load_group(g + 2 * T);
+        for (int i = 0; i < kU; ++i)
+            x += a[decltype(st)::value][i] +
+                 __builtin_bit_cast(float, kGroup > 0 ? ix[i] : ix2[decltype(st)::value][kGroup > 0 ? 0 : i]);
+        if constexpr (kGroup > 0) {
+            if (with_group) load_group(g + 2 * T);
+        }
         load_vals(st, g + 2 * T);
         float v[64];
 #pragma unroll
@@ -3612,7 +3642,7 @@ __global__ __launch_bounds__(256, 2) void k_calib_aggregate_team(const PeerPtrs 
             if (g + j < t1) cursor_next(c, g + j);
     };
     // (every wave of the team runs the same number of steps, and with them of barriers)
-    for (int64_t s = 0; s < steps; s += kGroup) {
+    for (int64_t s = 0; s < steps; s += (kGroup == 4 ? 4 : 2)) {
         const int64_t gb = t0 + s * T;
         body(gb, Index<0>{}, false);
         if (s + 1 < steps) body(gb + T, Index<1>{}, kGroup == 2);
@@ -4113,12 +4143,12 @@ static int launch_decode(const uint8_t* const* h_idx12, const float* const* h_va
             return use_dct ? launch_decode_as<aggregate_team<true, U>()>(k_decode_aggregate<true, U, BITS, false, true>, pp, d_scale, n_peers,\
                                               k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq,  \
                                               stream, si, sv)                                                        \
-                           : launch_decode_as(k_decode_aggregate<false, U, BITS, false, true>, pp, d_scale, n_peers,  \
+                           : launch_decode_as<4>(k_decode_aggregate<false, U, BITS, false, true>, pp, d_scale, n_peers,\
                                               k, d_desc, single, n_tensors, total, reduce_mode, normalise, d_sumsq,  \
                                               stream, si, sv);                                                       \
         return use_dct ? launch_decode_as<aggregate_team<true, U>()>(k_decode_aggregate<true, U, BITS>, pp, d_scale, n_peers, k, d_desc,\
                                           single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream)         \
-                       : launch_decode_as(k_decode_aggregate<false, U, BITS>, pp, d_scale, n_peers, k, d_desc,        \
+                       : launch_decode_as<4>(k_decode_aggregate<false, U, BITS>, pp, d_scale, n_peers, k, d_desc,     \
                                           single, n_tensors, total, reduce_mode, normalise, d_sumsq, stream);
     switch (units) {
         TPLR_DECODE_CASE(8, 4)
@@ -4744,11 +4774,13 @@ int tplr_calib_aggregate(const uint8_t* const* h_idx12, const float* const* h_va
     const int64_t need = ((total_chunks + 7) / 8) * 8;
     const dim3 grid(static_cast<unsigned>(need < resident ? need : resident));
     const hipStream_t on = static_cast<hipStream_t>(stream);
-    if (use_dct && n_peers <= 16) {
+    if (!use_dct || n_peers <= 16) {
         // (the launch it stands for runs teams of four waves)
         const int64_t teams = (((total_chunks + 3) / 4 + 7) / 8) * 8;
         const dim3 tgrid(static_cast<unsigned>(teams < resident / 4 ? teams : resident / 4));
-        if (k <= 32)
+        if (!use_dct)
+            hipLaunchKernelGGL(k_calib_aggregate_team<0>, tgrid, dim3(256), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
+        else if (k <= 32)
             hipLaunchKernelGGL(k_calib_aggregate_team<4>, tgrid, dim3(256), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
         else
             hipLaunchKernelGGL(k_calib_aggregate_team<2>, tgrid, dim3(256), 0, on, pp, n_peers, k, d_desc, n_tensors, total_chunks);
