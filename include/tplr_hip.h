@@ -495,6 +495,11 @@ int tplr_calib_copy(const void* d_src, void* d_dst, int64_t n_bytes, void* strea
  * The aggregate's chunk-pattern fill (tplr_calib_aggregate with no peers) is held against it. */
 int tplr_calib_fill(void* d_dst, int64_t n_bytes, int pattern, void* stream);
 
+/* Test aid, no counterpart in the reference: fills the LDS of every compute unit with `word` (one resident round of
+ * workgroups that write 80 000 bytes each).  LDS keeps its contents from kernel to kernel; the tests run the
+ * aggregate kernels after it to show that nothing they read before writing it decides anything. */
+int tplr_debug_fill_lds(int word, void* stream);
+
 /* Measurement aid, no counterpart in the reference: the memory side of tplr_encode_topk_pack_batch alone.  Same
  * grid, same chunk ranges and the same 64 streaming row loads per chunk from the tensors of d_desc, without the
  * transform, the select and the payload stores.  Its duration is the time the memory system needs to hand the

@@ -56,6 +56,7 @@ SIGNATURES = {
     "tplr_calib_encode": (_i32, [_vp, _i32, _i64, _vp]),
     "tplr_calib_copy": (_i32, [_vp, _vp, _i64, _vp]),
     "tplr_calib_fill": (_i32, [_vp, _i64, _i32, _vp]),
+    "tplr_debug_fill_lds": (_i32, [_i32, _vp]),
     "tplr_calib_aggregate": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _i32, _i64, _vp]),
     "tplr_ef_encode_topk_pack_batch": (_i32, [_vp, _vp, _i32, _i64, C.c_float, _i32, _i32, _vp, _vp, _vp]),
     "tplr_ef_subtract_batch": (_i32, [_vp, _vp, _i32, _vp, _i32, _i64, _i32, _vp]),

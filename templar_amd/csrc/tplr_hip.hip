@@ -3653,6 +3653,22 @@ __global__ __launch_bounds__(256, 2) void k_calib_aggregate_team(const PeerPtrs 
     }
 }
 
+// Test aid: every compute unit's LDS filled with one word.  Two workgroups of 80 000 bytes fit a compute unit, and a
+// grid of two per compute unit is one resident round, so the launch reaches (nearly) every LDS byte of the device.
+// (`sink` may be null.)
+__global__ __launch_bounds__(256, 2) void k_fill_lds(uint32_t word, uint32_t* __restrict__ sink) {
+    __shared__ uint32_t all[20000];
+    volatile uint32_t* const out = all;  // (LDS is dead when the kernel ends, as far as the optimiser knows)
+    for (int i = threadIdx.x; i < 20000; i += 256) out[i] = word;
+    // (stay for a fixed while, about 0.1 ms: the dispatcher then has to place every workgroup of the round on a slot
+    // of its own instead of handing the slots of the first ones on)
+    for (int i = 0; i < 32; ++i) __builtin_amdgcn_s_sleep(127);
+    __syncthreads();
+    uint32_t s = 0;
+    for (int i = 255 - threadIdx.x; i < 20000; i += 256) s += out[i];
+    if (sink && s == 0x12345678u) sink[0] = s;
+}
+
 }  // namespace tplr
 
 // =========================================================================================
@@ -4814,6 +4830,16 @@ int tplr_calib_copy(const void* d_src, void* d_dst, int64_t n_bytes, void* strea
     if (n_bytes == 0) return 0;
     hipLaunchKernelGGL(k_calib_copy, dim3(256 * 16), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const v4f*>(d_src), static_cast<v4f*>(d_dst), n_bytes >> 4);
+    return launch_status();
+}
+
+int tplr_debug_fill_lds(int word, void* stream) {
+    int n_cu = 256, dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+        n_cu = v;
+    hipLaunchKernelGGL(k_fill_lds, dim3(static_cast<unsigned>(2 * n_cu)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint32_t>(word), static_cast<uint32_t*>(nullptr));
     return launch_status();
 }
 

@@ -98,3 +98,44 @@ def test_miner_step_twice(dev):
         snaps.append((idx12.clone(), val.clone(), [e.clone() for e in efs]))
     assert torch.equal(snaps[0][0], snaps[1][0]) and torch.equal(snaps[0][1].view(torch.int32), snaps[1][1].view(torch.int32))
     assert all(torch.equal(a.view(torch.int32), b.view(torch.int32)) for a, b in zip(snaps[0][2], snaps[1][2]))
+
+
+@pytest.mark.parametrize("P,k,use_dct", [(15, 32, True), (7, 16, True), (20, 32, True), (15, 32, False), (40, 32, True)])
+def test_aggregate_does_not_depend_on_what_lds_held(dev, P, k, use_dct):
+    """LDS keeps what the last kernel on a compute unit left.  The aggregate's fast scatter marks a slot it has
+    claimed with an all-ones word, and lanes without an entry scatter to slots that are not cleared with the tile:
+    if such a slot held all ones from an earlier kernel, every chunk was taken for one with a repeated index and done
+    again on the exact path - the same result ten times slower.  Here every LDS word of the device is set to all
+    ones (then to a NaN, then to zero) before the launch: results must be the same bits, and the launches after the
+    all-ones fill must not take longer than after the zero fill."""
+    from templar_amd import _lib
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    # (several chunks per wave: a wave's first chunk is scattered serially and never touches those slots)
+    shapes = [(4096, 4096), (2048, 4096), (64, 64)]
+    grads = [workloads.student_t3(s, 700 + i, row_scale=True, device=dev) for i, s in enumerate(shapes)]
+    idxs, vals = _payloads(dev, grads, k, P, use_dct)
+    outs = [torch.empty_like(g) for g in grads]
+    ob = tc.TensorBatch(outs)
+    scale = tc.peer_clip_scales_batch(ob, vals, k)
+    run = lambda: tc.batch_decompress_decode_batch(ob, idxs, vals, k, scale=scale, use_dct=use_dct)
+    snaps, times = [], {}
+    for word in (0, -1, 0x7FC00000, 0):
+        _lib.check(lib.tplr_debug_fill_lds(word, stream), "tplr_debug_fill_lds")
+        for o in outs:
+            o.fill_(float("nan"))
+        run()
+        torch.cuda.synchronize()
+        snaps.append([o.clone() for o in outs])
+        _lib.check(lib.tplr_debug_fill_lds(word, stream), "tplr_debug_fill_lds")
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(10):
+            run()
+        b.record()
+        torch.cuda.synchronize()
+        times[word] = a.elapsed_time(b)
+    for s in snaps[1:]:
+        for x, y in zip(snaps[0], s):
+            assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "the result depends on what LDS held"
+    assert times[-1] < 2.0 * times[0] + 0.5, f"launches after an all-ones LDS take {times[-1]:.2f} ms against {times[0]:.2f} ms"
