@@ -139,3 +139,28 @@ def test_aggregate_does_not_depend_on_what_lds_held(dev, P, k, use_dct):
         for x, y in zip(snaps[0], s):
             assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "the result depends on what LDS held"
     assert times[-1] < 2.0 * times[0] + 0.5, f"launches after an all-ones LDS take {times[-1]:.2f} ms against {times[0]:.2f} ms"
+
+
+@pytest.mark.parametrize("k,use_dct", [(32, True), (64, True), (64, False), (8, False)])
+def test_encode_and_miner_step_do_not_depend_on_what_lds_held(dev, k, use_dct):
+    """The same for the send side: the staging buffer and the candidate slots of the select, and the miner step's
+    tile, are written before they are read whatever LDS held."""
+    from templar_amd import _lib
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    shapes = [(4096, 2048), (1024, 512), (64, 64)]
+    grads = [workloads.student_t3(s, 800 + i, row_scale=True, device=dev) for i, s in enumerate(shapes)]
+    batch = tc.TensorBatch(grads)
+    snaps = []
+    for word in (0, -1, 0x7FC00000):
+        _lib.check(lib.tplr_debug_fill_lds(word, stream), "tplr_debug_fill_lds")
+        idx, val = tc.encode_compress_batch(batch, k, use_dct=use_dct)
+        efs = [torch.full_like(g, 0.25) for g in grads]
+        _lib.check(lib.tplr_debug_fill_lds(word, stream), "tplr_debug_fill_lds")
+        i2, v2, _ = tc.error_feedback_step_batch(tc.TensorBatch(efs), batch, 0.9, k, use_dct=use_dct)
+        torch.cuda.synchronize()
+        snaps.append([idx.clone(), val.view(torch.int32).clone(), i2.clone(), v2.view(torch.int32).clone()] +
+                     [e.view(torch.int32).clone() for e in efs])
+    for s in snaps[1:]:
+        for x, y in zip(snaps[0], s):
+            assert torch.equal(x, y), "the result depends on what LDS held"
