@@ -3683,9 +3683,9 @@ static inline int launch_status() {
 
 static inline unsigned grid8(int64_t n) { return static_cast<unsigned>(((n + 7) / 8) * 8); }
 
-// persistent grids: exactly one resident set of single-wave workgroups, as the occupancy
-// calculator reports it for the kernel at hand (registers or LDS bound it); a larger grid
-// would leave a second, mostly empty round
+// persistent grids: exactly one resident set of workgroups of `threads` threads (one wave, or a team of
+// waves), as the occupancy calculator reports it for the kernel at hand (registers or LDS bound it); a
+// larger grid would leave a second, mostly empty round
 template <typename Kernel>
 static int persistent_grid(Kernel kernel, int64_t total, int threads = 64) {
     int n_cu = 256, per_cu = 0, dev = 0, v = 0;
