@@ -2042,11 +2042,12 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK, !kCod
 // the k selected values go back into a cleared tile exactly as the one-peer decode adds them (0 + value * 2^-5),
 // through the inverse transform, and the difference is stored.  Two waves per SIMD (a whole tile, 64 more
 // registers): the launch moves 14 GB and is bound by that.
-// Workgroups are teams of four waves, as in the aggregate: wave w takes every fourth chunk of the team's range, the
-// team reads rows of 1 KB at the same moment and meets at a barrier before it stores them (6 % off the launch).
-// (k <= 32 only: at k = 64 the team form is 2 % slower than single waves)
+// Workgroups are teams of four (two) waves, as in the aggregate: wave w takes every fourth chunk of the team's range,
+// the team reads rows of 1 KB at the same moment and meets at a barrier before it stores them (6 % off the launch).
+// (at k = 64 the select's instantiation is at the register limit: teams of four are 2 % slower than single
+// waves there, teams of two 4.5 % faster)
 template <bool kTwo>
-constexpr int ef_team() { return kTwo ? 1 : 4; }
+constexpr int ef_team() { return kTwo ? 2 : 4; }
 template <bool kTwo>
 __global__ __launch_bounds__(64 * ef_team<kTwo>(), 2) void k_ef_step(const tplr_tensor_desc* __restrict__ table,
                                                    const tplr_tensor_desc* __restrict__ grad_table, int n_tensors,
