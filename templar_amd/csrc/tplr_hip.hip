@@ -575,17 +575,19 @@ __device__ __forceinline__ void set_wave_priority(int level) {
 // Without the transform the kernel waits more than it computes, and workgroups of two waves that take alternate
 // chunks and meet at a barrier before they request their rows (512 contiguous bytes per row at the same moment) are
 // 6 % faster; with the transform, where the vector ALU is the bound, any team is slower (8 % with four waves).
-template <bool kUseDct>
-constexpr int encode_team() { return kUseDct ? 1 : 2; }
+// kEf also writes every chunk back, and rows written together are served sooner: teams of four without the
+// transform (8 % off the two-launch miner step against single waves), of two with it (4 %).
+template <bool kUseDct, bool kEf = false>
+constexpr int encode_team() { return kUseDct ? (kEf ? 2 : 1) : (kEf ? 4 : 2); }
 
 template <bool kTwo, bool kUseDct, bool kEf = false>
-__global__ __launch_bounds__(64 * encode_team<kUseDct>(), 3) void k_encode_topk_pack(const tplr_tensor_desc* __restrict__ table,
+__global__ __launch_bounds__((64 * encode_team<kUseDct, kEf>()), 3) void k_encode_topk_pack(const tplr_tensor_desc* __restrict__ table,
                                                             const tplr_tensor_desc single, int n_tensors,
                                                             int64_t total, int k, uint8_t* __restrict__ idx12,
                                                             float* __restrict__ val,
                                                             const tplr_tensor_desc* __restrict__ grad_table,
                                                             float decay) {
-    constexpr int T = encode_team<kUseDct>();
+    constexpr int T = encode_team<kUseDct, kEf>();
     __shared__ __align__(16) float buf_all[T][kHalfFloats];
     __shared__ uint64_t cand_all[T][kCandCap];
     const int wv = T > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)) : 0;  // wave of the team
@@ -3913,15 +3915,15 @@ int tplr_ef_encode_topk_pack_batch(const tplr_tensor_desc* d_ef_desc, const tplr
     tplr_tensor_desc none = {};
     if (k > 32) {
         if (use_dct)
-            return launch_encode_as(k_encode_topk_pack<true, true, true>, d_ef_desc, none, n_tensors, total_chunks, k,
+            return launch_encode_as<encode_team<true, true>()>(k_encode_topk_pack<true, true, true>, d_ef_desc, none, n_tensors, total_chunks, k,
                                     d_idx12, d_val, stream, d_grad_desc, decay);
-        return launch_encode_as<encode_team<false>()>(k_encode_topk_pack<true, false, true>, d_ef_desc, none, n_tensors, total_chunks, k,
+        return launch_encode_as<encode_team<false, true>()>(k_encode_topk_pack<true, false, true>, d_ef_desc, none, n_tensors, total_chunks, k,
                                 d_idx12, d_val, stream, d_grad_desc, decay);
     }
     if (use_dct)
-        return launch_encode_as(k_encode_topk_pack<false, true, true>, d_ef_desc, none, n_tensors, total_chunks, k,
+        return launch_encode_as<encode_team<true, true>()>(k_encode_topk_pack<false, true, true>, d_ef_desc, none, n_tensors, total_chunks, k,
                                 d_idx12, d_val, stream, d_grad_desc, decay);
-    return launch_encode_as<encode_team<false>()>(k_encode_topk_pack<false, false, true>, d_ef_desc, none, n_tensors, total_chunks, k,
+    return launch_encode_as<encode_team<false, true>()>(k_encode_topk_pack<false, false, true>, d_ef_desc, none, n_tensors, total_chunks, k,
                             d_idx12, d_val, stream, d_grad_desc, decay);
 }
 
