@@ -1650,10 +1650,11 @@ __global__ __launch_bounds__((64 * aggregate_team<kUseDct, kUnits, kWideK, !kCod
                     (void*)uniform64(reinterpret_cast<int64_t>(o0.chunk0)), 0,
                     (skip0 || tripped) ? 0 : static_cast<int>((63 * ld0 + 64) * 4), 0x00020000);
                 const int ld4 = static_cast<int>(ld0) * 4;
-                static_for<8>([&](auto qt) {
+                // (sixteen groups of four: 1.2 % faster than eight of eight in teams; thirty-two of two 13 % slower)
+                static_for<16>([&](auto qt) {
                     constexpr int q = decltype(qt)::value;
 #pragma unroll
-                    for (int r = q * 8; r < (q + 1) * 8; ++r)
+                    for (int r = q * 4; r < (q + 1) * 4; ++r)
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v[r]), wr, lane * 4, r * ld4, 2);
                     mean_trip(ms);
                 });
